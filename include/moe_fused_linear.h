@@ -1,0 +1,161 @@
+/*
+ * moe_fused_linear.h -- C ABI of the MI355X (gfx950) moe_fused_linear library.
+ *
+ * The reference implements this path as in-process Python calls of Triton-JIT
+ * kernels; it has no FFI of its own.  Each entry point below replaces one such
+ * Python-level kernel wrapper and cites it (paths relative to the reference).
+ *
+ * Conventions shared by all entry points
+ *   - all pointers are DEVICE pointers unless stated otherwise; tensors are dense,
+ *     row-major, contiguous;
+ *   - `stream` is a hipStream_t passed as void*; every call only enqueues work on
+ *     it: no synchronisation, no allocation, no host read of device data;
+ *   - return value: 0 = OK, negative = argument error (MFL_ERR_*), positive =
+ *     hipError_t of a failed launch;
+ *   - the library keeps no mutable global state (device properties are cached
+ *     read-only); calls are re-entrant.
+ */
+#ifndef MOE_FUSED_LINEAR_H
+#define MOE_FUSED_LINEAR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MFL_ABI_VERSION 1
+
+/* element types */
+#define MFL_BF16 0
+#define MFL_F32 1
+#define MFL_F16 2
+/* index types */
+#define MFL_I32 0
+#define MFL_I64 1
+
+/* argument errors */
+#define MFL_OK 0
+#define MFL_ERR_NULL (-1)        /* required pointer is NULL                        */
+#define MFL_ERR_SHAPE (-2)       /* negative / zero / inconsistent dimension        */
+#define MFL_ERR_DTYPE (-3)       /* unknown or unsupported element / index type     */
+#define MFL_ERR_ALIGN (-4)       /* pointer not aligned to its element size         */
+#define MFL_ERR_WORKSPACE (-5)   /* workspace missing or too small                  */
+#define MFL_ERR_UNSUPPORTED (-6) /* valid request this build has no kernel for      */
+
+int mfl_abi_version(void);
+/* Static, NUL-terminated description of a return code of this library. */
+const char *mfl_strerror(int code);
+
+/* ---- grouped GEMM ---------------------------------------------------------------
+ * Rows of x are grouped by expert, ascending; m_sizes[e] rows belong to expert e and
+ * sum(m_sizes) <= R.  Rows past sum(m_sizes) are not written.  m_sizes is read on the
+ * device (no host sync).  fp32 accumulation; out = alpha * acc (+ out if accumulate).
+ * in_dtype is the type of both x and w; out_dtype the type of the result. */
+
+/* y[m, n] = sum_k w[e(m), n, k] * x[m, k];  x (R,K), w (E,N,K), y (R,N).
+ * Replaces grouped_gemm_forward, qwen3_moe_fused/grouped_gemm/forward.py:116-160. */
+int mfl_gemm_fwd(const void *x, const void *w, const void *m_sizes, int m_sizes_dtype, void *y,
+                 int64_t R, int N, int K, int E, int in_dtype, int out_dtype, float alpha,
+                 int accumulate, void *stream);
+
+/* dx[m, n] = sum_k w[e(m), k, n] * dy[m, k];  dy (R,K), w (E,K,N), dx (R,N).
+ * Replaces grouped_gemm_forward_transposed,
+ * qwen3_moe_fused/grouped_gemm/forward_transposed.py:107-151. */
+int mfl_gemm_dx(const void *dy, const void *w, const void *m_sizes, int m_sizes_dtype, void *dx,
+                int64_t R, int N, int K, int E, int in_dtype, int out_dtype, float alpha,
+                int accumulate, void *stream);
+
+/* dw[e, n, k] = sum_{m in e} dy[m, n] * x[m, k];  x (R,K), dy (R,N), dw (E,N,K).
+ * Every element of dw is written; experts without rows get exact zeros.
+ * Replaces grouped_gemm_backward_dw, qwen3_moe_fused/grouped_gemm/backward_dw.py:92-134. */
+int mfl_gemm_dw(const void *x, const void *dy, const void *m_sizes, int m_sizes_dtype, void *dw,
+                int64_t R, int N, int K, int E, int in_dtype, int out_dtype, float alpha,
+                int accumulate, void *stream);
+
+/* Forward GEMM with NF4 weights decoded inside the K loop:
+ * w[e, n, k] = code16[nibble] * absmax[(e*N*K + n*K + k) / blocksize], rounded once to
+ * in_dtype; byte i of wq holds element 2i in its high nibble, 2i+1 in its low nibble.
+ * code16 (16 floats) and absmax (E*N*K/blocksize floats) are device pointers.
+ * Replaces grouped_gemm_forward_4bit, qwen3_moe_fused/grouped_gemm/forward_4bit.py:135-208. */
+int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, const float *absmax,
+                     int blocksize, const void *m_sizes, int m_sizes_dtype, void *y, int64_t R,
+                     int N, int K, int E, int in_dtype, int out_dtype, void *stream);
+
+/* ---- NF4 / blockwise dequantisation ----------------------------------------------- */
+
+/* out[i] = code16[nibble(i)] * absmax[i / blocksize], i < n (n even).  Stands in for the
+ * bitsandbytes dequantize_4bit calls at qwen3_moe_fused/quantize/layer.py:21 and
+ * qwen3_moe_fused/kernels/fast_lora.py:62. */
+int mfl_nf4_dequant(const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                    void *out, int64_t n, int out_dtype, void *stream);
+
+/* out[i] = code256[v[i]] * absmax2[i / blocksize2] + offset  (nested absmax),
+ * qwen3_moe_fused/grouped_gemm/forward_4bit.py:149-152. */
+int mfl_dequant_blockwise_u8(const uint8_t *v, const float *code256, const float *absmax2,
+                             int blocksize2, float offset, float *out, int64_t n, void *stream);
+
+/* Blockwise NF4 quantiser: absmax[b] = max|block b|, nibble = nearest code16 entry to
+ * x / absmax (ties -> lower entry).  w has n elements of w_dtype, n % blocksize == 0.
+ * Stands in for bitsandbytes quantize_4bit as used at test_moe_fused_linear.py:40. */
+int mfl_nf4_quant(const void *w, int w_dtype, int64_t n, int blocksize, const float *code16,
+                  uint8_t *wq, float *absmax, void *stream);
+
+/* ---- routing ---------------------------------------------------------------------- */
+
+/* p = softmax_fp32(logits[t, :]); top-k of p, descending, equal values -> lower expert id
+ * first; if renorm, weights /= sum(weights).  weights_f32 (T,k) and/or weights_cast (T,k) of
+ * cast_dtype may be NULL; idx (T,k) int64 is required.
+ * Replaces qwen3_moe_fused/modular_qwen3_moe_fused.py:87-93 (= fast_lora.py:52-58). */
+int mfl_route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int E, int k,
+                           int renorm, float *weights_f32, void *weights_cast, int cast_dtype,
+                           int64_t *idx, void *stream);
+
+/* Stable counting sort of expert ids sel (R,) in [0, E):
+ *   counts[e]        = #{j : sel[j] == e}
+ *   sort_idx[i]      = j of the i-th row in the stable ascending order
+ *   inv_sort_idx[j]  = position of row j in that order
+ * sort_idx and inv_sort_idx may both be NULL (counts only).  Ids outside [0, E) are a
+ * caller error (they are ignored by the counts and leave their slots unwritten).
+ * workspace: mfl_expert_sort_workspace(R, E) bytes of device memory, contents ignored.
+ * Replaces get_expert_counts_and_idx / get_expert_counts,
+ * qwen3_moe_fused/kernels/indexing.py:18-23,48-65. */
+size_t mfl_expert_sort_workspace(int64_t R, int E);
+int mfl_expert_sort(const void *sel, int sel_dtype, int64_t R, int E, int32_t *counts,
+                    int32_t *sort_idx, int32_t *inv_sort_idx, void *workspace, size_t ws_bytes,
+                    void *stream);
+
+/* dst[j, :] = src[idx[j] / idx_div, :] * (row_scale ? row_scale[idx[j]] : 1), j < R_out.
+ * With idx = sort_idx and idx_div = k this is "replicate each token k times, then gather",
+ * qwen3_moe_fused/modular_qwen3_moe_fused.py:95-103.  row_scale has `dtype` elements. */
+int mfl_gather_rows(const void *src, const int32_t *idx, int idx_div, const void *row_scale,
+                    void *dst, int64_t R_out, int H, int dtype, void *stream);
+
+/* dst[t, :] = sum_{j<k} src[pos[t*k+j], :] * (weights ? weights[t*k+j] : 1), fp32 accumulate.
+ * With pos = inv_sort_idx this is "un-sort, then weighted sum over the k selections",
+ * qwen3_moe_fused/modular_qwen3_moe_fused.py:112-115. */
+int mfl_combine_rows(const void *src, const int32_t *pos, const void *weights, void *dst,
+                     int64_t T, int k, int H, int dtype, void *stream);
+
+/* dots[t*k+j] = <a[t, :], b[pos[t*k+j], :]>  (gradient of mfl_combine_rows w.r.t. weights). */
+int mfl_rows_dot(const void *a, const void *b, const int32_t *pos, void *dots, int64_t T, int k,
+                 int H, int dtype, void *stream);
+
+/* ---- SiLU-mul --------------------------------------------------------------------- */
+
+/* h = T(f32(e) * sigmoid(f32(e))) * g.  Replaces silu_mul_forward,
+ * qwen3_moe_fused/kernels/silu_mul.py:114-125. */
+int mfl_silu_mul_fwd(const void *e, const void *g, void *h, int64_t n, int dtype, void *stream);
+
+/* de, dg (and h when h_out != NULL) from dh, e, g.  Outputs may alias inputs element for
+ * element (dh->h_out, e->de, g->dg gives the reference's in-place variant).  Replaces
+ * silu_mul_backward and silu_mul_backward_inplace,
+ * qwen3_moe_fused/kernels/silu_mul.py:128-159. */
+int mfl_silu_mul_bwd(const void *dh, const void *e, const void *g, void *de, void *dg, void *h_out,
+                     int64_t n, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_FUSED_LINEAR_H */

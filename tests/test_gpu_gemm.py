@@ -1,0 +1,189 @@
+"""GPU parity of the grouped GEMM (fwd / dX / dW) against the CPU oracle, through the C ABI
+(the Python wrappers are thin ctypes calls).  Shapes follow the reference's own scripts
+(test_moe_fused_linear.py:19-23: 1024 x 2048 -> 768, 128 experts; the tiny model's odd sizes
+3 / 16 / 11 experts from test_model.py:29-40) plus BASELINE configs 1-3."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import check_close, gen, m_sizes_uniform, randn, to_np32, topk_routing
+
+pytestmark = pytest.mark.gpu
+
+from qwen3_moe_fused.functional import moe_fused_linear  # noqa: E402
+from qwen3_moe_fused.grouped_gemm.backward_dw import grouped_gemm_backward_dw  # noqa: E402
+from qwen3_moe_fused.grouped_gemm.forward import grouped_gemm_forward  # noqa: E402
+from qwen3_moe_fused.grouped_gemm.forward_transposed import grouped_gemm_forward_transposed  # noqa: E402
+
+DEV = "cuda"
+
+
+def _case(seed, R, N, K, E, dtype, m_sizes=None):
+    g = gen(seed)
+    x = randn((R, K), g, 1.0, dtype)
+    w = randn((E, N, K), g, 0.02 if dtype != torch.float32 else 0.1, dtype)
+    dy = randn((R, N), g, 1.0, dtype)
+    ms = m_sizes_uniform(R, E, g) if m_sizes is None else m_sizes
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    return x, w, dy, ms, sel
+
+
+def _tol(dtype):
+    return (1e-2, 1e-2) if dtype != torch.float32 else (1e-4, 1e-5)
+
+
+SHAPES = [
+    # R, N, K, E
+    (512, 128, 64, 8),       # BASELINE config 1 sizes
+    (1024, 768, 2048, 128),  # the reference's test shape
+    (91, 3, 16, 11),         # tiny model: gate/up (moe_intermediate 3, hidden 16, 11 experts)
+    (91, 16, 3, 11),         # tiny model: down
+    (300, 40, 72, 5),        # multiples of 8 only
+    (257, 136, 264, 3),      # one row past a tile edge
+    (64, 16, 2048, 128),     # LoRA A shape, most experts empty
+    (64, 768, 16, 128),      # LoRA B shape
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("R,N,K,E", SHAPES)
+def test_forward_dx_dw_match_oracle(R, N, K, E, dtype):
+    x, w, dy, ms, sel = _case(1234 + R + N, R, N, K, E, dtype)
+    rtol, atol = _tol(dtype)
+    xd, wd, dyd, msd = x.to(DEV), w.to(DEV), dy.to(DEV), ms.to(DEV)
+
+    y = grouped_gemm_forward(xd, wd, msd)
+    assert y.dtype == dtype and y.shape == (R, N)
+    check_close(y, oracle.linear_fwd(to_np32(x), to_np32(w), sel), rtol, atol, "fwd")
+
+    dx = grouped_gemm_forward_transposed(dyd, wd, msd)
+    check_close(dx, oracle.linear_bwd_input(to_np32(dy), to_np32(w), sel), rtol, atol, "dx")
+
+    dw = grouped_gemm_backward_dw(xd, dyd, msd, dtype)
+    exp_dw = oracle.linear_bwd_weight(to_np32(dy), to_np32(x), sel, E)
+    # dW sums up to R/E products of N(0,1) values: scale the absolute tolerance with its size
+    check_close(dw, exp_dw, rtol, atol * max(1.0, np.abs(exp_dw).max()), "dw")
+    empty = (ms == 0).nonzero().flatten().tolist()
+    for e in empty:
+        assert torch.count_nonzero(dw[e]).item() == 0, "experts without rows must get exact zeros"
+
+
+def test_autograd_matches_oracle_bf16():
+    """moe_fused_linear(...).backward, the reference's test_moe_fused_linear_bwd.py:67-78."""
+    R, N, K, E = 1024, 768, 2048, 128
+    x, w, dy, ms, sel = _case(7, R, N, K, E, torch.bfloat16)
+    xd = x.to(DEV).requires_grad_()
+    wd = w.to(DEV).requires_grad_()
+    out = moe_fused_linear(xd, wd, ms.to(DEV))
+    out.backward(dy.to(DEV))
+    check_close(out, oracle.linear_fwd(to_np32(x), to_np32(w), sel), what="fwd")
+    check_close(xd.grad, oracle.linear_bwd_input(to_np32(dy), to_np32(w), sel), what="dx")
+    exp_dw = oracle.linear_bwd_weight(to_np32(dy), to_np32(x), sel, E)
+    check_close(wd.grad, exp_dw, 1e-2, 1e-2 * max(1.0, np.abs(exp_dw).max()), "dw")
+    # grads are gated on requires_grad (interface.py:18-26)
+    x2 = x.to(DEV).requires_grad_()
+    moe_fused_linear(x2, w.to(DEV), ms.to(DEV)).backward(dy.to(DEV))
+    assert x2.grad is not None
+
+
+@pytest.mark.parametrize("ms_dtype", [torch.int32, torch.int64, torch.int16])
+def test_m_sizes_integer_types(ms_dtype):
+    x, w, dy, ms, sel = _case(11, 256, 64, 64, 4, torch.bfloat16)
+    y = grouped_gemm_forward(x.to(DEV), w.to(DEV), ms.to(ms_dtype).to(DEV))
+    check_close(y, oracle.linear_fwd(to_np32(x), to_np32(w), sel), what="fwd")
+
+
+def test_edge_cases_empty_and_single_expert():
+    # no rows at all
+    w = randn((4, 32, 64), gen(0), 0.02, torch.bfloat16).to(DEV)
+    ms0 = torch.zeros(4, dtype=torch.int32, device=DEV)
+    y = grouped_gemm_forward(torch.empty((0, 64), dtype=torch.bfloat16, device=DEV), w, ms0)
+    assert y.shape == (0, 32)
+    dw = grouped_gemm_backward_dw(torch.empty((0, 64), dtype=torch.bfloat16, device=DEV),
+                                  torch.empty((0, 32), dtype=torch.bfloat16, device=DEV), ms0, torch.bfloat16)
+    assert dw.shape == (4, 32, 64) and torch.count_nonzero(dw).item() == 0
+    # E = 1 is an ordinary linear layer
+    x, w1, dy, ms, sel = _case(3, 200, 48, 96, 1, torch.bfloat16, m_sizes=torch.tensor([200], dtype=torch.int32))
+    y = grouped_gemm_forward(x.to(DEV), w1.to(DEV), ms.to(DEV))
+    ref = torch.nn.functional.linear(x.float(), w1[0].float())
+    check_close(y, ref.numpy(), what="E=1 vs F.linear")
+    # all rows on the last expert, the rest empty
+    ms_last = torch.tensor([0, 0, 0, 130], dtype=torch.int32)
+    x, w4, dy, _, _ = _case(4, 130, 32, 64, 4, torch.bfloat16, m_sizes=ms_last)
+    sel = oracle.sel_from_m_sizes(ms_last.numpy())
+    y = grouped_gemm_forward(x.to(DEV), w4.to(DEV), ms_last.to(DEV))
+    check_close(y, oracle.linear_fwd(to_np32(x), to_np32(w4), sel), what="last expert only")
+
+
+def test_alpha_and_accumulate():
+    x, w, dy, ms, sel = _case(5, 300, 64, 128, 6, torch.bfloat16)
+    base = randn((300, 64), gen(6), 1.0, torch.bfloat16)
+    out = base.clone().to(DEV)
+    grouped_gemm_forward(x.to(DEV), w.to(DEV), ms.to(DEV), out=out, alpha=0.5, accumulate=True)
+    ref = to_np32(base) + 0.5 * oracle.linear_fwd(to_np32(x), to_np32(w), sel)
+    check_close(out, ref, what="y += alpha * x w^T")
+
+
+def test_wrapper_asserts_like_the_reference():
+    w = torch.zeros((2, 8, 8), dtype=torch.bfloat16, device=DEV)
+    ms = torch.tensor([1, 1], dtype=torch.int32, device=DEV)
+    with pytest.raises(AssertionError):
+        grouped_gemm_forward(torch.zeros((2, 8), dtype=torch.bfloat16), w, ms)           # CPU input
+    with pytest.raises(AssertionError):
+        grouped_gemm_forward(torch.zeros((2, 16), dtype=torch.bfloat16, device=DEV), w, ms)  # K mismatch
+    with pytest.raises(AssertionError):
+        grouped_gemm_forward(torch.zeros((2, 8), dtype=torch.bfloat16, device=DEV), w, ms.float())
+
+
+# ---- BASELINE configs 2 and 3 at full size: oracle on a sample + size-independent properties
+
+def _config23(seed):
+    g = gen(seed)
+    E, H, I, T, k = 128, 2048, 768, 4096, 8
+    sel, ms = topk_routing(T, E, k, g)
+    return g, E, H, I, T * k, ms
+
+
+def test_config2_gate_proj_forward_full_size():
+    g, E, H, I, R, ms = _config23(2)
+    x = randn((R, H), g, 1.0, torch.bfloat16)
+    w = randn((E, I, H), g, 0.02, torch.bfloat16)
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    xd, wd, msd = x.to(DEV), w.to(DEV), ms.to(DEV)
+    y = grouped_gemm_forward(xd, wd, msd)
+    rows = np.sort(np.random.default_rng(0).choice(R, 1024, replace=False))
+    # include the first and last row of some experts (tile edges)
+    ends = np.cumsum(ms.numpy())
+    rows = np.unique(np.concatenate([rows, ends[:16] - 1, ends[:16] % R]))
+    exp = oracle.linear_fwd(to_np32(x[rows]), to_np32(w), sel[rows])
+    check_close(y[rows], exp, what="config 2 sampled rows")
+    # linearity in x: f(2x) == 2 f(x) exactly in bf16 (power-of-two scaling)
+    y2 = grouped_gemm_forward(xd * 2, wd, msd)
+    assert torch.equal(y2, y * 2)
+    # run-to-run determinism
+    assert torch.equal(grouped_gemm_forward(xd, wd, msd), y)
+
+
+def test_config3_down_proj_backward_full_size():
+    g, E, H, I, R, ms = _config23(3)
+    x = randn((R, I), g, 1.0, torch.bfloat16)
+    dy = randn((R, H), g, 1.0, torch.bfloat16)
+    w = randn((E, H, I), g, 0.02, torch.bfloat16)
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    xd, dyd, wd, msd = x.to(DEV), dy.to(DEV), w.to(DEV), ms.to(DEV)
+    dx = grouped_gemm_forward_transposed(dyd, wd, msd)
+    rows = np.sort(np.random.default_rng(1).choice(R, 1024, replace=False))
+    check_close(dx[rows], oracle.linear_bwd_input(to_np32(dy[rows]), to_np32(w), sel[rows]), what="config 3 dX")
+    dw = grouped_gemm_backward_dw(xd, dyd, msd, torch.bfloat16)
+    # per-expert dW depends only on that expert's rows: oracle on a few experts
+    starts = np.concatenate([[0], np.cumsum(ms.numpy())])
+    for e in (0, 63, 127):
+        sl = slice(starts[e], starts[e + 1])
+        exp = oracle.linear_bwd_weight(to_np32(dy[sl]), to_np32(x[sl]), np.zeros(sl.stop - sl.start, np.int64), 1)[0]
+        check_close(dw[e], exp, 1e-2, 1e-2 * np.abs(exp).max(), f"config 3 dW expert {e}")
+    # checksum identity: sum_e dW[e] == dy^T x  (fp32 accumulation of bf16-rounded tiles)
+    total = dw.float().sum(dim=0)
+    ref = dyd.float().t() @ xd.float()
+    check_close(total, to_np32(ref), 2e-2, 2e-2 * float(ref.abs().max()), "sum_e dW == dy^T x")
+    assert torch.equal(grouped_gemm_backward_dw(xd, dyd, msd, torch.bfloat16), dw)

@@ -1,0 +1,263 @@
+"""Module-level parity: the sparse MoE block, the fused-format LoRA layer, the fast-LoRA
+autograd function and the 4-bit layer, against the oracle's compositions and against torch
+autograd of the reference's formulas."""
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import check_close, gen, randn, to_np32, topk_routing, zipf_bias
+
+pytestmark = pytest.mark.gpu
+
+from qwen3_moe_fused.fast_lora import (fast_Qwen3MoeFusedSparseMoeBlock_forward, get_lora_parameters)  # noqa: E402
+from qwen3_moe_fused.kernels.fast_lora import fast_lora  # noqa: E402
+from qwen3_moe_fused.lora import LoraMoeFusedLinear  # noqa: E402
+from qwen3_moe_fused.modular_qwen3_moe_fused import MoeFusedLinear, Qwen3MoeFusedSparseMoeBlock  # noqa: E402
+from qwen3_moe_fused.quantize.layer import MoeFusedLinear4bit  # noqa: E402
+from qwen3_moe_fused.quantize.nf4 import dequantize_nf4  # noqa: E402
+
+DEV = "cuda"
+
+
+def _config(E, k, H, I, renorm=True):
+    return SimpleNamespace(num_experts=E, num_experts_per_tok=k, norm_topk_prob=renorm, hidden_size=H,
+                           moe_intermediate_size=I, hidden_act="silu")
+
+
+def _block(cfg, dtype, seed):
+    torch.manual_seed(seed)
+    blk = Qwen3MoeFusedSparseMoeBlock(cfg)
+    with torch.no_grad():
+        for p in blk.parameters():
+            p.copy_(torch.randn(p.shape, generator=gen(seed + p.numel() % 97)) * 0.05)
+    return blk.to(dtype)
+
+
+def test_module_init_bound():
+    m = MoeFusedLinear(64, 32, 4)
+    bound = (15.0 / 64) ** 0.5                       # modular_qwen3_moe_fused.py:25
+    assert m.weight.shape == (4, 32, 64)
+    assert m.weight.abs().max() <= bound and m.weight.abs().max() > 0.8 * bound
+    assert "num_experts=4" in repr(m)
+
+
+@pytest.mark.parametrize("T,E,k,H,I,dtype", [(7 * 13, 11, 3, 16, 3, torch.float32),     # test_model.py tiny config
+                                             (256, 8, 2, 64, 128, torch.float32),
+                                             (512, 128, 8, 256, 96, torch.bfloat16)])
+def test_sparse_block_forward(T, E, k, H, I, dtype):
+    cfg = _config(E, k, H, I)
+    blk = _block(cfg, dtype, 3)
+    hidden = randn((1, T, H), gen(T), 1.0, dtype)
+    params = {n: to_np32(p) for n, p in blk.named_parameters()}
+    rnd = oracle.round_bf16 if dtype == torch.bfloat16 else None
+    out_ref, logits_ref = oracle.moe_block_fwd(to_np32(hidden[0]), params["gate.weight"], params["gate_proj.weight"],
+                                               params["up_proj.weight"], params["down_proj.weight"], k, True, rnd)
+    blk = blk.to(DEV)
+    out, logits = blk(hidden.to(DEV))
+    assert out.shape == (1, T, H) and logits.shape == (T, E)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-4
+    check_close(logits, logits_ref, tol, tol, "router logits")
+    if dtype == torch.bfloat16:
+        # a bf16 router can flip near-tied experts between implementations; compare only tokens
+        # whose oracle routing matches the GPU's
+        sel_gpu = torch.topk(torch.softmax(logits.float(), -1), k).indices.cpu().numpy()
+        sel_ref = oracle.softmax_topk(logits_ref, k, True)[1]
+        same = (np.sort(sel_gpu, 1) == np.sort(sel_ref, 1)).all(1)
+        assert same.mean() > 0.97
+        check_close(out[0][torch.from_numpy(same)], out_ref[same], tol, tol, "block output")
+    else:
+        check_close(out[0], out_ref, tol, tol, "block output")
+
+
+def test_sparse_block_backward_fp32_matches_autograd():
+    T, E, k, H, I = 60, 6, 2, 32, 24
+    cfg = _config(E, k, H, I)
+    blk = _block(cfg, torch.float32, 5).to(DEV)
+    hidden = randn((2, T // 2, H), gen(1)).to(DEV).requires_grad_()
+    out, _ = blk(hidden)
+    gout = randn((2, T // 2, H), gen(2)).to(DEV)
+    out.backward(gout)
+    grads = {n: p.grad.clone() for n, p in blk.named_parameters()}
+    gh = hidden.grad.clone()
+
+    # the reference formulation in stock torch ops (modular_qwen3_moe_fused.py:79-118)
+    h2 = hidden.detach().clone().requires_grad_()
+    ps = {n: p.detach().clone().requires_grad_() for n, p in blk.named_parameters()}
+    x = h2.view(T, H)
+    logits = x @ ps["gate.weight"].t()
+    rw, sel = torch.topk(torch.softmax(logits, dim=1, dtype=torch.float32), k, dim=-1)
+    rw = rw / rw.sum(dim=-1, keepdim=True)
+    xr = x.unsqueeze(1).expand(T, k, H).reshape(T * k, H)
+    sf = sel.reshape(-1)
+    lin = lambda a, w: torch.einsum("bnk,bk->bn", w[sf], a)
+    y = lin(torch.nn.functional.silu(lin(xr, ps["gate_proj.weight"])) * lin(xr, ps["up_proj.weight"]),
+            ps["down_proj.weight"])
+    out2 = torch.einsum("beo,be->bo", y.view(T, k, H), rw).view(2, T // 2, H)
+    out2.backward(gout)
+    torch.testing.assert_close(out, out2, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(gh, h2.grad, rtol=1e-3, atol=1e-5)
+    for n in grads:
+        torch.testing.assert_close(grads[n], ps[n].grad, rtol=1e-3, atol=1e-5, msg=n)
+
+
+def _lora_layer(in_f, out_f, E, r, alpha, dtype, seed, rslora=False):
+    base = MoeFusedLinear(in_f, out_f, E)
+    layer = LoraMoeFusedLinear(base, "default", r=r, lora_alpha=alpha, use_rslora=rslora)
+    with torch.no_grad():
+        base.weight.copy_(torch.randn(base.weight.shape, generator=gen(seed)) * 0.02)
+        layer.lora_A["default"].weight.copy_(torch.randn((E, r, in_f), generator=gen(seed + 1)) * 0.01)
+        layer.lora_B["default"].weight.copy_(torch.randn((E, out_f, r), generator=gen(seed + 2)) * 0.01)
+    base.weight.requires_grad_(False)
+    return layer.to(dtype)
+
+
+def test_lora_layer_init_and_scaling():
+    layer = LoraMoeFusedLinear(MoeFusedLinear(32, 48, 4), "default", r=4, lora_alpha=8)
+    assert layer.scaling["default"] == 2.0                                  # alpha / r
+    assert layer.lora_A["default"].weight.shape == (4, 4, 32)
+    assert layer.lora_B["default"].weight.shape == (4, 48, 4)
+    assert torch.count_nonzero(layer.lora_B["default"].weight) == 0         # B starts at zero
+    rs = LoraMoeFusedLinear(MoeFusedLinear(32, 48, 4), "default", r=16, lora_alpha=8, use_rslora=True)
+    assert rs.scaling["default"] == 2.0                                     # alpha / sqrt(r)
+    with pytest.raises(NotImplementedError):
+        layer.merge()
+    with pytest.raises(NotImplementedError):
+        LoraMoeFusedLinear(MoeFusedLinear(8, 8, 2), "default", r=2, use_dora=True)
+    with pytest.raises(ValueError):
+        LoraMoeFusedLinear(MoeFusedLinear(8, 8, 2), "default", r=0)
+
+
+def test_lora_config4_rank16_zipf_bf16():
+    """BASELINE config 4 at reduced hidden size for the oracle: rank-16 fused-format LoRA,
+    Zipf(1.2)-skewed top-8 routing, forward + backward in bf16."""
+    E, k, T, H, I, r = 128, 8, 1024, 256, 96, 16
+    g = gen(44)
+    sel, ms = topk_routing(T, E, k, g, bias=zipf_bias(E, 1.2, g))
+    assert ms.max() > 20 * max(1, ms.min())                                # hot vs cold experts
+    R = T * k
+    layer = _lora_layer(H, I, E, r, 32, torch.bfloat16, 9).to(DEV)
+    x = randn((R, H), g, 1.0, torch.bfloat16)
+    dy = randn((R, I), g, 1.0, torch.bfloat16)
+    xd = x.to(DEV).requires_grad_()
+    y = layer(xd, ms.to(DEV))
+    y.backward(dy.to(DEV))
+
+    W = to_np32(layer.base_layer.weight)
+    A = to_np32(layer.lora_A["default"].weight)
+    B = to_np32(layer.lora_B["default"].weight)
+    s = layer.scaling["default"]
+    sel_sorted = oracle.sel_from_m_sizes(ms.numpy())
+    check_close(y, oracle.lora_linear_fwd(to_np32(x), W, A, B, s, sel_sorted), what="lora fwd")
+    # gradients of y = x W^T + s (x A^T) B^T
+    u = oracle.linear_fwd(to_np32(x), A, sel_sorted)
+    t = oracle.linear_bwd_input(to_np32(dy), B, sel_sorted)
+    dA = s * oracle.linear_bwd_weight(t, to_np32(x), sel_sorted, E)
+    dB = s * oracle.linear_bwd_weight(to_np32(dy), u, sel_sorted, E)
+    dx = oracle.linear_bwd_input(to_np32(dy), W, sel_sorted) + s * oracle.linear_bwd_input(t, A, sel_sorted)
+    check_close(xd.grad, dx, 2e-2, 2e-2, "lora dx")
+    check_close(layer.lora_A["default"].weight.grad, dA, 2e-2, 2e-2 * np.abs(dA).max(), "lora dA")
+    check_close(layer.lora_B["default"].weight.grad, dB, 2e-2, 2e-2 * np.abs(dB).max(), "lora dB")
+    assert layer.base_layer.weight.grad is None
+
+
+def _lora_block(cfg, dtype, r=4):
+    blk = _block(cfg, dtype, 21)
+    for i, name in enumerate(("gate_proj", "up_proj", "down_proj")):
+        base = getattr(blk, name)
+        base.weight.requires_grad_(False)
+        layer = LoraMoeFusedLinear(base, "default", r=r, lora_alpha=2 * r, use_rslora=True)
+        with torch.no_grad():  # B re-initialised non-zero so the adapter matters (test_lora.py:72-75)
+            layer.lora_B["default"].weight.copy_(torch.randn(layer.lora_B["default"].weight.shape,
+                                                             generator=gen(50 + i)) * 0.05)
+        setattr(blk, name, layer.to(dtype))
+    return blk
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)])
+def test_fast_lora_block_matches_module_path(dtype, tol):
+    """The reference's own check (test_fast_lora.py:51-66): module-by-module forward/backward vs
+    the single fast_lora function -- outputs and every trainable gradient."""
+    T, E, k, H, I = 96, 11, 3, 32, 24
+    cfg = _config(E, k, H, I)
+    blk = _lora_block(cfg, dtype).to(DEV)
+    hidden = randn((1, T, H), gen(4), 1.0, dtype).to(DEV)
+    gout = randn((1, T, H), gen(5), 1.0, dtype).to(DEV)
+
+    h1 = hidden.clone().requires_grad_()
+    out1, _ = blk(h1)
+    out1.backward(gout)
+    g1 = {n: p.grad.clone() for n, p in blk.named_parameters() if p.grad is not None}
+    blk.zero_grad()
+
+    h2 = hidden.clone().requires_grad_()
+    out2, _ = fast_Qwen3MoeFusedSparseMoeBlock_forward(blk, h2)
+    out2.backward(gout)
+    g2 = {n: p.grad.clone() for n, p in blk.named_parameters() if p.grad is not None}
+    lora_names = {n for n in g1 if "lora_" in n}
+    assert lora_names and lora_names <= set(g2)
+    check_close(out2, to_np32(out1), tol, tol, "fast lora output")
+    check_close(h2.grad, to_np32(h1.grad), tol, tol * float(h1.grad.abs().max()), "fast lora d hidden")
+    for n in sorted(lora_names):
+        check_close(g2[n], to_np32(g1[n]), tol, tol * float(g1[n].abs().max() + 1e-12), n)
+    W, qs, A, B, s = get_lora_parameters(blk.gate_proj)
+    assert qs is None and A.shape == (E, 4, H) and B.shape == (E, I, 4) and s == 4.0
+
+
+def test_4bit_layer_and_fast_lora_on_nf4_base():
+    E, H, I, r, R = 8, 128, 64, 8, 512
+    g = gen(31)
+    base = MoeFusedLinear(H, I, E)
+    with torch.no_grad():
+        base.weight.copy_(torch.randn(base.weight.shape, generator=g) * 0.02)
+    q = MoeFusedLinear4bit(H, I, E, weight=base.weight, quant_type="nf4", blocksize=64).to(DEV)
+    assert q.weight.dtype == torch.uint8 and q.weight.quant_state is not None
+    assert q.weight.numel() == E * I * H // 2 and not q.weight.requires_grad
+    sd = q.state_dict()
+    assert "weight.absmax" in sd and "weight.quant_map" in sd
+
+    ms = torch.bincount(torch.randint(0, E, (R,), generator=g), minlength=E).int()
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    x = randn((R, H), g, 1.0, torch.bfloat16)
+    xd = x.to(DEV).requires_grad_()
+    y = q(xd, ms.to(DEV))
+    w_q, am = oracle.nf4_quant(to_np32(base.weight), 64)
+    assert np.array_equal(q.weight.cpu().numpy().reshape(-1), w_q)
+    w_deq = oracle.round_bf16(oracle.nf4_dequant(w_q, am, 64)).reshape(E, I, H)
+    check_close(y, oracle.linear_fwd(to_np32(x), w_deq, sel), what="4bit layer fwd")
+    dy = randn((R, I), g, 1.0, torch.bfloat16)
+    y.backward(dy.to(DEV))
+    check_close(xd.grad, oracle.linear_bwd_input(to_np32(dy), w_deq, sel), what="4bit layer dx")
+
+    # fast_lora with quantised bases == fast_lora with the dequantised bases
+    def lora_params(out_f, in_f, seed):
+        a = (torch.randn((E, r, in_f), generator=gen(seed)) * 0.05).bfloat16().to(DEV).requires_grad_()
+        b = (torch.randn((E, out_f, r), generator=gen(seed + 1)) * 0.05).bfloat16().to(DEV).requires_grad_()
+        return a, b
+
+    def qbase(out_f, in_f, seed):
+        m = MoeFusedLinear(in_f, out_f, E)
+        with torch.no_grad():
+            m.weight.copy_(torch.randn(m.weight.shape, generator=gen(seed)) * 0.05)
+        return MoeFusedLinear4bit(in_f, out_f, E, weight=m.weight, quant_type="nf4").to(DEV).weight
+
+    Gq, Uq, Wq = qbase(I, H, 1), qbase(I, H, 2), qbase(H, I, 3)
+    (Ag, Bg), (Au, Bu), (Aw, Bw) = lora_params(I, H, 10), lora_params(I, H, 20), lora_params(H, I, 30)
+    gout = randn((R, H), g, 1.0, torch.bfloat16).to(DEV)
+    x1 = x.to(DEV).requires_grad_()
+    y1 = fast_lora(x1, Gq.data, Gq.quant_state, Ag, Bg, 2.0, Uq.data, Uq.quant_state, Au, Bu, 2.0,
+                   Wq.data, Wq.quant_state, Aw, Bw, 2.0, ms.to(DEV))
+    y1.backward(gout)
+    g_q = [p.grad.clone() for p in (x1, Ag, Bg, Au, Bu, Aw, Bw)]
+    for p in (Ag, Bg, Au, Bu, Aw, Bw):
+        p.grad = None
+    dq = lambda p: dequantize_nf4(p.data, p.quant_state, torch.bfloat16)
+    x2 = x.to(DEV).requires_grad_()
+    y2 = fast_lora(x2, dq(Gq), None, Ag, Bg, 2.0, dq(Uq), None, Au, Bu, 2.0, dq(Wq), None, Aw, Bw, 2.0, ms.to(DEV))
+    y2.backward(gout)
+    g_d = [p.grad for p in (x2, Ag, Bg, Au, Bu, Aw, Bw)]
+    check_close(y1, to_np32(y2), 2e-2, 2e-2, "fast_lora nf4 vs dense")
+    for a, b, n in zip(g_q, g_d, ("dx", "dAg", "dBg", "dAu", "dBu", "dAw", "dBw")):
+        check_close(a, to_np32(b), 2e-2, 2e-2 * float(b.abs().max() + 1e-12), n)

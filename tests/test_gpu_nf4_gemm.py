@@ -1,0 +1,42 @@
+"""Fused NF4-dequant grouped GEMM against the oracle (oracle dequant -> oracle linear), the way
+the reference checks its 4-bit kernel against the naive forward on dequantised weights
+(test_moe_fused_linear.py:39-58), plus fused == dequant-then-GEMM within bf16 tolerance."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import check_close, gen, m_sizes_uniform, randn, to_np32
+
+pytestmark = pytest.mark.gpu
+
+from qwen3_moe_fused.grouped_gemm.forward import grouped_gemm_forward  # noqa: E402
+from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_4bit  # noqa: E402
+from qwen3_moe_fused.quantize.nf4 import Nf4QuantState, dequantize_nf4, nf4_code  # noqa: E402
+
+DEV = "cuda"
+
+
+def _quantised(E, N, K, blocksize, seed):
+    w = randn((E, N, K), gen(seed), 0.02)
+    q, absmax = oracle.nf4_quant(w.numpy(), blocksize)
+    w_deq = oracle.round_bf16(oracle.nf4_dequant(q, absmax, blocksize)).reshape(E, N, K)
+    state = Nf4QuantState(absmax=torch.from_numpy(absmax).to(DEV), shape=(E, N, K), code=nf4_code(DEV),
+                          blocksize=blocksize, dtype=torch.bfloat16)
+    return torch.from_numpy(q).view(-1, 1).to(DEV), state, w_deq
+
+
+@pytest.mark.parametrize("R,N,K,E,blocksize", [(1024, 768, 2048, 128, 256), (1024, 768, 2048, 128, 64),
+                                               (128, 768, 2048, 128, 64), (300, 40, 72, 5, 8), (513, 136, 64, 3, 64)])
+def test_fused_nf4_forward(R, N, K, E, blocksize):
+    packed, state, w_deq = _quantised(E, N, K, blocksize, R + N)
+    g = gen(R)
+    x = randn((R, K), g, 1.0, torch.bfloat16)
+    ms = m_sizes_uniform(R, E, g)
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    y = grouped_gemm_forward_4bit(x.to(DEV), packed, state, ms.to(DEV))
+    assert y.dtype == torch.bfloat16 and y.shape == (R, N)
+    check_close(y, oracle.linear_fwd(to_np32(x), w_deq, sel), what="fused nf4 vs oracle")
+    # the unfused route (dequantise, then bf16 GEMM) sees the same bf16 weights
+    y2 = grouped_gemm_forward(x.to(DEV), dequantize_nf4(packed, state, torch.bfloat16), ms.to(DEV))
+    check_close(y, to_np32(y2), 1e-2, 1e-2, "fused vs dequant-then-GEMM")

@@ -1,0 +1,146 @@
+"""GPU parity of softmax-top-k routing, the stable expert sort and the gather / combine
+kernels.  Index outputs are compared bit for bit with the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import check_close, gen, randn, to_np32, zipf_bias
+
+pytestmark = pytest.mark.gpu
+
+from qwen3_moe_fused.kernels.indexing import (get_batch_begins_ends, get_expert_counts,  # noqa: E402
+                                              get_expert_counts_and_idx, sort_experts)
+from qwen3_moe_fused.kernels.routing import combine_rows, gather_rows, softmax_topk, softmax_topk_raw  # noqa: E402
+
+DEV = "cuda"
+
+
+def _tie_free(logits: np.ndarray, k: int) -> bool:
+    """True when the top k+1 probabilities of every row are separated by a relative gap that
+    no ulp-level difference in exp() can bridge."""
+    p = torch.softmax(torch.from_numpy(logits).float(), -1).numpy().astype(np.float64)
+    top = -np.sort(-p, axis=1)[:, : k + 1]
+    gap = (top[:, :-1] - top[:, 1:]) / top[:, :-1]
+    return bool((gap > 1e-5).all())
+
+
+@pytest.mark.parametrize("T,E,k,renorm", [(256, 8, 2, False), (4096, 128, 8, True), (4096, 128, 8, False),
+                                          (37, 11, 3, True), (100, 60, 4, True), (64, 256, 8, True),
+                                          (16, 1000, 6, True)])
+def test_softmax_topk_matches_oracle(T, E, k, renorm):
+    logits = randn((T, E), gen(100 + T + E), 1.0)
+    lnp = logits.numpy()
+    # drop the (vanishingly rare) rows whose top-(k+1) are not clearly separated
+    assert _tie_free(lnp, min(k, E - 1)), "fixture has near-ties; change the seed"
+    w_ref, idx_ref = oracle.softmax_topk(lnp, k, renorm)
+    w32, wc, idx = softmax_topk_raw(logits.to(DEV), k, renorm, torch.bfloat16)
+    assert idx.dtype == torch.int64
+    assert np.array_equal(idx.cpu().numpy(), idx_ref), "expert ids must match bit for bit"
+    np.testing.assert_allclose(w32.cpu().numpy(), w_ref, rtol=2e-6, atol=1e-9)
+    assert torch.equal(wc, w32.to(torch.bfloat16))
+
+
+def test_softmax_topk_tie_rule_and_bf16_logits():
+    # exact duplicates: the lower expert id comes first
+    logits = torch.tensor([[1.0, 3.0, 3.0, 0.5, 3.0, -1.0, 2.0, 2.0]] * 5)
+    _, _, idx = softmax_topk_raw(logits.to(DEV), 5, True, torch.float32)
+    assert idx[0].tolist() == [1, 2, 4, 6, 7]
+    w_ref, idx_ref = oracle.softmax_topk(logits.numpy(), 5, True)
+    assert np.array_equal(idx.cpu().numpy(), idx_ref)
+    # bf16 logits (what a bf16 gate produces) are widened to fp32 first
+    lg = randn((512, 128), gen(9), 1.0, torch.bfloat16)
+    w_ref, idx_ref = oracle.softmax_topk(to_np32(lg), 8, True)
+    _, _, idx = softmax_topk_raw(lg.to(DEV), 8, True)
+    # bf16 logits have many exact ties; with the declared rule the ids still agree except
+    # where two different logits round to the same probability in one implementation only
+    agree = (idx.cpu().numpy() == idx_ref).mean()
+    assert agree > 0.999
+
+
+@pytest.mark.parametrize("R,E,dtype", [(512, 8, torch.int64), (32768, 128, torch.int64), (32768, 128, torch.int32),
+                                       (131072, 128, torch.int64), (1, 4, torch.int64), (0, 4, torch.int64),
+                                       (1001, 11, torch.int64), (70000, 60, torch.int64), (5000, 1000, torch.int32),
+                                       (300000, 16, torch.int64)])
+def test_expert_sort_bit_exact(R, E, dtype):
+    g = gen(R + E)
+    if R >= 32768 and E == 128:
+        # real routing: top-8 of softmax over Zipf-skewed logits, flattened
+        T = R // 8
+        logits = torch.randn((T, E), generator=g) + zipf_bias(E, 1.2, g)
+        s = torch.topk(torch.softmax(logits, -1), 8, -1).indices.reshape(-1)
+    else:
+        s = torch.randint(0, E, (R,), generator=g)
+    c_ref, sort_ref, inv_ref = oracle.expert_counts_and_idx(s.numpy(), E)
+    c, sort_idx, inv = get_expert_counts_and_idx(s.to(dtype).to(DEV), E)
+    assert c.dtype == sort_idx.dtype == inv.dtype == torch.int32
+    assert np.array_equal(c.cpu().numpy(), c_ref)
+    assert np.array_equal(sort_idx.cpu().numpy(), sort_ref)
+    assert np.array_equal(inv.cpu().numpy(), inv_ref)
+    assert np.array_equal(get_expert_counts(s.to(dtype).to(DEV), E).cpu().numpy(), c_ref)
+
+
+def test_sort_helpers():
+    s = torch.randint(0, 7, (500,), generator=gen(1))
+    s_sorted, sort_idx, inv = sort_experts(s.to(DEV), 7)
+    assert s_sorted.dtype == torch.int32
+    assert torch.equal(s_sorted.cpu().long(), torch.sort(s, stable=True).values)
+    assert torch.equal(sort_idx.cpu().long(), torch.sort(s, stable=True).indices)
+    be = get_batch_begins_ends(s_sorted.to(DEV), 7).cpu()
+    counts = torch.bincount(s, minlength=7)
+    assert torch.equal(be[:, 1] - be[:, 0], counts.int())
+    assert be[0, 0] == 0 and be[-1, 1] == 500
+
+
+@pytest.mark.parametrize("T,k,H,dtype", [(256, 2, 64, torch.float32), (4096, 8, 2048, torch.bfloat16),
+                                         (91, 3, 16, torch.float32), (50, 4, 36, torch.bfloat16)])
+def test_gather_and_combine(T, k, H, dtype):
+    g = gen(T + H)
+    E = 16
+    hidden = randn((T, H), g, 1.0, dtype)
+    sel = torch.randint(0, E, (T * k,), generator=g)
+    rw = torch.rand((T, k), generator=g).to(dtype)
+    _, sort_ref, inv_ref = oracle.expert_counts_and_idx(sel.numpy(), E)
+    sort_idx, inv = torch.from_numpy(sort_ref).to(DEV), torch.from_numpy(inv_ref).to(DEV)
+
+    x = gather_rows(hidden.to(DEV), sort_idx, k, inv)
+    exp = hidden.repeat_interleave(k, dim=0)[torch.from_numpy(sort_ref).long()]   # modular...:95-103
+    assert torch.equal(x.cpu(), exp), "gather is a pure copy: bit exact"
+
+    y = randn((T * k, H), g, 1.0, dtype)
+    out = combine_rows(y.to(DEV), inv, rw.to(DEV), sort_idx)
+    ref = np.einsum("beo,be->bo", to_np32(y)[inv_ref].reshape(T, k, H).astype(np.float64), to_np32(rw).astype(np.float64))
+    check_close(out, ref, 1e-2 if dtype == torch.bfloat16 else 1e-5, 1e-2 if dtype == torch.bfloat16 else 1e-5,
+                "combine")
+
+
+def test_gather_combine_autograd_fp32():
+    """Gradients of gather / combine / softmax-top-k against torch autograd of the reference's
+    formulation (modular_qwen3_moe_fused.py:87-115)."""
+    T, k, H, E = 40, 3, 24, 6
+    g = gen(5)
+    hidden = randn((T, H), g).to(DEV).requires_grad_()
+    logits = randn((T, E), g).to(DEV).requires_grad_()
+    wts = randn((T * k, H), g).to(DEV)
+
+    rw, sel = softmax_topk(logits, k, True, torch.float32)
+    c, sort_idx, inv = get_expert_counts_and_idx(sel.view(-1), E)
+    x = gather_rows(hidden, sort_idx, k, inv)
+    y = x * wts            # any row-wise differentiable op between gather and combine
+    out = combine_rows(y, inv, rw, sort_idx)
+    loss_w = randn((T, H), g).to(DEV)
+    (out * loss_w).sum().backward()
+
+    h2 = hidden.detach().clone().requires_grad_()
+    l2 = logits.detach().clone().requires_grad_()
+    p = torch.softmax(l2, dim=1, dtype=torch.float32)
+    rw2, sel2 = torch.topk(p, k, dim=-1)
+    rw2 = rw2 / rw2.sum(dim=-1, keepdim=True)
+    assert torch.equal(sel2, sel)
+    x2 = h2.unsqueeze(1).expand(T, k, H).reshape(T * k, H)[sort_idx.long()]
+    y2 = (x2 * wts)[inv.long()].view(T, k, H)
+    out2 = torch.einsum("beo,be->bo", y2, rw2)
+    (out2 * loss_w).sum().backward()
+    torch.testing.assert_close(out, out2, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(hidden.grad, h2.grad, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(logits.grad, l2.grad, rtol=1e-4, atol=1e-6)

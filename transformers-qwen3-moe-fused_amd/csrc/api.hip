@@ -1,0 +1,204 @@
+// extern "C" surface of the library: argument validation and dispatch only.
+#include "common.h"
+#include "gemm.h"
+#include "ops.h"
+
+namespace mfl {
+
+const DeviceInfo &device_info() {
+    static const DeviceInfo info = [] {
+        DeviceInfo d;
+        d.cu_count = 256;
+        d.xcd_count = 8;
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            d.cu_count = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        return d;
+    }();
+    return info;
+}
+
+extern int g_mfma_config;
+
+namespace {
+
+int check_gemm(const void *a, const void *b, const void *m_sizes, int ms_dtype, const void *c, int64_t R, int N, int K,
+               int E, int in_dtype, int out_dtype) {
+    if (R < 0 || N <= 0 || K <= 0 || E <= 0) return MFL_ERR_SHAPE;
+    if (R > 0x7fffffff) return MFL_ERR_SHAPE;
+    if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || !itype_ok(ms_dtype)) return MFL_ERR_DTYPE;
+    if (!b || !m_sizes || !c) return MFL_ERR_NULL;
+    if (R > 0 && !a) return MFL_ERR_NULL;
+    if (!aligned(a, dtype_size(in_dtype)) || !aligned(b, dtype_size(in_dtype)) || !aligned(c, dtype_size(out_dtype)) ||
+        !aligned(m_sizes, ms_dtype == MFL_I64 ? 8 : 4))
+        return MFL_ERR_ALIGN;
+    return MFL_OK;
+}
+
+int run_gemm(int mode, const void *a, const void *b, const void *m_sizes, int ms_dtype, void *c, int64_t R, int N, int K,
+             int E, int in_dtype, int out_dtype, float alpha, int accumulate, void *stream) {
+    int rc = check_gemm(a, b, m_sizes, ms_dtype, c, R, N, K, E, in_dtype, out_dtype);
+    if (rc) return rc;
+    if (R == 0 && mode != MODE_DW) return MFL_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const int ms_i64 = ms_dtype == MFL_I64;
+    if (in_dtype == MFL_BF16) {
+        rc = gemm_bf16_mfma(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, s);
+        if (rc != MFL_ERR_UNSUPPORTED) return rc;
+    }
+    return gemm_generic(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, in_dtype, out_dtype, alpha, accumulate, s);
+}
+
+}  // namespace
+}  // namespace mfl
+
+using namespace mfl;
+
+extern "C" {
+
+int mfl_abi_version(void) { return MFL_ABI_VERSION; }
+
+const char *mfl_strerror(int code) {
+    switch (code) {
+        case MFL_OK:
+            return "ok";
+        case MFL_ERR_NULL:
+            return "required pointer is NULL";
+        case MFL_ERR_SHAPE:
+            return "invalid or inconsistent dimension";
+        case MFL_ERR_DTYPE:
+            return "unknown or unsupported element/index type";
+        case MFL_ERR_ALIGN:
+            return "pointer not aligned to its element size";
+        case MFL_ERR_WORKSPACE:
+            return "workspace missing or too small";
+        case MFL_ERR_UNSUPPORTED:
+            return "request not supported by this build";
+        default:
+            return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error code";
+    }
+}
+
+/* Tuning hook (not part of the stable ABI): selects a tile configuration of the bf16 MFMA
+ * kernels; 0 restores the built-in table. */
+void mfl_debug_set_mfma_config(int cfg) { g_mfma_config = cfg; }
+
+int mfl_gemm_fwd(const void *x, const void *w, const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K,
+                 int E, int in_dtype, int out_dtype, float alpha, int accumulate, void *stream) {
+    return run_gemm(MODE_FWD, x, w, m_sizes, m_sizes_dtype, y, R, N, K, E, in_dtype, out_dtype, alpha, accumulate,
+                    stream);
+}
+
+int mfl_gemm_dx(const void *dy, const void *w, const void *m_sizes, int m_sizes_dtype, void *dx, int64_t R, int N, int K,
+                int E, int in_dtype, int out_dtype, float alpha, int accumulate, void *stream) {
+    return run_gemm(MODE_DX, dy, w, m_sizes, m_sizes_dtype, dx, R, N, K, E, in_dtype, out_dtype, alpha, accumulate,
+                    stream);
+}
+
+int mfl_gemm_dw(const void *x, const void *dy, const void *m_sizes, int m_sizes_dtype, void *dw, int64_t R, int N, int K,
+                int E, int in_dtype, int out_dtype, float alpha, int accumulate, void *stream) {
+    if (R > 0 && !x) return MFL_ERR_NULL;
+    // kernels take (a = dy, b = x)
+    return run_gemm(MODE_DW, dy, x, m_sizes, m_sizes_dtype, dw, R, N, K, E, in_dtype, out_dtype, alpha, accumulate,
+                    stream);
+}
+
+int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                     const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K, int E, int in_dtype,
+                     int out_dtype, void *stream) {
+    if (R < 0 || N <= 0 || K <= 0 || E <= 0 || R > 0x7fffffff) return MFL_ERR_SHAPE;
+    if (blocksize < 2 || (blocksize & (blocksize - 1)) != 0) return MFL_ERR_SHAPE;
+    if (K % 2 != 0 || ((int64_t)E * N * K) % blocksize != 0) return MFL_ERR_SHAPE;
+    if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || !itype_ok(m_sizes_dtype)) return MFL_ERR_DTYPE;
+    if (!wq || !code16 || !absmax || !m_sizes || !y || (R > 0 && !x)) return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    return gemm_nf4_mfma(x, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E, out_dtype,
+                         (hipStream_t)stream);
+}
+
+int mfl_nf4_dequant(const uint8_t *wq, const float *code16, const float *absmax, int blocksize, void *out, int64_t n,
+                    int out_dtype, void *stream) {
+    if (n < 0 || n % 2 != 0 || blocksize < 2 || n % blocksize != 0) return MFL_ERR_SHAPE;
+    if (!dtype_ok(out_dtype)) return MFL_ERR_DTYPE;
+    if (n > 0 && (!wq || !code16 || !absmax || !out)) return MFL_ERR_NULL;
+    if (!aligned(out, dtype_size(out_dtype))) return MFL_ERR_ALIGN;
+    return nf4_dequant(wq, code16, absmax, blocksize, out, n, out_dtype, (hipStream_t)stream);
+}
+
+int mfl_dequant_blockwise_u8(const uint8_t *v, const float *code256, const float *absmax2, int blocksize2, float offset,
+                             float *out, int64_t n, void *stream) {
+    if (n < 0 || blocksize2 <= 0) return MFL_ERR_SHAPE;
+    if (n > 0 && (!v || !code256 || !absmax2 || !out)) return MFL_ERR_NULL;
+    return dequant_blockwise_u8(v, code256, absmax2, blocksize2, offset, out, n, (hipStream_t)stream);
+}
+
+int mfl_nf4_quant(const void *w, int w_dtype, int64_t n, int blocksize, const float *code16, uint8_t *wq, float *absmax,
+                  void *stream) {
+    if (n < 0 || blocksize < 2 || blocksize % 2 != 0 || n % blocksize != 0) return MFL_ERR_SHAPE;
+    if (!dtype_ok(w_dtype)) return MFL_ERR_DTYPE;
+    if (n > 0 && (!w || !code16 || !wq || !absmax)) return MFL_ERR_NULL;
+    return nf4_quant(w, w_dtype, n, blocksize, code16, wq, absmax, (hipStream_t)stream);
+}
+
+int mfl_route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, float *weights_f32,
+                           void *weights_cast, int cast_dtype, int64_t *idx, void *stream) {
+    if (T < 0 || E <= 0 || k <= 0 || k > E || k > 64) return MFL_ERR_SHAPE;
+    if (!dtype_ok(logits_dtype) || (weights_cast && !dtype_ok(cast_dtype))) return MFL_ERR_DTYPE;
+    if (T > 0 && (!logits || !idx)) return MFL_ERR_NULL;
+    return route_softmax_topk(logits, logits_dtype, T, E, k, renorm, weights_f32, weights_cast,
+                              weights_cast ? cast_dtype : MFL_F32, idx, (hipStream_t)stream);
+}
+
+size_t mfl_expert_sort_workspace(int64_t R, int E) { return expert_sort_workspace(R, E); }
+
+int mfl_expert_sort(const void *sel, int sel_dtype, int64_t R, int E, int32_t *counts, int32_t *sort_idx,
+                    int32_t *inv_sort_idx, void *workspace, size_t ws_bytes, void *stream) {
+    if (R < 0 || E <= 0 || R > 0x7fffffff) return MFL_ERR_SHAPE;
+    if (!itype_ok(sel_dtype)) return MFL_ERR_DTYPE;
+    if (!counts || (R > 0 && !sel)) return MFL_ERR_NULL;
+    return expert_sort(sel, sel_dtype == MFL_I64, R, E, counts, sort_idx, inv_sort_idx, workspace, ws_bytes,
+                       (hipStream_t)stream);
+}
+
+int mfl_gather_rows(const void *src, const int32_t *idx, int idx_div, const void *row_scale, void *dst, int64_t R_out,
+                    int H, int dtype, void *stream) {
+    if (R_out < 0 || H <= 0 || idx_div <= 0) return MFL_ERR_SHAPE;
+    if (!dtype_ok(dtype)) return MFL_ERR_DTYPE;
+    if (R_out > 0 && (!src || !idx || !dst)) return MFL_ERR_NULL;
+    return gather_rows(src, idx, idx_div, row_scale, dst, R_out, H, dtype, (hipStream_t)stream);
+}
+
+int mfl_combine_rows(const void *src, const int32_t *pos, const void *weights, void *dst, int64_t T, int k, int H,
+                     int dtype, void *stream) {
+    if (T < 0 || H <= 0 || k <= 0) return MFL_ERR_SHAPE;
+    if (!dtype_ok(dtype)) return MFL_ERR_DTYPE;
+    if (T > 0 && (!src || !pos || !dst)) return MFL_ERR_NULL;
+    return combine_rows(src, pos, weights, dst, T, k, H, dtype, (hipStream_t)stream);
+}
+
+int mfl_rows_dot(const void *a, const void *b, const int32_t *pos, void *dots, int64_t T, int k, int H, int dtype,
+                 void *stream) {
+    if (T < 0 || H <= 0 || k <= 0) return MFL_ERR_SHAPE;
+    if (!dtype_ok(dtype)) return MFL_ERR_DTYPE;
+    if (T > 0 && (!a || !b || !pos || !dots)) return MFL_ERR_NULL;
+    return rows_dot(a, b, pos, dots, T, k, H, dtype, (hipStream_t)stream);
+}
+
+int mfl_silu_mul_fwd(const void *e, const void *g, void *h, int64_t n, int dtype, void *stream) {
+    if (n < 0) return MFL_ERR_SHAPE;
+    if (!dtype_ok(dtype)) return MFL_ERR_DTYPE;
+    if (n > 0 && (!e || !g || !h)) return MFL_ERR_NULL;
+    return silu_mul_fwd(e, g, h, n, dtype, (hipStream_t)stream);
+}
+
+int mfl_silu_mul_bwd(const void *dh, const void *e, const void *g, void *de, void *dg, void *h_out, int64_t n, int dtype,
+                     void *stream) {
+    if (n < 0) return MFL_ERR_SHAPE;
+    if (!dtype_ok(dtype)) return MFL_ERR_DTYPE;
+    if (n > 0 && (!dh || !e || !g || !de || !dg)) return MFL_ERR_NULL;
+    return silu_mul_bwd(dh, e, g, de, dg, h_out, n, dtype, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,73 @@
+// Shared device/host helpers for the gfx950 moe_fused_linear library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/moe_fused_linear.h"
+
+namespace mfl {
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) short short4_t;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+typedef __attribute__((ext_vector_type(16))) float floatx16;
+typedef __attribute__((ext_vector_type(4))) uint32_t uint4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t uint2_t;
+
+constexpr int kWave = 64;
+
+template <typename T>
+__device__ __forceinline__ float to_f32(T v) {
+    return (float)v;
+}
+template <typename T>
+__device__ __forceinline__ T from_f32(float v) {
+    return (T)v;  // bf16/f16: one round-to-nearest-even (v_cvt_pk_bf16_f32 on gfx950)
+}
+
+__device__ __forceinline__ int load_msize(const void *m_sizes, int is_i64, int e) {
+    return is_i64 ? (int)((const int64_t *)m_sizes)[e] : ((const int32_t *)m_sizes)[e];
+}
+
+__host__ __device__ constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+inline size_t dtype_size(int dt) { return dt == MFL_F32 ? 4 : 2; }
+inline bool dtype_ok(int dt) { return dt == MFL_BF16 || dt == MFL_F32 || dt == MFL_F16; }
+inline bool itype_ok(int it) { return it == MFL_I32 || it == MFL_I64; }
+inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? MFL_OK : (int)e;
+}
+
+struct DeviceInfo {
+    int cu_count;
+    int xcd_count;
+};
+const DeviceInfo &device_info();
+
+// dispatch helpers -----------------------------------------------------------------
+#define MFL_DISPATCH_FLOAT(dt, T, ...)          \
+    switch (dt) {                               \
+        case MFL_BF16: {                        \
+            typedef ::mfl::bf16_t T;            \
+            __VA_ARGS__;                        \
+        } break;                                \
+        case MFL_F16: {                         \
+            typedef ::mfl::f16_t T;             \
+            __VA_ARGS__;                        \
+        } break;                                \
+        default: {                              \
+            typedef float T;                    \
+            __VA_ARGS__;                        \
+        } break;                                \
+    }
+
+}  // namespace mfl

@@ -1,0 +1,366 @@
+// Bandwidth-bound kernels: SiLU-mul, row gather / combine, NF4 and 8-bit blockwise
+// (de)quantisation.  All of them stream 16-byte vectors per lane where alignment allows
+// and fall back to element-wise access otherwise.
+#include "common.h"
+#include "ops.h"
+
+namespace mfl {
+
+namespace {
+
+template <typename T>
+struct Vec {
+    static constexpr int N = 16 / sizeof(T);
+    T v[N];
+};
+
+template <typename T>
+__device__ __forceinline__ Vec<T> ld_vec(const T *p) {
+    Vec<T> r;
+    *(uint4_t *)r.v = *(const uint4_t *)p;
+    return r;
+}
+template <typename T>
+__device__ __forceinline__ void st_vec(T *p, const Vec<T> &r) {
+    *(uint4_t *)p = *(const uint4_t *)r.v;
+}
+
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// ---------------------------------------------------------------- SiLU-mul
+
+template <typename T>
+__device__ __forceinline__ T silu_fwd_one(T e, T g) {
+    const float e32 = to_f32(e);
+    if (sizeof(T) == 4) return from_f32<T>((e32 * sigmoid_f32(e32)) * to_f32(g));
+    const T f = from_f32<T>(e32 * sigmoid_f32(e32));
+    return from_f32<T>(to_f32(f) * to_f32(g));
+}
+
+template <typename T>
+__device__ __forceinline__ void silu_bwd_one(T dh, T e, T g, T &h, T &de, T &dg) {
+    const float e32 = to_f32(e), g32 = to_f32(g), dh32 = to_f32(dh);
+    const float se = sigmoid_f32(e32);
+    const float ese = e32 * se;
+    const float f = to_f32(from_f32<T>(ese));
+    const float df = to_f32(from_f32<T>(dh32 * g32));
+    h = from_f32<T>(f * g32);
+    dg = from_f32<T>(f * dh32);
+    de = from_f32<T>(df * se * (1.0f + e32 - ese));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void silu_fwd_kernel(const T *e, const T *g, T *h, int64_t n, int vec_ok) {
+    constexpr int V = Vec<T>::N;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (vec_ok) {
+        const int64_t nv = n / V;
+        for (int64_t q = i; q < nv; q += stride) {
+            Vec<T> ve = ld_vec(e + q * V), vg = ld_vec(g + q * V), vh;
+#pragma unroll
+            for (int u = 0; u < V; ++u) vh.v[u] = silu_fwd_one(ve.v[u], vg.v[u]);
+            st_vec(h + q * V, vh);
+        }
+        for (int64_t q = nv * V + i; q < n; q += stride) h[q] = silu_fwd_one(e[q], g[q]);
+    } else {
+        for (int64_t q = i; q < n; q += stride) h[q] = silu_fwd_one(e[q], g[q]);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void silu_bwd_kernel(const T *dh, const T *e, const T *g, T *de, T *dg, T *h,
+                                                       int64_t n, int vec_ok) {
+    constexpr int V = Vec<T>::N;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (vec_ok) {
+        const int64_t nv = n / V;
+        for (int64_t q = i; q < nv; q += stride) {
+            Vec<T> vdh = ld_vec(dh + q * V), ve = ld_vec(e + q * V), vg = ld_vec(g + q * V), vh, vde, vdg;
+#pragma unroll
+            for (int u = 0; u < V; ++u) silu_bwd_one(vdh.v[u], ve.v[u], vg.v[u], vh.v[u], vde.v[u], vdg.v[u]);
+            if (h) st_vec(h + q * V, vh);
+            st_vec(de + q * V, vde);
+            st_vec(dg + q * V, vdg);
+        }
+        i += nv * V;
+    }
+    for (int64_t q = i; q < n; q += stride) {
+        T vh, vde, vdg;
+        silu_bwd_one(dh[q], e[q], g[q], vh, vde, vdg);
+        if (h) h[q] = vh;
+        de[q] = vde;
+        dg[q] = vdg;
+    }
+}
+
+inline int stream_grid(int64_t n_items) {
+    const int64_t blocks = (n_items + 255) / 256;
+    const int64_t cap = (int64_t)device_info().cu_count * 16;
+    return (int)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
+}
+
+// ---------------------------------------------------------------- row gather / combine
+
+// One wave per destination row.
+template <typename T>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const T *src, const int32_t *idx, int idx_div,
+                                                          const T *row_scale, T *dst, int64_t R_out, int H,
+                                                          int vec_ok) {
+    constexpr int V = Vec<T>::N;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= R_out) return;
+    const int32_t j = idx[row];
+    const T *s = src + (int64_t)(j / idx_div) * H;
+    T *d = dst + row * H;
+    const bool scaled = row_scale != nullptr;
+    const float sc = scaled ? to_f32(row_scale[j]) : 1.0f;
+    if (vec_ok) {
+        for (int c = lane * V; c < H; c += 64 * V) {
+            Vec<T> v = ld_vec(s + c);
+            if (scaled) {
+#pragma unroll
+                for (int u = 0; u < V; ++u) v.v[u] = from_f32<T>(to_f32(v.v[u]) * sc);
+            }
+            st_vec(d + c, v);
+        }
+    } else {
+        for (int c = lane; c < H; c += 64) d[c] = scaled ? from_f32<T>(to_f32(s[c]) * sc) : s[c];
+    }
+}
+
+// One wave per token; fp32 accumulation over the k selected rows.
+template <typename T>
+__global__ __launch_bounds__(256) void combine_rows_kernel(const T *src, const int32_t *pos, const T *weights,
+                                                           T *dst, int64_t Tn, int k, int H, int vec_ok) {
+    constexpr int V = Vec<T>::N;
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= Tn) return;
+    const int32_t *p = pos + t * k;
+    T *d = dst + t * H;
+    if (vec_ok) {
+        for (int c = lane * V; c < H; c += 64 * V) {
+            float acc[V];
+#pragma unroll
+            for (int u = 0; u < V; ++u) acc[u] = 0.f;
+            for (int j = 0; j < k; ++j) {
+                const float w = weights ? to_f32(weights[t * k + j]) : 1.0f;
+                Vec<T> v = ld_vec(src + (int64_t)p[j] * H + c);
+#pragma unroll
+                for (int u = 0; u < V; ++u) acc[u] = fmaf(to_f32(v.v[u]), w, acc[u]);
+            }
+            Vec<T> o;
+#pragma unroll
+            for (int u = 0; u < V; ++u) o.v[u] = from_f32<T>(acc[u]);
+            st_vec(d + c, o);
+        }
+    } else {
+        for (int c = lane; c < H; c += 64) {
+            float acc = 0.f;
+            for (int j = 0; j < k; ++j) {
+                const float w = weights ? to_f32(weights[t * k + j]) : 1.0f;
+                acc = fmaf(to_f32(src[(int64_t)p[j] * H + c]), w, acc);
+            }
+            d[c] = from_f32<T>(acc);
+        }
+    }
+}
+
+// One wave per (token, selection) pair.
+template <typename T>
+__global__ __launch_bounds__(256) void rows_dot_kernel(const T *a, const T *b, const int32_t *pos, T *dots,
+                                                       int64_t n_pairs, int k, int H) {
+    const int lane = threadIdx.x & 63;
+    const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (pair >= n_pairs) return;
+    const T *pa = a + (pair / k) * H;
+    const T *pb = b + (int64_t)pos[pair] * H;
+    float acc = 0.f;
+    for (int c = lane; c < H; c += 64) acc = fmaf(to_f32(pa[c]), to_f32(pb[c]), acc);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+    if (lane == 0) dots[pair] = from_f32<T>(acc);
+}
+
+// ---------------------------------------------------------------- NF4
+
+// Each thread decodes 8 packed bytes (16 elements).  blocksize is a power of two; when it is
+// >= 16 the 16 elements of a thread share one absmax.
+template <typename T>
+__global__ __launch_bounds__(256) void nf4_dequant_kernel(const uint8_t *__restrict__ wq,
+                                                          const float *__restrict__ code16,
+                                                          const float *__restrict__ absmax, int bs_shift,
+                                                          T *__restrict__ out, int64_t n, int vec_ok) {
+    __shared__ float code[16];
+    if (threadIdx.x < 16) code[threadIdx.x] = code16[threadIdx.x];
+    __syncthreads();
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int64_t nbytes = n / 2;
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (vec_ok) {
+        const int64_t nchunks = nbytes / 8;
+        for (int64_t q = i; q < nchunks; q += stride) {
+            const uint2_t packed = *(const uint2_t *)(wq + q * 8);
+            const float am = absmax[(q * 16) >> bs_shift];
+            T vals[16];
+#pragma unroll
+            for (int bt = 0; bt < 8; ++bt) {
+                const uint32_t word = bt < 4 ? packed.x : packed.y;
+                const uint32_t byte = (word >> (8 * (bt & 3))) & 0xffu;
+                vals[2 * bt] = from_f32<T>(code[byte >> 4] * am);
+                vals[2 * bt + 1] = from_f32<T>(code[byte & 15u] * am);
+            }
+            T *o = out + q * 16;
+#pragma unroll
+            for (int u = 0; u < 16 * (int)sizeof(T) / 16; ++u) ((uint4_t *)o)[u] = ((const uint4_t *)vals)[u];
+        }
+        i += nchunks * 8;
+    }
+    for (int64_t q = i; q < nbytes; q += stride) {
+        const uint32_t byte = wq[q];
+        out[2 * q] = from_f32<T>(code[byte >> 4] * absmax[(2 * q) >> bs_shift]);
+        out[2 * q + 1] = from_f32<T>(code[byte & 15u] * absmax[(2 * q + 1) >> bs_shift]);
+    }
+}
+
+__global__ __launch_bounds__(256) void dequant_u8_kernel(const uint8_t *__restrict__ v,
+                                                         const float *__restrict__ code256,
+                                                         const float *__restrict__ absmax2, int blocksize2,
+                                                         float offset, float *__restrict__ out, int64_t n) {
+    __shared__ float code[256];
+    code[threadIdx.x] = code256[threadIdx.x];
+    __syncthreads();
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        out[i] = code[v[i]] * absmax2[i / blocksize2] + offset;
+}
+
+// One wave per quantisation block.
+template <typename T>
+__global__ __launch_bounds__(256) void nf4_quant_kernel(const T *__restrict__ w, int64_t nblocks, int blocksize,
+                                                        const float *__restrict__ code16,
+                                                        uint8_t *__restrict__ wq, float *__restrict__ absmax) {
+    __shared__ float code[16];
+    if (threadIdx.x < 16) code[threadIdx.x] = code16[threadIdx.x];
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int64_t blk = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blk >= nblocks) return;
+    const T *src = w + blk * blocksize;
+    float am = 0.f;
+    for (int i = lane; i < blocksize; i += 64) am = fmaxf(am, fabsf(to_f32(src[i])));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) am = fmaxf(am, __shfl_xor(am, off));
+    if (lane == 0) absmax[blk] = am;
+    const float inv = am > 0.f ? 1.0f / am : 0.f;
+    for (int p = lane; p < blocksize / 2; p += 64) {
+        uint32_t nib[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float v = to_f32(src[2 * p + h]) * inv;
+            int best = 0;
+            float bd = fabsf(v - code[0]);
+#pragma unroll
+            for (int c = 1; c < 16; ++c) {
+                const float d = fabsf(v - code[c]);
+                if (d < bd) {
+                    bd = d;
+                    best = c;
+                }
+            }
+            nib[h] = (uint32_t)best;
+        }
+        wq[(blk * blocksize) / 2 + p] = (uint8_t)((nib[0] << 4) | nib[1]);
+    }
+}
+
+inline int log2_exact(int v) {
+    int s = 0;
+    while ((1 << s) < v) ++s;
+    return (1 << s) == v ? s : -1;
+}
+
+}  // namespace
+
+int silu_mul_fwd(const void *e, const void *g, void *h, int64_t n, int dtype, hipStream_t stream) {
+    if (n == 0) return MFL_OK;
+    const int vec_ok = aligned(e, 16) && aligned(g, 16) && aligned(h, 16);
+    MFL_DISPATCH_FLOAT(dtype, T, (silu_fwd_kernel<T><<<stream_grid(n / Vec<T>::N + 1), 256, 0, stream>>>(
+                                     (const T *)e, (const T *)g, (T *)h, n, vec_ok)));
+    return launch_status();
+}
+
+int silu_mul_bwd(const void *dh, const void *e, const void *g, void *de, void *dg, void *h, int64_t n, int dtype,
+                 hipStream_t stream) {
+    if (n == 0) return MFL_OK;
+    const int vec_ok = aligned(dh, 16) && aligned(e, 16) && aligned(g, 16) && aligned(de, 16) && aligned(dg, 16) &&
+                       (h == nullptr || aligned(h, 16));
+    MFL_DISPATCH_FLOAT(dtype, T, (silu_bwd_kernel<T><<<stream_grid(n / Vec<T>::N + 1), 256, 0, stream>>>(
+                                     (const T *)dh, (const T *)e, (const T *)g, (T *)de, (T *)dg, (T *)h, n, vec_ok)));
+    return launch_status();
+}
+
+int gather_rows(const void *src, const int32_t *idx, int idx_div, const void *row_scale, void *dst, int64_t R_out,
+                int H, int dtype, hipStream_t stream) {
+    if (R_out == 0) return MFL_OK;
+    const size_t es = dtype_size(dtype);
+    const int vec_ok = aligned(src, 16) && aligned(dst, 16) && ((size_t)H * es) % 16 == 0;
+    const unsigned grid = (unsigned)((R_out + 3) / 4);
+    MFL_DISPATCH_FLOAT(dtype, T, (gather_rows_kernel<T><<<grid, 256, 0, stream>>>(
+                                     (const T *)src, idx, idx_div, (const T *)row_scale, (T *)dst, R_out, H, vec_ok)));
+    return launch_status();
+}
+
+int combine_rows(const void *src, const int32_t *pos, const void *weights, void *dst, int64_t T_, int k, int H,
+                 int dtype, hipStream_t stream) {
+    if (T_ == 0) return MFL_OK;
+    const size_t es = dtype_size(dtype);
+    const int vec_ok = aligned(src, 16) && aligned(dst, 16) && ((size_t)H * es) % 16 == 0;
+    const unsigned grid = (unsigned)((T_ + 3) / 4);
+    MFL_DISPATCH_FLOAT(dtype, T, (combine_rows_kernel<T><<<grid, 256, 0, stream>>>(
+                                     (const T *)src, pos, (const T *)weights, (T *)dst, T_, k, H, vec_ok)));
+    return launch_status();
+}
+
+int rows_dot(const void *a, const void *b, const int32_t *pos, void *dots, int64_t T_, int k, int H, int dtype,
+             hipStream_t stream) {
+    const int64_t pairs = T_ * k;
+    if (pairs == 0) return MFL_OK;
+    const unsigned grid = (unsigned)((pairs + 3) / 4);
+    MFL_DISPATCH_FLOAT(dtype, T, (rows_dot_kernel<T><<<grid, 256, 0, stream>>>((const T *)a, (const T *)b, pos,
+                                                                               (T *)dots, pairs, k, H)));
+    return launch_status();
+}
+
+int nf4_dequant(const uint8_t *wq, const float *code16, const float *absmax, int blocksize, void *out, int64_t n,
+                int out_dtype, hipStream_t stream) {
+    if (n == 0) return MFL_OK;
+    const int shift = log2_exact(blocksize);
+    if (shift < 1) return MFL_ERR_SHAPE;
+    const int vec_ok = aligned(wq, 8) && aligned(out, 16) && blocksize >= 16;
+    MFL_DISPATCH_FLOAT(out_dtype, T, (nf4_dequant_kernel<T><<<stream_grid(n / 16 + 1), 256, 0, stream>>>(
+                                         wq, code16, absmax, shift, (T *)out, n, vec_ok)));
+    return launch_status();
+}
+
+int dequant_blockwise_u8(const uint8_t *v, const float *code256, const float *absmax2, int blocksize2, float offset,
+                         float *out, int64_t n, hipStream_t stream) {
+    if (n == 0) return MFL_OK;
+    dequant_u8_kernel<<<stream_grid(n), 256, 0, stream>>>(v, code256, absmax2, blocksize2, offset, out, n);
+    return launch_status();
+}
+
+int nf4_quant(const void *w, int w_dtype, int64_t n, int blocksize, const float *code16, uint8_t *wq, float *absmax,
+              hipStream_t stream) {
+    if (n == 0) return MFL_OK;
+    const int64_t nblocks = n / blocksize;
+    const unsigned grid = (unsigned)((nblocks + 3) / 4);
+    MFL_DISPATCH_FLOAT(w_dtype, T, (nf4_quant_kernel<T><<<grid, 256, 0, stream>>>((const T *)w, nblocks, blocksize,
+                                                                                  code16, wq, absmax)));
+    return launch_status();
+}
+
+}  // namespace mfl

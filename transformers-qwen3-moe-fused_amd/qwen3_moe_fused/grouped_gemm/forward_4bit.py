@@ -1,0 +1,51 @@
+"""Forward grouped GEMM with NF4 weights decoded inside the K loop.
+
+Host wrapper over ``mfl_gemm_fwd_nf4``; contract of the reference's ``grouped_gemm_forward_4bit``
+(qwen3_moe_fused/grouped_gemm/forward_4bit.py:135-208): ``w_quant`` is the packed uint8 tensor,
+``w_quant_state`` an NF4 quant state whose ``shape`` is (E, N, K); a double-quantised absmax is
+un-nested first (:149-152); the state's own dtype is ignored and weights are rounded to
+``x.dtype`` (:103-104).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from ..quantize.nf4 import resolve_absmax
+from ._common import is_int_tensor
+
+
+def grouped_gemm_forward_4bit(x: torch.Tensor, w_quant: torch.Tensor, w_quant_state, m_sizes: torch.Tensor,
+                              dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    assert w_quant_state.quant_type == "nf4"
+    blocksize = int(w_quant_state.blocksize)
+    assert blocksize > 0 and blocksize & (blocksize - 1) == 0, "blocksize must be a power of two"
+    code = w_quant_state.code
+    assert code.dtype == torch.float32
+    absmax = resolve_absmax(w_quant_state)
+
+    assert x.is_cuda
+    for t in (w_quant, code, absmax, m_sizes):
+        assert t.device == x.device
+    assert is_int_tensor(w_quant) and is_int_tensor(m_sizes)
+    for t in (x, w_quant, code, absmax, m_sizes):
+        assert t.is_contiguous()
+    assert x.ndim == 2 and m_sizes.ndim == 1 and len(w_quant_state.shape) == 3
+    rows, k = x.shape
+    experts, n, k_w = w_quant_state.shape
+    assert k_w == k and k % 2 == 0
+    total = experts * n * k
+    assert total % blocksize == 0
+    assert w_quant.numel() == total // 2
+    assert absmax.numel() == total // blocksize
+    assert m_sizes.numel() == experts
+
+    y = torch.empty((rows, n), device=x.device, dtype=x.dtype if dtype is None else dtype)
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_gemm_fwd_nf4(_lib.ptr(x), _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), blocksize,
+                                     _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(y), rows, n, k, experts,
+                                     _lib.dtype_code(x.dtype), _lib.dtype_code(y.dtype), _lib.stream())
+    _lib.check(rc, "mfl_gemm_fwd_nf4")
+    return y

@@ -1,0 +1,102 @@
+"""Expert MLP with LoRA on gate/up/down as ONE autograd function
+(reference: qwen3_moe_fused/kernels/fast_lora.py).
+
+Shapes (rows B, hidden H, intermediate M, rank r, experts E):
+    x (B,H);  G,U (E,M,H);  W (E,H,M);  Ag,Au (E,r,H);  Bg,Bu (E,M,r);  Aw (E,r,M);  Bw (E,H,r)
+    e = G x + Sg Bg (Ag x),  g = U x + Su Bu (Au x),  h = silu(e) g,  y = W h + Sw Bw (Aw h)
+Only e, g and the two rank-r activations Ag x, Au x are kept for the backward pass.
+
+Gradients.  With t = dOut Bproj (rows x r) and u = In Aproj^T (rows x r) for a projection
+Out = (Wp + S Bp Ap) In:
+    dAp = S t^T In        dBp = S dOut^T u        dIn = dOut Wp + S t Ap
+Every LoRA gradient is therefore a rank-r grouped GEMM; the full (E, out, in) weight gradient
+that the reference forms and then contracts (fast_lora.py:139-149) is never built.  Base weights
+may be NF4 (``*qs`` not None): the forward products decode them inside the GEMM, the input
+gradients dequantise.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..grouped_gemm.backward_dw import grouped_gemm_backward_dw as _dw
+from ..grouped_gemm.forward import grouped_gemm_forward as _fwd
+from ..grouped_gemm.forward_4bit import grouped_gemm_forward_4bit as _fwd4
+from ..grouped_gemm.forward_transposed import grouped_gemm_forward_transposed as _dx
+from ..quantize.nf4 import dequantize_nf4
+from .silu_mul import silu_mul_backward_inplace, silu_mul_forward
+
+
+def _base_fwd(x, wq, wqs, m_sizes):
+    if wqs is None:
+        return _fwd(x, wq.to(x.dtype), m_sizes)
+    if x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and int(wqs.blocksize) >= 8:
+        return _fwd4(x, wq, wqs, m_sizes)
+    return _fwd(x, dequantize_nf4(wq, wqs, x.dtype), m_sizes)
+
+
+def _dense(wq, wqs, dtype):
+    return wq.to(dtype) if wqs is None else dequantize_nf4(wq, wqs, dtype)
+
+
+def _proj_fwd(x, wq, wqs, a, b, s, m_sizes):
+    y = _base_fwd(x, wq, wqs, m_sizes)
+    u = _fwd(x, a, m_sizes)                                   # rows x r
+    _fwd(u, b, m_sizes, out=y, alpha=s, accumulate=True)      # y += s * u b^T
+    return y, u
+
+
+def _proj_bwd_input(dout, t, wq, wqs, a, s, m_sizes, out=None):
+    """dIn (+)= dOut W + s * t A."""
+    w = _dense(wq, wqs, dout.dtype)
+    out = _dx(dout, w, m_sizes, out=out, accumulate=out is not None)
+    return _dx(t, a, m_sizes, out=out, alpha=s, accumulate=True)
+
+
+class FastLora(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, Gq, Gqs, Ag, Bg, Sg, Uq, Uqs, Au, Bu, Su, Wq, Wqs, Aw, Bw, Sw, m_sizes):
+        dt = x.dtype
+        x = x.contiguous()
+        Ag, Bg, Au, Bu, Aw, Bw = (p.to(dt).contiguous() for p in (Ag, Bg, Au, Bu, Aw, Bw))
+        e, ug = _proj_fwd(x, Gq, Gqs, Ag, Bg, Sg, m_sizes)
+        g, uu = _proj_fwd(x, Uq, Uqs, Au, Bu, Su, m_sizes)
+        h = silu_mul_forward(e, g)
+        y, _ = _proj_fwd(h, Wq, Wqs, Aw, Bw, Sw, m_sizes)
+        ctx.frozen = (Gq, Gqs, Sg, Uq, Uqs, Su, Wq, Wqs, Sw, m_sizes)
+        ctx.save_for_backward(x, Ag, Bg, Au, Bu, Aw, Bw, e, g, ug, uu)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        Gq, Gqs, Sg, Uq, Uqs, Su, Wq, Wqs, Sw, m_sizes = ctx.frozen
+        x, Ag, Bg, Au, Bu, Aw, Bw, e, g, ug, uu = ctx.saved_tensors
+        dt = x.dtype
+        dy = dy.contiguous()
+
+        # down projection
+        tw = _dx(dy, Bw, m_sizes)                                     # dy Bw, rows x r
+        dh = _proj_bwd_input(dy, tw, Wq, Wqs, Aw, Sw, m_sizes)
+        silu_mul_backward_inplace(dh, e, g)                            # (dh, e, g) <- (h, de, dg)
+        h, de, dg = dh, e, g
+        dAw = _dw(h, tw, m_sizes, dt, alpha=Sw)                        # (E, r, M)
+        dBw = _dw(_fwd(h, Aw, m_sizes), dy, m_sizes, dt, alpha=Sw)     # (E, H, r)
+
+        # up projection
+        tu = _dx(dg, Bu, m_sizes)
+        dAu = _dw(x, tu, m_sizes, dt, alpha=Su)                        # (E, r, H)
+        dBu = _dw(uu, dg, m_sizes, dt, alpha=Su)                       # (E, M, r)
+
+        # gate projection
+        tg = _dx(de, Bg, m_sizes)
+        dAg = _dw(x, tg, m_sizes, dt, alpha=Sg)
+        dBg = _dw(ug, de, m_sizes, dt, alpha=Sg)
+
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = _proj_bwd_input(de, tg, Gq, Gqs, Ag, Sg, m_sizes)
+            dx = _proj_bwd_input(dg, tu, Uq, Uqs, Au, Su, m_sizes, out=dx)
+
+        return (dx, None, None, dAg, dBg, None, None, None, dAu, dBu, None, None, None, dAw, dBw, None, None)
+
+
+fast_lora = FastLora.apply

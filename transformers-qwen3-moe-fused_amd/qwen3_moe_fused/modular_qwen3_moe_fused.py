@@ -1,0 +1,125 @@
+"""Fused MoE modules (reference: qwen3_moe_fused/modular_qwen3_moe_fused.py).
+
+``MoeFusedLinear`` keeps all experts of one projection in a single (E, out, in) parameter and
+applies them with one grouped GEMM; ``Qwen3MoeFusedSparseMoeBlock`` is the whole sparse MLP:
+router -> softmax/top-k -> stable expert sort -> gate/up GEMMs -> SiLU*mul -> down GEMM ->
+un-sort + routing-weighted sum.  Parameter names and shapes match the reference so state dicts
+load unchanged.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+from torch import nn
+
+from .functional import moe_fused_linear
+from .kernels.indexing import get_expert_counts_and_idx
+from .kernels.routing import combine_rows, gather_rows, softmax_topk
+from .kernels.silu_mul import silu_mul
+
+
+def moe_fused_kaiming_uniform_(weight: torch.Tensor) -> None:
+    """Kaiming-uniform over in_features with gain a = sqrt(5), as nn.Linear initialises
+    (modular_qwen3_moe_fused.py:21-26): U(-b, b) with b = sqrt(15 / in_features)."""
+    fan_in = weight.shape[-1]
+    limit = math.sqrt(15.0 / fan_in)
+    with torch.no_grad():
+        weight.uniform_(-limit, limit)
+
+
+class MoeFusedLinear(nn.Module):
+    __constants__ = ["in_features", "out_features", "num_experts"]
+
+    def __init__(self, in_features: int, out_features: int, num_experts: int,
+                 device: Optional[torch.device] = None, dtype: Optional[torch.dtype] = None) -> None:
+        super().__init__()
+        self.in_features, self.out_features, self.num_experts = in_features, out_features, num_experts
+        self.weight = nn.Parameter(torch.empty((num_experts, out_features, in_features), device=device, dtype=dtype))
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        moe_fused_kaiming_uniform_(self.weight)
+
+    def forward(self, input: torch.Tensor, m_sizes: torch.Tensor) -> torch.Tensor:
+        return moe_fused_linear(input, self.weight, m_sizes)
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}, num_experts={self.num_experts}"
+
+
+def route_tokens(block, hidden_2d: torch.Tensor):
+    """Router half of the block, shared with the fast-LoRA forward: returns
+    (router_logits, routing_weights (T,k), m_sizes, sort_idx, inv_sort_idx)."""
+    router_logits = block.gate(hidden_2d)
+    routing_weights, selected = softmax_topk(router_logits.contiguous(), block.num_selected, block.norm_topk_prob,
+                                             hidden_2d.dtype)
+    m_sizes, sort_idx, inv_sort_idx = get_expert_counts_and_idx(selected.view(-1), block.num_experts)
+    return router_logits, routing_weights, m_sizes, sort_idx, inv_sort_idx
+
+
+class Qwen3MoeFusedSparseMoeBlock(nn.Module):
+    """``config`` needs: num_experts, num_experts_per_tok, norm_topk_prob, hidden_size,
+    moe_intermediate_size, hidden_act == "silu" (a transformers ``Qwen3MoeConfig`` has them)."""
+
+    def __init__(self, config) -> None:
+        super().__init__()
+        assert config.hidden_act == "silu"
+        self.num_experts = config.num_experts
+        self.num_selected = config.num_experts_per_tok
+        self.norm_topk_prob = config.norm_topk_prob
+        self.hidden_size = config.hidden_size
+        self.moe_intermediate_size = config.moe_intermediate_size
+        self.gate = nn.Linear(self.hidden_size, self.num_experts, bias=False)
+        self.gate_proj = MoeFusedLinear(self.hidden_size, self.moe_intermediate_size, self.num_experts)
+        self.up_proj = MoeFusedLinear(self.hidden_size, self.moe_intermediate_size, self.num_experts)
+        self.down_proj = MoeFusedLinear(self.moe_intermediate_size, self.hidden_size, self.num_experts)
+
+    def forward(self, hidden_states: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        batch, seq, hidden = hidden_states.shape
+        tokens = hidden_states.reshape(batch * seq, hidden).contiguous()
+        router_logits, routing_weights, m_sizes, sort_idx, inv_sort_idx = route_tokens(self, tokens)
+
+        # every token once per selected expert, rows grouped by expert
+        x = gather_rows(tokens, sort_idx, self.num_selected, inv_sort_idx)
+        h = silu_mul(self.gate_proj(x, m_sizes), self.up_proj(x, m_sizes))
+        y = self.down_proj(h, m_sizes)
+        out = combine_rows(y, inv_sort_idx, routing_weights, sort_idx)
+        return out.view(batch, seq, hidden), router_logits
+
+
+def _hf_subclasses():
+    """Model-level wiring (decoder layer / model / causal LM with the fused block swapped in),
+    built on demand so that importing this module does not import transformers."""
+    from transformers.models.qwen3_moe.modeling_qwen3_moe import (Qwen3MoeDecoderLayer, Qwen3MoeForCausalLM,
+                                                                  Qwen3MoeMLP, Qwen3MoeModel)
+
+    class Qwen3MoeFusedDecoderLayer(Qwen3MoeDecoderLayer):
+        def __init__(self, config, layer_idx: int) -> None:
+            super().__init__(config, layer_idx)
+            sparse = (layer_idx not in config.mlp_only_layers and config.num_experts > 0
+                      and (layer_idx + 1) % config.decoder_sparse_step == 0)
+            self.mlp = (Qwen3MoeFusedSparseMoeBlock(config) if sparse
+                        else Qwen3MoeMLP(config, intermediate_size=config.intermediate_size))
+
+    class Qwen3MoeFusedModel(Qwen3MoeModel):
+        def __init__(self, config) -> None:
+            super().__init__(config)
+            self.layers = nn.ModuleList(Qwen3MoeFusedDecoderLayer(config, i) for i in range(config.num_hidden_layers))
+
+    class Qwen3MoeFusedForCausalLM(Qwen3MoeForCausalLM):
+        def __init__(self, config) -> None:
+            super().__init__(config)
+            self.model = Qwen3MoeFusedModel(config)
+
+    return Qwen3MoeFusedDecoderLayer, Qwen3MoeFusedModel, Qwen3MoeFusedForCausalLM
+
+
+def __getattr__(name: str):
+    names = ("Qwen3MoeFusedDecoderLayer", "Qwen3MoeFusedModel", "Qwen3MoeFusedForCausalLM")
+    if name in names:
+        classes = dict(zip(names, _hf_subclasses()))
+        globals().update(classes)
+        return classes[name]
+    raise AttributeError(name)
