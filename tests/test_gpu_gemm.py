@@ -30,7 +30,7 @@ def _case(seed, R, N, K, E, dtype, m_sizes=None):
 
 
 def _tol(dtype):
-    return (1e-2, 1e-2) if dtype != torch.float32 else (1e-4, 1e-5)
+    return (1e-2, 1e-2) if dtype != torch.float32 else (1e-4, 1e-4)  # the reference's fp32 figures (test_moe_fused_linear.py:30-32)
 
 
 SHAPES = [

@@ -16,13 +16,14 @@ from qwen3_moe_fused.kernels.routing import combine_rows, gather_rows, softmax_t
 DEV = "cuda"
 
 
-def _tie_free(logits: np.ndarray, k: int) -> bool:
-    """True when the top k+1 probabilities of every row are separated by a relative gap that
-    no ulp-level difference in exp() can bridge."""
-    p = torch.softmax(torch.from_numpy(logits).float(), -1).numpy().astype(np.float64)
+def _tie_free_rows(logits: np.ndarray, k: int) -> np.ndarray:
+    """Rows whose top k+1 probabilities are separated by a relative gap that no ulp-level
+    difference in exp() can bridge; only there is the top-k order independent of the exp()
+    implementation."""
+    p = torch.softmax(torch.from_numpy(logits).double(), -1).numpy()
     top = -np.sort(-p, axis=1)[:, : k + 1]
     gap = (top[:, :-1] - top[:, 1:]) / top[:, :-1]
-    return bool((gap > 1e-5).all())
+    return (gap > 1e-5).all(axis=1)
 
 
 @pytest.mark.parametrize("T,E,k,renorm", [(256, 8, 2, False), (4096, 128, 8, True), (4096, 128, 8, False),
@@ -31,12 +32,12 @@ def _tie_free(logits: np.ndarray, k: int) -> bool:
 def test_softmax_topk_matches_oracle(T, E, k, renorm):
     logits = randn((T, E), gen(100 + T + E), 1.0)
     lnp = logits.numpy()
-    # drop the (vanishingly rare) rows whose top-(k+1) are not clearly separated
-    assert _tie_free(lnp, min(k, E - 1)), "fixture has near-ties; change the seed"
+    clear = _tie_free_rows(lnp, min(k, E - 1))
+    assert clear.mean() > 0.99
     w_ref, idx_ref = oracle.softmax_topk(lnp, k, renorm)
     w32, wc, idx = softmax_topk_raw(logits.to(DEV), k, renorm, torch.bfloat16)
     assert idx.dtype == torch.int64
-    assert np.array_equal(idx.cpu().numpy(), idx_ref), "expert ids must match bit for bit"
+    assert np.array_equal(idx.cpu().numpy()[clear], idx_ref[clear]), "expert ids must match bit for bit"
     np.testing.assert_allclose(w32.cpu().numpy(), w_ref, rtol=2e-6, atol=1e-9)
     assert torch.equal(wc, w32.to(torch.bfloat16))
 

@@ -28,8 +28,8 @@ int check_gemm(const void *a, const void *b, const void *m_sizes, int ms_dtype, 
     if (R < 0 || N <= 0 || K <= 0 || E <= 0) return MFL_ERR_SHAPE;
     if (R > 0x7fffffff) return MFL_ERR_SHAPE;
     if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || !itype_ok(ms_dtype)) return MFL_ERR_DTYPE;
-    if (!b || !m_sizes || !c) return MFL_ERR_NULL;
-    if (R > 0 && !a) return MFL_ERR_NULL;
+    if (!m_sizes) return MFL_ERR_NULL;
+    if (R > 0 && (!a || !b || !c)) return MFL_ERR_NULL;
     if (!aligned(a, dtype_size(in_dtype)) || !aligned(b, dtype_size(in_dtype)) || !aligned(c, dtype_size(out_dtype)) ||
         !aligned(m_sizes, ms_dtype == MFL_I64 ? 8 : 4))
         return MFL_ERR_ALIGN;
@@ -41,6 +41,7 @@ int run_gemm(int mode, const void *a, const void *b, const void *m_sizes, int ms
     int rc = check_gemm(a, b, m_sizes, ms_dtype, c, R, N, K, E, in_dtype, out_dtype);
     if (rc) return rc;
     if (R == 0 && mode != MODE_DW) return MFL_OK;
+    if (mode == MODE_DW && !c) return MFL_ERR_NULL;  // dW is written (zeros) even without rows
     hipStream_t s = (hipStream_t)stream;
     const int ms_i64 = ms_dtype == MFL_I64;
     if (in_dtype == MFL_BF16) {
@@ -111,7 +112,7 @@ int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, cons
     if (blocksize < 2 || (blocksize & (blocksize - 1)) != 0) return MFL_ERR_SHAPE;
     if (K % 2 != 0 || ((int64_t)E * N * K) % blocksize != 0) return MFL_ERR_SHAPE;
     if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || !itype_ok(m_sizes_dtype)) return MFL_ERR_DTYPE;
-    if (!wq || !code16 || !absmax || !m_sizes || !y || (R > 0 && !x)) return MFL_ERR_NULL;
+    if (!wq || !code16 || !absmax || !m_sizes || (R > 0 && (!x || !y))) return MFL_ERR_NULL;
     if (R == 0) return MFL_OK;
     if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
     return gemm_nf4_mfma(x, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E, out_dtype,

@@ -101,14 +101,17 @@ class MoeFusedLinear4bit(MoeFusedLinear):
         self.quant_storage = quant_storage
 
     def _apply(self, fn, recurse=True):
-        # nn.Module._apply would strip the Parameter subclass; move the packed weight ourselves
-        packed = self.weight
-        probe = fn(torch.empty(0))
-        super()._apply(fn, recurse)
-        if isinstance(packed, Nf4Params):
-            moved = packed.to(probe.device) if probe.device != packed.device or packed.quant_state is None else packed
-            self._parameters["weight"] = moved
-            self.quant_state = moved.quant_state
+        # nn.Module._apply would swap the data under the Parameter subclass and drop its quant state:
+        # take the packed weight out, let the module move everything else, move the weight ourselves.
+        packed = self._parameters.pop("weight")
+        try:
+            super()._apply(fn, recurse)
+            target = fn(torch.empty(0, device=packed.device)).device
+            moved = packed.to(target) if isinstance(packed, Nf4Params) else fn(packed)
+        finally:
+            self._parameters["weight"] = packed
+        self._parameters["weight"] = moved
+        self.quant_state = getattr(moved, "quant_state", None)
         return self
 
     def set_compute_type(self, x: torch.Tensor) -> None:
