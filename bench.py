@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the moe_fused_linear hot path on one MI355X.
+
+A step is one forward grouped GEMM over one synthetic batch at BASELINE config 2
+(Qwen3-30B-A3B gate_proj: 128 experts, weight (128, 768, 2048) bf16, 4096 tokens routed
+top-8 -> 32768 rows sorted by expert).  Inputs are resident in HBM before the timed region.
+One JSON line is printed; dX / dW at config 3 and the bandwidth-bound neighbours are reported
+under "extra" from separate short timed loops.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "transformers-qwen3-moe-fused_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+E, HIDDEN, INTER, TOKENS, TOPK = 128, 2048, 768, 4096, 8
+ROWS = TOKENS * TOPK
+
+
+def _event_us(fn, iters, warm, stream):
+    import torch
+
+    for i in range(warm):
+        fn(i)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record(stream)
+    for i in range(iters):
+        fn(i)
+    stop.record(stream)
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e3 / iters
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing (profiling runs)")
+    ap.add_argument("--no-extra", action="store_true", help="time the forward GEMM only (profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from qwen3_moe_fused import _lib
+    from qwen3_moe_fused.grouped_gemm.backward_dw import grouped_gemm_backward_dw
+    from qwen3_moe_fused.grouped_gemm.forward import grouped_gemm_forward
+    from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_4bit
+    from qwen3_moe_fused.grouped_gemm.forward_transposed import grouped_gemm_forward_transposed
+    from qwen3_moe_fused.kernels.indexing import get_expert_counts_and_idx
+    from qwen3_moe_fused.kernels.routing import softmax_topk_raw
+    from qwen3_moe_fused.kernels.silu_mul import silu_mul_forward
+    from qwen3_moe_fused.quantize.nf4 import dequantize_nf4, quantize_nf4
+
+    _lib.lib()  # fail loudly when the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream()
+
+    # ---- synthetic inputs of config 2 (seeded on the CPU, then copied)
+    g = torch.Generator().manual_seed(0)
+    logits = torch.randn((TOKENS, E), generator=g)
+    x0 = torch.randn((ROWS, HIDDEN), generator=g).to(torch.bfloat16)
+    w0 = (torch.randn((E, INTER, HIDDEN), generator=g) * 0.02).to(torch.bfloat16)
+    _, _, sel = softmax_topk_raw(logits.to(dev), TOPK, True, torch.bfloat16)
+    m_sizes, sort_idx, inv_sort_idx = get_expert_counts_and_idx(sel.view(-1), E)
+    # three rotating copies: the 403 MB weight stream must come from HBM, not from the 256 MB MALL
+    NB = 3
+    xs = [x0.to(dev)] + [x0.to(dev).clone() for _ in range(NB - 1)]
+    ws = [w0.to(dev)] + [w0.to(dev).clone() for _ in range(NB - 1)]
+    ys = [torch.empty((ROWS, INTER), device=dev, dtype=torch.bfloat16) for _ in range(NB)]
+
+    def step(i):
+        grouped_gemm_forward(xs[i % NB], ws[i % NB], m_sizes, out=ys[i % NB])
+
+    for i in range(args.warmup):
+        step(i)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record(stream)
+    for i in range(args.steps):
+        step(i)
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_us = ev0.elapsed_time(ev1) * 1e3 / args.steps
+
+    flop = 2.0 * ROWS * INTER * HIDDEN                              # 103.08 GFLOP
+    alg_bytes = 2.0 * (ROWS * HIDDEN + E * INTER * HIDDEN + ROWS * INTER)   # 587.2 MB: x + w + y, once each
+    ms_per_step = wall * 1e3 / args.steps
+    tflops = flop * args.steps / wall / 1e12
+    achieved_gbs = alg_bytes / (kernel_us * 1e-6) / 1e9
+
+    out = {
+        "metric": "bf16 grouped-GEMM TFLOP/s fwd/dX/dW at 30B-A3B MoE shapes + % MFMA peak",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: Qwen3-30B-A3B gate_proj forward grouped GEMM", "experts": E,
+                   "rows": ROWS, "in_features": HIDDEN, "out_features": INTER, "tokens": TOKENS, "top_k": TOPK,
+                   "routing": "softmax top-8 of N(0,1) logits, rows sorted by expert"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved_gbs / PEAK_HBM_GBS, 4), "traffic": None,
+                     "kernel_us": round(kernel_us, 2), "algorithmic_bytes": alg_bytes,
+                     "mfma_tflops": round(flop / kernel_us / 1e6, 1),
+                     "mfma_frac": round(flop / kernel_us / 1e6 / PEAK_BF16_TFLOPS, 4)},
+    }
+
+    if not args.no_extra:
+        extra = {}
+        dys = [torch.randn((ROWS, HIDDEN), device=dev, dtype=torch.bfloat16) for _ in range(NB)]   # grad of down_proj out
+        hs = [torch.randn((ROWS, INTER), device=dev, dtype=torch.bfloat16) for _ in range(NB)]     # down_proj input
+        wd = [w.view(E, HIDDEN, INTER) for w in ws]                                                # (128, 2048, 768)
+        it, wm = 50, 5
+        us = _event_us(lambda i: grouped_gemm_forward_transposed(dys[i % NB], wd[i % NB], m_sizes), it, wm, stream)
+        extra["dx_down_proj"] = {"us": round(us, 1), "tflops": round(flop / us / 1e6, 1),
+                                 "mfma_frac": round(flop / us / 1e6 / PEAK_BF16_TFLOPS, 4),
+                                 "hbm_frac": round(alg_bytes / us / 1e3 / PEAK_HBM_GBS, 4)}
+        dws = [torch.empty((E, HIDDEN, INTER), device=dev, dtype=torch.bfloat16) for _ in range(NB)]
+        us = _event_us(lambda i: grouped_gemm_backward_dw(hs[i % NB], dys[i % NB], m_sizes, torch.bfloat16,
+                                                          out=dws[i % NB]), it, wm, stream)
+        extra["dw_down_proj"] = {"us": round(us, 1), "tflops": round(flop / us / 1e6, 1),
+                                 "mfma_frac": round(flop / us / 1e6 / PEAK_BF16_TFLOPS, 4),
+                                 "hbm_frac": round(alg_bytes / us / 1e3 / PEAK_HBM_GBS, 4)}
+        del dws
+        us = _event_us(lambda i: silu_mul_forward(hs[i % NB], hs[(i + 1) % NB]), it, wm, stream)
+        b = 3.0 * ROWS * INTER * 2
+        extra["silu_mul_fwd"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / PEAK_HBM_GBS, 4)}
+        selv = sel.view(-1)
+        us = _event_us(lambda i: get_expert_counts_and_idx(selv, E), it, wm, stream)
+        b = ROWS * 8 + 2 * ROWS * 4 + E * 4
+        extra["expert_sort_32768"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 2)}
+        lg = logits.to(dev)
+        us = _event_us(lambda i: softmax_topk_raw(lg, TOPK, True, torch.bfloat16), it, wm, stream)
+        b = TOKENS * E * 4 + TOKENS * TOPK * (4 + 2 + 8)
+        extra["softmax_topk_4096"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 2)}
+        # NF4: fused dequant+GEMM vs dequant-then-GEMM at 16 / 256 / 16384 tokens (config 5 gate_proj)
+        packed, qstate = quantize_nf4(ws[0], 64)
+        nf4 = {}
+        for tokens in (16, 256, 16384):
+            lgt = torch.randn((tokens, E), device=dev)
+            _, _, s5 = softmax_topk_raw(lgt, TOPK, True, torch.bfloat16)
+            ms5, _, _ = get_expert_counts_and_idx(s5.view(-1), E)
+            x5 = torch.randn((tokens * TOPK, HIDDEN), device=dev, dtype=torch.bfloat16)
+            n_it = 20 if tokens > 1000 else 50
+            us_f = _event_us(lambda i: grouped_gemm_forward_4bit(x5, packed, qstate, ms5), n_it, 3, stream)
+            us_u = _event_us(lambda i: grouped_gemm_forward(x5, dequantize_nf4(packed, qstate, torch.bfloat16), ms5),
+                             n_it, 3, stream)
+            active = int((ms5 > 0).sum().item())                       # host read outside any timed loop
+            packed_bytes = active * INTER * HIDDEN * (0.5 + 4.0 / 64)
+            nf4[f"tokens_{tokens}"] = {"fused_us": round(us_f, 1), "dequant_then_gemm_us": round(us_u, 1),
+                                       "active_experts": active,
+                                       "fused_packed_gbs": round(packed_bytes / us_f / 1e3, 1),
+                                       "fused_tflops": round(2.0 * tokens * TOPK * INTER * HIDDEN / us_f / 1e6, 1)}
+        extra["nf4_gate_proj"] = nf4
+        out["extra"] = extra
+
+    if not args.no_cpu_baseline:
+        import oracle
+
+        xs_np = x0.float().numpy()
+        w_np = w0.float().numpy()
+        sel_sorted = oracle.sel_from_m_sizes(m_sizes.cpu().numpy())
+        rows_done, t_cpu, chunk = 0, 0.0, 1024
+        while t_cpu < 10.0 and rows_done + chunk <= ROWS:
+            sl = slice(rows_done, rows_done + chunk)
+            t1 = time.perf_counter()
+            y_ref = oracle.linear_fwd(xs_np[sl], w_np, sel_sorted[sl])
+            t_cpu += time.perf_counter() - t1
+            rows_done += chunk
+        # the sample doubles as a parity check of the benchmarked output
+        got = ys[0][:chunk].float().cpu().numpy() if rows_done == chunk else None
+        out["cpu_baseline"] = {"value": round(2.0 * rows_done * INTER * HIDDEN / t_cpu / 1e12, 5), "unit": "TFLOP/s",
+                               "cores": oracle.num_threads(), "kind": "port",
+                               "sample": f"first {rows_done} of {ROWS} rows of the same batch, oracle/moe_oracle.c "
+                                         f"orc_linear_fwd_f32 (OpenMP over rows), {t_cpu:.1f} s",
+                               "host_cpus": os.cpu_count()}
+        del got, y_ref
+
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
