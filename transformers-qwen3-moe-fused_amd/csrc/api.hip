@@ -20,6 +20,7 @@ const DeviceInfo &device_info() {
 }
 
 extern int g_mfma_config;
+extern int g_pipe_config;
 
 namespace {
 
@@ -45,6 +46,8 @@ int run_gemm(int mode, const void *a, const void *b, const void *m_sizes, int ms
     hipStream_t s = (hipStream_t)stream;
     const int ms_i64 = ms_dtype == MFL_I64;
     if (in_dtype == MFL_BF16) {
+        rc = gemm_bf16_pipe(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, s);
+        if (rc != MFL_ERR_UNSUPPORTED) return rc;
         rc = gemm_bf16_mfma(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, s);
         if (rc != MFL_ERR_UNSUPPORTED) return rc;
     }
@@ -83,7 +86,19 @@ const char *mfl_strerror(int code) {
 
 /* Tuning hook (not part of the stable ABI): selects a tile configuration of the bf16 MFMA
  * kernels; 0 restores the built-in table. */
-void mfl_debug_set_mfma_config(int cfg) { g_mfma_config = cfg; }
+void mfl_debug_set_mfma_config(int cfg) {
+    // 0..99: configuration of the register-staged kernels (pipelined kernels off);
+    // 100 + n: configuration n of the pipelined kernels; negative: built-in table.
+    if (cfg >= 100) {
+        g_pipe_config = cfg - 100;
+    } else if (cfg >= 0) {
+        g_pipe_config = -1;
+        g_mfma_config = cfg;
+    } else {
+        g_pipe_config = 0;
+        g_mfma_config = 0;
+    }
+}
 
 int mfl_gemm_fwd(const void *x, const void *w, const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K,
                  int E, int in_dtype, int out_dtype, float alpha, int accumulate, void *stream) {
