@@ -1,5 +1,5 @@
 // Pipelined bf16 grouped GEMM for CDNA4: global -> LDS copies that bypass the register file
-// (global_load_lds_dwordx4), a ring of S LDS stages so several K steps are in flight per
+// (global_load_lds_dwordx4), a ring of S LDS stages so several reduction steps are in flight per
 // compute unit, XOR-swizzled stage layouts (no padding: the copy engine writes 1 KiB of
 // consecutive LDS per wave instruction), v_mfma_f32_32x32x16_bf16, persistent workgroups.
 //
@@ -13,10 +13,21 @@
 //   RS stage: row r holds BI elements; chunk c of row r is stored at c ^ ((r & 3) << 1): the
 //             four rows a transposing read (ds_read_b64_tr_b16) touches fall in different banks.
 //
+// Tiles.  A tile is MB x NB blocks of 32 x 32.  The WGM x WGN waves of a workgroup split the
+// columns in contiguous runs and take the 32-row blocks round robin (wave row w owns blocks
+// w, w + WGM, ...).  In the row-grouped products (FWD, DX) a tile covers up to 32*MB rows of ONE
+// expert; MB is chosen so that a typical expert fits in one tile: its weights are then streamed
+// by exactly one workgroup per column slice, and a few rows more or less change the number of
+// active blocks, not the number of tiles.  Experts with more rows are cut into equal parts.
+// The reduction loop is instantiated once per number of active row blocks of a wave, so blocks
+// past the last row cost no MFMA and there is no branch inside the loop.
+//
 // Shapes this kernel takes (the caller falls back to gemm_bf16_mfma.hip otherwise):
 //   FWD, DX: K % BK == 0, N % 8 == 0.   DW: N % 8 == 0, K % 8 == 0.
 // Rows or columns past a tile's valid range are loaded from a clamped (valid) address and never
 // stored; in DW the rows of the last, partial reduction step are zeroed in LDS before use.
+#include <type_traits>
+
 #include "common.h"
 #include "gemm.h"
 
@@ -40,13 +51,16 @@ __device__ __forceinline__ void wait_vmcnt() {
 template <int BI, int BK, bool RC>
 struct Stage {
     static constexpr int kRowBytes = RC ? BK * 2 : BI * 2;
-    static constexpr int kRows = RC ? BI : BK;
     static constexpr int kBytes = BI * BK * 2;
     static constexpr int kWaveLoads = kBytes / 1024;       // 1 KiB per wave-wide copy
-    static constexpr int kRowsPerLoad = 1024 / kRowBytes;  // rows covered by one copy
     static constexpr int kChunksPerRow = kRowBytes / 16;
     static constexpr int kRowsPer256 = kRowBytes >= 256 ? 1 : 256 / kRowBytes;
-    static_assert(kRowBytes <= 1024 && 1024 % kRowBytes == 0, "row must divide a 1 KiB copy");
+    static_assert(kBytes % 1024 == 0 && kChunksPerRow % 8 == 0, "stage must be whole copies, rows whole 128 B");
+
+    // stage row and physical chunk that lane `lane` of wave-load `load` fills (a copy covers 64
+    // consecutive chunks of the stage, whatever the row length)
+    __device__ static __forceinline__ int row_of(int load, int lane) { return (load * 64 + lane) / kChunksPerRow; }
+    __device__ static __forceinline__ int phys_of(int load, int lane) { return (load * 64 + lane) % kChunksPerRow; }
 
     // physical 16-byte chunk of logical chunk c in row `row`
     __device__ static __forceinline__ int swz(int row, int c) {
@@ -61,8 +75,8 @@ struct Stage {
 template <int BI, int BK, bool RC>
 __device__ __forceinline__ int64_t lane_src_offset(int load, int lane, int64_t ld, int i_lim) {
     typedef Stage<BI, BK, RC> S;
-    const int row = load * S::kRowsPerLoad + lane / S::kChunksPerRow;  // stage row
-    const int phys = lane % S::kChunksPerRow;
+    const int row = S::row_of(load, lane);
+    const int phys = S::phys_of(load, lane);
     const int c = S::swz(row, phys);  // XOR swizzle is its own inverse
     if (RC) {
         int i = row;
@@ -75,17 +89,74 @@ __device__ __forceinline__ int64_t lane_src_offset(int load, int lane, int64_t l
     }
 }
 
-struct RowTile {
-    int expert, i0, i_end, jt;
+// Per-lane LDS byte offsets (within an operand's part of a stage) of the MFMA fragment reads of
+// the wave's blocks: block t of the wave starts at row first + t * stride.
+// RC: one offset per 16-wide reduction sub-step (the block adds a constant).
+// RS: one offset per block (the sub-step adds a constant).
+template <int BI, int BK, bool RC, int TB>
+struct FragOffsets {
+    static constexpr int kCount = RC ? BK / 16 : TB;
+    int off[kCount];
+    int block_bytes;  // RC only: byte distance between consecutive blocks of the wave
+
+    __device__ __forceinline__ void init(int first, int stride, int lane) {
+        typedef Stage<BI, BK, RC> S;
+        block_bytes = stride * S::kRowBytes;
+        if (RC) {
+            const int row = first + (lane & 31);
+#pragma unroll
+            for (int ks = 0; ks < kCount; ++ks)
+                off[ks] = row * S::kRowBytes + S::swz(row, ks * 2 + (lane >> 5)) * 16;
+        } else {
+            const int g = lane >> 4, il = lane & 15;
+            const int r = 8 * (g >> 1) + (il >> 2);
+#pragma unroll
+            for (int t = 0; t < kCount; ++t) {
+                const int i = first + t * stride + 16 * (g & 1) + 4 * (il & 3);
+                off[t] = r * S::kRowBytes + S::swz(r, i >> 3) * 16 + (i & 7) * 2;
+            }
+        }
+    }
+
+    // fragment of the wave's block t at sub-step ks; `base` points at the operand's part of the stage
+    __device__ __forceinline__ bf16x8 load(const unsigned char *base, int t, int ks) const {
+        typedef Stage<BI, BK, RC> S;
+        if (RC) {
+            return *(const bf16x8 *)(base + off[ks] + t * block_bytes);
+        } else {
+            const unsigned char *p = base + off[t] + ks * 16 * S::kRowBytes;
+            const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)p);
+            const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(p + 4 * S::kRowBytes));
+            union {
+                short4_t h[2];
+                bf16x8 v;
+            } u;
+            u.h[0] = lo;
+            u.h[1] = hi;
+            return u.v;
+        }
+    }
 };
 
-// Number of tiles of the row-grouped modes: sum over experts of ceil(m_e / BM) * n_tiles_n.
+// ---- tile enumeration of the row-grouped products -------------------------------------------
+
+// An expert with m rows is cut into ceil(m / BM) parts of equal height (a multiple of 32).
+template <int BM>
+__device__ __forceinline__ int m_tiles_of(int m) {
+    return ceil_div(m, BM);
+}
+template <int BM>
+__device__ __forceinline__ int tile_rows_of(int m) {
+    const int t = ceil_div(m, BM);
+    return t == 0 ? 0 : ceil_div(ceil_div(m, t), 32) * 32;
+}
+
 template <int BM>
 __device__ __forceinline__ int count_row_tiles(const void *m_sizes, int ms_i64, int E, int n_tiles_n, int lane) {
     int total = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
         const int e = e0 + lane;
-        int t = e < E ? ceil_div(load_msize(m_sizes, ms_i64, e), BM) * n_tiles_n : 0;
+        int t = e < E ? m_tiles_of<BM>(load_msize(m_sizes, ms_i64, e)) * n_tiles_n : 0;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off);
         total += t;
@@ -93,10 +164,13 @@ __device__ __forceinline__ int count_row_tiles(const void *m_sizes, int ms_i64, 
     return total;
 }
 
+struct RowTile {
+    int expert, i0, i_end, jt;
+};
+
 // (expert, first row, row bound, n-tile) of logical tile L < total.  Within an expert the
-// m-tiles of one n-tile are consecutive: workgroups that share a slice of the weight matrix
-// run side by side, and a boundary between scheduling rounds costs a re-read of the expert's
-// rows (small) rather than of its weights (large).
+// m-tiles of one n-tile are consecutive, so workgroups that share a slice of the weight matrix
+// run side by side.
 template <int BM>
 __device__ __forceinline__ RowTile locate_row_tile(const void *m_sizes, int ms_i64, int E, int n_tiles_n, int64_t R,
                                                    int L, int lane) {
@@ -105,7 +179,7 @@ __device__ __forceinline__ RowTile locate_row_tile(const void *m_sizes, int ms_i
     for (int e0 = 0; e0 < E; e0 += 64) {
         const int e = e0 + lane;
         const int m = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
-        const int t = ceil_div(m, BM) * n_tiles_n;
+        const int t = m_tiles_of<BM>(m) * n_tiles_n;
         int tinc = t, minc = m;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
@@ -122,10 +196,12 @@ __device__ __forceinline__ RowTile locate_row_tile(const void *m_sizes, int ms_i
             const int local = L - __shfl(tbeg, src);
             const int m_start = row_carry + __shfl(minc - m, src);
             const int m_size = __shfl(m, src);
-            const int m_tiles = ceil_div(m_size, BM);
+            const int m_tiles = m_tiles_of<BM>(m_size);
+            const int rows = tile_rows_of<BM>(m_size);
             rt.expert = e0 + src;
-            rt.i0 = m_start + (local % m_tiles) * BM;
+            rt.i0 = m_start + (local % m_tiles) * rows;
             rt.i_end = m_start + m_size;
+            if (rt.i_end > rt.i0 + rows) rt.i_end = rt.i0 + rows;
             if ((int64_t)rt.i_end > R) rt.i_end = (int)R;
             rt.jt = local / m_tiles;
             return rt;
@@ -136,93 +212,23 @@ __device__ __forceinline__ RowTile locate_row_tile(const void *m_sizes, int ms_i
     return rt;
 }
 
-// Per-lane LDS byte offsets (within an operand's part of a stage) of the MFMA fragment reads.
-// RC: one offset per 16-wide reduction sub-step (the row block adds a constant).
-// RS: one offset per 32-row block of the tile (the sub-step adds a constant).
-template <int BI, int BK, bool RC, int TB>
-struct FragOffsets {
-    static constexpr int kCount = RC ? BK / 16 : TB;
-    int off[kCount];
+template <int V>
+using IC = std::integral_constant<int, V>;
 
-    __device__ __forceinline__ void init(int wave_row0, int lane) {
-        typedef Stage<BI, BK, RC> S;
-        if (RC) {
-            const int row = wave_row0 + (lane & 31);
-#pragma unroll
-            for (int ks = 0; ks < kCount; ++ks)
-                off[ks] = row * S::kRowBytes + S::swz(row, ks * 2 + (lane >> 5)) * 16;
-        } else {
-            const int g = lane >> 4, il = lane & 15;
-            const int r = 8 * (g >> 1) + (il >> 2);
-#pragma unroll
-            for (int bi = 0; bi < kCount; ++bi) {
-                const int i = wave_row0 + bi * 32 + 16 * (g & 1) + 4 * (il & 3);
-                off[bi] = r * S::kRowBytes + S::swz(r, i >> 3) * 16 + (i & 7) * 2;
-            }
-        }
-    }
-
-    // fragment of row block bi at sub-step ks; `base` points at the operand's part of the stage
-    __device__ __forceinline__ bf16x8 load(const unsigned char *base, int bi, int ks) const {
-        typedef Stage<BI, BK, RC> S;
-        if (RC) {
-            return *(const bf16x8 *)(base + off[ks] + bi * 32 * S::kRowBytes);
-        } else {
-            const unsigned char *p = base + off[bi] + ks * 16 * S::kRowBytes;
-            const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)p);
-            const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(p + 4 * S::kRowBytes));
-            union {
-                short4_t h[2];
-                bf16x8 v;
-            } u;
-            u.h[0] = lo;
-            u.h[1] = hi;
-            return u.v;
-        }
-    }
-};
-
-// One more wave than the WGM x WGN that multiply runs ahead of them when PF > 0: it touches
-// one dword of every 128-byte line of reduction step kt + S - 1 + PF (a 4-byte copy per lane into
-// a scratch corner of LDS) so that the copies proper find their data in L2.  Tiles share
-// operands (rows of an expert are read by every n-tile, weights by every m-tile), so only a
-// fraction of the bytes the stages hold in flight is new to L2; with its own memory counter the
-// extra wave keeps many more first-touch misses in flight than the stage ring can.
-template <int BI, int BK, bool RC>
-__device__ __forceinline__ void touch_lines(const unsigned char *tile, int ld, int lim, int kt, int red, int lane,
-                                            unsigned char *scratch) {
-    constexpr int LINES = BI * BK * 2 / 128;
-#pragma unroll
-    for (int j = 0; j < LINES / 64; ++j) {
-        const int idx = j * 64 + lane;
-        const unsigned char *p;
-        if (RC) {
-            int row = idx / (BK * 2 / 128), seg = idx % (BK * 2 / 128);
-            if (row >= lim) row = lim - 1;
-            p = tile + ((int64_t)row * ld + kt * BK) * 2 + seg * 128;
-        } else {
-            constexpr int SEGS = BI * 2 / 128 > 0 ? BI * 2 / 128 : 1;
-            int r = kt * BK + idx / SEGS, seg = idx % SEGS;
-            if (r >= red) r = red - 1;
-            int col = seg * 64;
-            if (col >= lim) col = lim - 8;
-            p = tile + ((int64_t)r * ld + col) * 2;
-        }
-        __builtin_amdgcn_global_load_lds((global_void_ptr)p, (lds_void_ptr)scratch, 4, 0, 0);
-    }
-}
-
-template <int BM, int BN, int BK, int S, int WGM, int WGN, int PF, int MODE, typename TO>
-__global__ __launch_bounds__((WGM * WGN + (PF > 0 ? 1 : 0)) * 64) void gemm_pipe_kernel(const bf16_t *__restrict__ a,
+template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODE, typename TO>
+__global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *__restrict__ a,
                                                                   const bf16_t *__restrict__ b,
                                                                   const void *__restrict__ m_sizes, int ms_i64,
                                                                   TO *__restrict__ c, int64_t R, int N, int K, int E,
                                                                   float alpha, int accumulate) {
+    constexpr int BM = MB * 32, BN = NB * 32;
     constexpr int NW = WGM * WGN;
     constexpr bool A_RC = MODE != MODE_DW;
     constexpr bool B_RC = MODE == MODE_FWD;
-    constexpr int WTM = BM / WGM, WTN = BN / WGN;
-    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int TM = (MB + WGM - 1) / WGM;  // row blocks per wave (the last may not exist)
+    static_assert(NB % WGN == 0, "column blocks must split evenly over the waves");
+    constexpr int TN = NB / WGN;
+    constexpr int WTN = TN * 32;
     constexpr int KS = BK / 16;
     typedef Stage<BM, BK, A_RC> SA;
     typedef Stage<BN, BK, B_RC> SB;
@@ -240,8 +246,8 @@ __global__ __launch_bounds__((WGM * WGN + (PF > 0 ? 1 : 0)) * 64) void gemm_pipe
 
     FragOffsets<BM, BK, A_RC, TM> fo_a;
     FragOffsets<BN, BK, B_RC, TN> fo_b;
-    fo_a.init(wm * WTM, lane);
-    fo_b.init(wn * WTN, lane);
+    fo_a.init(wm * 32, WGM * 32, lane);
+    fo_b.init(wn * WTN, 32, lane);
 
     // ---- tile range of this workgroup: XCD x owns logical tiles [x*chunk, (x+1)*chunk)
     int total, tiles_n = 0, per_expert = 0;
@@ -310,29 +316,6 @@ __global__ __launch_bounds__((WGM * WGN + (PF > 0 ? 1 : 0)) * 64) void gemm_pipe
         const int i_lim = i_end - i0 < BM ? i_end - i0 : BM;  // valid rows (or columns) of A from the tile origin
         const int j_lim = j_end - j0 < BN ? j_end - j0 : BN;
 
-        if (PF > 0 && wave == NW) {
-            // ---- the wave that runs ahead: same barrier sequence as the others, no arithmetic
-            unsigned char *scratch = smem + S * STAGE_BYTES;
-            auto touch = [&](int step) {
-                if (step < KT) {
-                    touch_lines<BM, BK, A_RC>(a_tile, lda, i_lim, step, red, lane, scratch);
-#ifndef MFL_EXP_PF_A_ONLY
-                    touch_lines<BN, BK, B_RC>(b_tile, ldb, j_lim, step, red, lane, scratch);
-#endif
-                    wait_vmcnt<40>();
-                }
-            };
-            __builtin_amdgcn_s_barrier();
-            for (int step = S - 1; step < S - 1 + PF; ++step) touch(step);
-            for (int kt = 0; kt < KT; ++kt) {
-                __builtin_amdgcn_s_barrier();
-                touch(kt + S - 1 + PF);
-                if (MODE == MODE_DW && (kt + 1) * BK > red) __builtin_amdgcn_s_barrier();
-            }
-            if (sizeof(TO) == 2 && !accumulate) __builtin_amdgcn_s_barrier();
-            continue;
-        }
-
         // per-lane 32-bit source offsets of this wave's copies (tile origin, reduction step 0);
         // the step advances a wave-uniform base pointer
         uint32_t lane_off[LPW];
@@ -346,17 +329,9 @@ __global__ __launch_bounds__((WGM * WGN + (PF > 0 ? 1 : 0)) * 64) void gemm_pipe
         const int64_t step_b = B_RC ? (int64_t)BK * 2 : (int64_t)BK * ldb * 2;
 
         auto issue = [&](int kt) {
-#ifdef MFL_EXP_NOLOAD
-            return;
-#endif
             unsigned char *st = smem + (kt % S) * STAGE_BYTES;
-#ifdef MFL_EXP_ROT
-            const int kk = MODE == MODE_DW ? kt : (kt + (L * MFL_EXP_ROT) % KT) % KT;
-#else
-            const int kk = kt;
-#endif
-            const unsigned char *pa = a_tile + kk * step_a;
-            const unsigned char *pb = b_tile + kk * step_b;
+            const unsigned char *pa = a_tile + kt * step_a;
+            const unsigned char *pb = b_tile + kt * step_b;
             // In DW the last step may be partial: lanes whose row lies past the end re-read the
             // last valid row; those rows are zeroed in LDS before use.
             const bool tail = MODE == MODE_DW && (kt + 1) * BK > red;
@@ -364,7 +339,7 @@ __global__ __launch_bounds__((WGM * WGN + (PF > 0 ? 1 : 0)) * 64) void gemm_pipe
             for (int q = 0; q < LA; ++q) {
                 uint32_t o = lane_off[q];
                 if (!A_RC && tail) {
-                    const int row = (wave * LA + q) * SA::kRowsPerLoad + lane / SA::kChunksPerRow + kt * BK;
+                    const int row = SA::row_of(wave * LA + q, lane) + kt * BK;
                     if (row >= red) o -= (uint32_t)(row - (red - 1)) * (uint32_t)lda * 2u;
                 }
                 __builtin_amdgcn_global_load_lds((global_void_ptr)(pa + o), (lds_void_ptr)(st + (wave * LA + q) * 1024),
@@ -374,7 +349,7 @@ __global__ __launch_bounds__((WGM * WGN + (PF > 0 ? 1 : 0)) * 64) void gemm_pipe
             for (int q = 0; q < LB; ++q) {
                 uint32_t o = lane_off[LA + q];
                 if (!B_RC && tail) {
-                    const int row = (wave * LB + q) * SB::kRowsPerLoad + lane / SB::kChunksPerRow + kt * BK;
+                    const int row = SB::row_of(wave * LB + q, lane) + kt * BK;
                     if (row >= red) o -= (uint32_t)(row - (red - 1)) * (uint32_t)ldb * 2u;
                 }
                 __builtin_amdgcn_global_load_lds((global_void_ptr)(pb + o),
@@ -384,14 +359,17 @@ __global__ __launch_bounds__((WGM * WGN + (PF > 0 ? 1 : 0)) * 64) void gemm_pipe
 
         floatx16 acc[TM][TN];
 #pragma unroll
-        for (int bi = 0; bi < TM; ++bi)
+        for (int t = 0; t < TM; ++t)
 #pragma unroll
             for (int bj = 0; bj < TN; ++bj)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[bi][bj][r] = 0.f;
-        bool blk_on[TM];
-#pragma unroll
-        for (int bi = 0; bi < TM; ++bi) blk_on[bi] = (wm * WTM + bi * 32) < i_lim;
+                for (int r = 0; r < 16; ++r) acc[t][bj][r] = 0.f;
+
+        // row blocks of this wave that hold at least one valid row: blocks wm, wm+WGM, ... below
+        // ceil(i_lim / 32)
+        const int n_blocks = ceil_div(i_lim, 32);
+        int active = n_blocks > wm ? ceil_div(n_blocks - wm, WGM) : 0;
+        if (active > TM) active = TM;
 
         // every store of the previous tile has left, every wave is done with the stages
         wait_vmcnt<0>();
@@ -402,114 +380,114 @@ __global__ __launch_bounds__((WGM * WGN + (PF > 0 ? 1 : 0)) * 64) void gemm_pipe
         for (int s = 0; s < S - 1; ++s)
             if (s < KT) issue(s);
 
-        for (int kt = 0; kt < KT; ++kt) {
-            // step kt has landed for this wave's copies; the barrier extends that to all waves
-            // and tells us everybody finished reading step kt-1, whose stage is refilled next
-            if (kt + S - 2 < KT)
-                wait_vmcnt<(S - 2) * LPW>();
-            else
-                wait_vmcnt<0>();
-#ifndef MFL_EXP_NOBARRIER
-            __builtin_amdgcn_s_barrier();
-#endif
-            if (kt + S - 1 < KT) issue(kt + S - 1);
-
-            unsigned char *st = smem + (kt % S) * STAGE_BYTES;
-            if (MODE == MODE_DW && (kt + 1) * BK > red) {
-                // zero the rows of A past the end of the expert (B's are multiplied by them)
-                const int first = red - kt * BK;
-                for (int q = tid; q < (BK - first) * SA::kChunksPerRow; q += NW * 64)
-                    *(uint4_t *)(st + first * SA::kRowBytes + q * 16) = uint4_t{0u, 0u, 0u, 0u};
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        // ---- reduction loop, instantiated per number of row blocks that are multiplied
+        auto k_loop = [&](auto ta_tag) {
+            constexpr int TA = decltype(ta_tag)::value;
+            for (int kt = 0; kt < KT; ++kt) {
+                // step kt has landed for this wave's copies; the barrier extends that to all
+                // waves and tells us everybody finished reading step kt-1, whose stage is
+                // refilled next
+                if (kt + S - 2 < KT)
+                    wait_vmcnt<(S - 2) * LPW>();
+                else
+                    wait_vmcnt<0>();
                 __builtin_amdgcn_s_barrier();
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-            }
-            const unsigned char *sa = st, *sb = st + SA::kBytes;
-#ifndef MFL_EXP_NOLDS
-            {
-                // Every wave multiplies, also one whose rows all lie past the tile edge: a branch
-                // here makes the compiler shuttle the accumulators between register files.
-                // Fragments of sub-step ks+1 are fetched while sub-step ks is multiplied.
-                bf16x8 fa[2][TM], fb[2][TN];
+                if (kt + S - 1 < KT) issue(kt + S - 1);
+
+                unsigned char *st = smem + (kt % S) * STAGE_BYTES;
+                if (MODE == MODE_DW && (kt + 1) * BK > red) {
+                    // zero the rows of A past the end of the expert (B's are multiplied by them)
+                    const int first = red - kt * BK;
+                    for (int q = tid; q < (BK - first) * SA::kChunksPerRow; q += NW * 64)
+                        *(uint4_t *)(st + first * SA::kRowBytes + q * 16) = uint4_t{0u, 0u, 0u, 0u};
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                    __builtin_amdgcn_s_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                }
+                const unsigned char *sa = st, *sb = st + SA::kBytes;
+                // fragments of sub-step ks+1 are fetched while sub-step ks is multiplied
+                bf16x8 fa[2][TA], fb[2][TN];
 #pragma unroll
                 for (int bj = 0; bj < TN; ++bj) fb[0][bj] = fo_b.load(sb, bj, 0);
 #pragma unroll
-                for (int bi = 0; bi < TM; ++bi) fa[0][bi] = fo_a.load(sa, bi, 0);
+                for (int t = 0; t < TA; ++t) fa[0][t] = fo_a.load(sa, t, 0);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     if (ks + 1 < KS) {
 #pragma unroll
                         for (int bj = 0; bj < TN; ++bj) fb[(ks + 1) & 1][bj] = fo_b.load(sb, bj, ks + 1);
 #pragma unroll
-                        for (int bi = 0; bi < TM; ++bi) fa[(ks + 1) & 1][bi] = fo_a.load(sa, bi, ks + 1);
+                        for (int t = 0; t < TA; ++t) fa[(ks + 1) & 1][t] = fo_a.load(sa, t, ks + 1);
                     }
 #pragma unroll
-                    for (int bi = 0; bi < TM; ++bi)
+                    for (int t = 0; t < TA; ++t)
 #pragma unroll
                         for (int bj = 0; bj < TN; ++bj)
-#ifdef MFL_EXP_NOMFMA
-                            acc[bi][bj][0] += (float)fa[ks & 1][bi][0] + (float)fb[ks & 1][bj][0];
-#else
-                            acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][bi], fb[ks & 1][bj],
-                                                                                  acc[bi][bj], 0, 0, 0);
-#endif
+                            acc[t][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][t], fb[ks & 1][bj],
+                                                                                 acc[t][bj], 0, 0, 0);
                 }
             }
-#endif
-        }
+        };
+        // a wave without valid rows still copies, and multiplies one block nobody stores
+        if (TM == 1 || active <= 1)
+            k_loop(IC<1>{});
+        else if (TM == 2 || active == 2)
+            k_loop(IC<(TM >= 2 ? 2 : 1)>{});
+        else if (TM == 3 || active == 3)
+            k_loop(IC<(TM >= 3 ? 3 : 1)>{});
+        else
+            k_loop(IC<TM>{});
 
         // ---- epilogue
         if (sizeof(TO) == 2 && !accumulate) {
-            // Stage the wave's tile in LDS as bf16, then write full rows: 8 lanes x 16 bytes per
-            // row instead of 2-byte stores scattered over 32 rows.
+            // One 32-row block of the wave at a time: stage it in LDS as bf16, then write full
+            // rows, 16 bytes per lane, instead of 2-byte stores scattered over 32 rows.
             __builtin_amdgcn_s_barrier();  // all waves are done reading the last stage
             constexpr int ROWB = WTN * 2 + 16;  // padded row, bytes
-            unsigned char *ep = smem + wave * (WTM * ROWB);
+            constexpr int CPR = WTN / 8;        // 16-byte chunks per row
+            unsigned char *ep = smem + wave * (32 * ROWB);
 #pragma unroll
-            for (int bi = 0; bi < TM; ++bi) {
-                if (!blk_on[bi]) continue;
+            for (int t = 0; t < TM; ++t) {
+                if (t >= active) continue;
 #pragma unroll
                 for (int bj = 0; bj < TN; ++bj)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const int row = bi * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                        const int row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                         const int col = bj * 32 + (lane & 31);
-                        *(bf16_t *)(ep + row * ROWB + col * 2) = (bf16_t)(acc[bi][bj][r] * alpha);
+                        *(bf16_t *)(ep + row * ROWB + col * 2) = (bf16_t)(acc[t][bj][r] * alpha);
                     }
-            }
-            // same wave reads back what it wrote: LDS ops of one wave complete in order
-            constexpr int LPR = WTN / 8;        // lanes per row
-            constexpr int RPI = 64 / LPR;       // rows per wave instruction
-            const int lrow = lane / LPR, lcol = (lane % LPR) * 8;
-#pragma unroll
-            for (int r0 = 0; r0 < WTM; r0 += RPI) {
-                const int row_l = r0 + lrow;
-                const int row = i0 + wm * WTM + row_l;
-                const int col = j0 + wn * WTN + lcol;
-                if (!blk_on[r0 / 32] || row >= i_end || col >= j_end) continue;
-                const uint4_t v = *(const uint4_t *)(ep + row_l * ROWB + lcol * 2);
-                bf16_t *dst = (bf16_t *)c_base + (int64_t)row * ldc + col;
-                if (col + 8 <= j_end) {
-                    *(uint4_t *)dst = v;
-                } else {
-                    const bf16_t *pv = (const bf16_t *)&v;
-                    for (int u = 0; u < j_end - col; ++u) dst[u] = pv[u];
+                // the same wave reads back what it wrote: LDS operations of one wave complete in order
+                const int row_base = i0 + (wm + WGM * t) * 32;
+                for (int q = lane; q < 32 * CPR; q += 64) {
+                    const int row_l = q / CPR, lcol = (q % CPR) * 8;
+                    const int row = row_base + row_l;
+                    const int col = j0 + wn * WTN + lcol;
+                    if (row >= i_end || col >= j_end) continue;
+                    const uint4_t v = *(const uint4_t *)(ep + row_l * ROWB + lcol * 2);
+                    bf16_t *dst = (bf16_t *)c_base + (int64_t)row * ldc + col;
+                    if (col + 8 <= j_end) {
+                        *(uint4_t *)dst = v;
+                    } else {
+                        const bf16_t *pv = (const bf16_t *)&v;
+                        for (int u = 0; u < j_end - col; ++u) dst[u] = pv[u];
+                    }
                 }
             }
         } else {
 #pragma unroll
-            for (int bi = 0; bi < TM; ++bi) {
-                if (!blk_on[bi]) continue;
+            for (int t = 0; t < TM; ++t) {
+                if (t >= active) continue;
 #pragma unroll
                 for (int bj = 0; bj < TN; ++bj) {
                     const int col = j0 + wn * WTN + bj * 32 + (lane & 31);
                     if (col >= j_end) continue;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const int row = i0 + wm * WTM + bi * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                        const int row = i0 + (wm + WGM * t) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                         if (row >= i_end) continue;
                         TO *p = c_base + (int64_t)row * ldc + col;
-                        float v = alpha * acc[bi][bj][r];
+                        float v = alpha * acc[t][bj][r];
                         if (accumulate) v += to_f32(*p);
                         *p = from_f32<TO>(v);
                     }
@@ -519,20 +497,20 @@ __global__ __launch_bounds__((WGM * WGN + (PF > 0 ? 1 : 0)) * 64) void gemm_pipe
     }
 }
 
-template <int BM, int BN, int BK, int S, int WGM, int WGN, int PF, typename TO>
+template <int MB, int NB, int BK, int S, int WGM, int WGN, typename TO>
 int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
                 int K, int E, float alpha, int accumulate, hipStream_t stream) {
-    constexpr int NT = (WGM * WGN + (PF > 0 ? 1 : 0)) * 64;
-    constexpr int STAGE_BYTES = (BM + BN) * BK * 2;
-    constexpr int EP_BYTES = WGM * WGN * (BM / WGM) * ((BN / WGN) * 2 + 16);
-    constexpr int LDS_BYTES = (S * STAGE_BYTES > EP_BYTES ? S * STAGE_BYTES : EP_BYTES) + 1024;  // + scratch corner
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int STAGE_BYTES = (MB + NB) * 32 * BK * 2;
+    constexpr int EP_BYTES = WGM * WGN * 32 * ((NB / WGN) * 64 + 16);
+    constexpr int LDS_BYTES = S * STAGE_BYTES > EP_BYTES ? S * STAGE_BYTES : EP_BYTES;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS capacity of a CDNA4 compute unit");
     const bf16_t *pa = (const bf16_t *)a, *pb = (const bf16_t *)b;
     TO *pc = (TO *)c;
     const int grid = device_info().cu_count / kXcd * kXcd;  // one persistent workgroup per CU
 #define MFL_PIPE(MODE)                                                                                          \
     {                                                                                                           \
-        auto kern = gemm_pipe_kernel<BM, BN, BK, S, WGM, WGN, PF, MODE, TO>;                                        \
+        auto kern = gemm_pipe_kernel<MB, NB, BK, S, WGM, WGN, MODE, TO>;                                        \
         static bool attr_set = false;                                                                           \
         if (!attr_set) {                                                                                        \
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,  \
@@ -562,29 +540,30 @@ int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, 
     if (mode == MODE_DX && (K % 64 != 0 || N % 8 != 0 || N < 8)) return MFL_ERR_UNSUPPORTED;
     if (mode == MODE_DW && (N % 8 != 0 || K % 8 != 0 || N < 8 || K < 8)) return MFL_ERR_UNSUPPORTED;
     if (mode != MODE_DW && R <= 0) return MFL_OK;
-#define MFL_LAUNCH(BM, BN, BK, S, WGM, WGN, PF)                                                                  \
-    (out_dtype == MFL_BF16 ? launch_pipe<BM, BN, BK, S, WGM, WGN, PF, bf16_t>(mode, a, b, m_sizes, ms_i64, c, R, \
-                                                                              N, K, E, alpha, accumulate, stream) \
-                           : launch_pipe<BM, BN, BK, S, WGM, WGN, PF, float>(mode, a, b, m_sizes, ms_i64, c, R,  \
-                                                                             N, K, E, alpha, accumulate, stream))
-    // Tile table (BM, BN, BK, stages, waves along M, waves along N, run-ahead distance).  The
-    // default per product was picked from timings at the Qwen3-30B-A3B expert shapes.
+#define MFL_LAUNCH(MB, NB, BK, S, WGM, WGN)                                                                       \
+    (out_dtype == MFL_BF16 ? launch_pipe<MB, NB, BK, S, WGM, WGN, bf16_t>(mode, a, b, m_sizes, ms_i64, c, R, N, K, \
+                                                                          E, alpha, accumulate, stream)           \
+                           : launch_pipe<MB, NB, BK, S, WGM, WGN, float>(mode, a, b, m_sizes, ms_i64, c, R, N, K, \
+                                                                         E, alpha, accumulate, stream))
+    // Tile table (row blocks, column blocks, BK, stages, waves along M, waves along N).  The default
+    // per product was picked from timings at the Qwen3-30B-A3B expert shapes.
+    // Row-grouped products: 320 x 192 tiles, i.e. every expert of up to 320 rows is one tile per
+    // 192-column slice (4 slices of N = 768: 512 tiles, two per CU).  DW: square 256 x 256 tiles.
     int cfg = g_pipe_config;
-    if (cfg == 0) {
-        if (mode == MODE_DX) return MFL_ERR_UNSUPPORTED;  // the register-staged kernel is faster there
-        cfg = 8;
-    }
+    if (cfg == 0) cfg = mode == MODE_DW ? 8 : 3;
     switch (cfg) {
         case 1:
-            return MFL_LAUNCH(128, 128, 64, 4, 2, 2, 0);
+            return MFL_LAUNCH(4, 4, 64, 4, 2, 2);
         case 2:
-            return MFL_LAUNCH(256, 128, 64, 3, 4, 2, 0);
+            return MFL_LAUNCH(8, 4, 64, 3, 4, 2);
+        case 3:
+            return MFL_LAUNCH(10, 6, 64, 2, 4, 2);
         case 4:
-            return MFL_LAUNCH(256, 128, 64, 3, 4, 2, 4);
-        case 7:
-            return MFL_LAUNCH(256, 256, 32, 4, 2, 4, 0);
+            return MFL_LAUNCH(10, 4, 64, 2, 4, 2);
+        case 5:
+            return MFL_LAUNCH(10, 8, 64, 2, 2, 4);
         default:
-            return MFL_LAUNCH(256, 256, 64, 2, 2, 4, 0);
+            return MFL_LAUNCH(8, 8, 64, 2, 2, 4);
     }
 #undef MFL_LAUNCH
 }
