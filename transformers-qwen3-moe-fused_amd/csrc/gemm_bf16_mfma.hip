@@ -444,7 +444,9 @@ int dispatch_mfma(int mode, const void *a, const void *b, const void *m_sizes, i
 int gemm_bf16_mfma(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
                    int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream) {
     // 16-byte chunks along every contiguous dimension
-    if (N % 8 != 0 || K % 8 != 0 || N < 32 || K < 32) return MFL_ERR_UNSUPPORTED;
+    // thin LoRA shapes (N or K = rank) run here too: the tile edges are masked, and those
+    // products are bound by streaming the wide operand, not by the matrix cores
+    if (N % 8 != 0 || K % 8 != 0 || N < 8 || K < 8) return MFL_ERR_UNSUPPORTED;
     if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, 4)) return MFL_ERR_UNSUPPORTED;
     if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
     return dispatch_mfma(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, nullptr, stream);

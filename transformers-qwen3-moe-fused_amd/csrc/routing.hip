@@ -124,29 +124,72 @@ __device__ __forceinline__ int64_t load_key(const void *sel, int is_i64, int64_t
 // when `local_rank` is given, store each row's rank among the rows of the same key seen so
 // far by this wave.  Within a batch, lanes sharing a key are found with one ballot per key
 // bit; their order is the lane order, which keeps the sort stable.
+constexpr int kSortChunk = 16;  // batches of 64 keys whose loads are issued together
+
 __device__ __forceinline__ void wave_count(const void *sel, int is_i64, int E, int key_bits, int64_t seg_begin,
                                            int64_t seg_end, int *hist, int32_t *local_rank, int lane) {
     const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-    for (int64_t base = seg_begin; base < seg_end; base += 64) {
-        const int64_t j = base + lane;
-        bool valid = j < seg_end;
-        int key = 0;
-        if (valid) {
-            const int64_t k64 = load_key(sel, is_i64, j);
-            valid = k64 >= 0 && k64 < E;
-            key = valid ? (int)k64 : 0;
+    for (int64_t chunk = seg_begin; chunk < seg_end; chunk += 64 * kSortChunk) {
+        // all loads of the chunk first: their latencies overlap instead of adding up
+        int keys[kSortChunk];
+#pragma unroll
+        for (int u = 0; u < kSortChunk; ++u) {
+            const int64_t j = chunk + u * 64 + lane;
+            int key = -1;
+            if (j < seg_end) {
+                const int64_t k64 = load_key(sel, is_i64, j);
+                key = (k64 >= 0 && k64 < E) ? (int)k64 : -1;
+            }
+            keys[u] = key;
         }
-        uint64_t same = __ballot(valid);
-        for (int b = 0; b < key_bits; ++b) {
-            const uint64_t bal = __ballot((key >> b) & 1);
-            same &= ((key >> b) & 1) ? bal : ~bal;
+#pragma unroll
+        for (int u = 0; u < kSortChunk; ++u) {
+            if (chunk + u * 64 >= seg_end) break;  // wave-uniform
+            const int key = keys[u];
+            const bool valid = key >= 0;
+            uint64_t same = __ballot(valid);
+            for (int b = 0; b < key_bits; ++b) {
+                const uint64_t bal = __ballot((key >> b) & 1);
+                same &= ((key >> b) & 1) ? bal : ~bal;
+            }
+            if (valid) {
+                const int before = hist[key];
+                const int rank = before + __popcll(same & lt_mask);
+                if (local_rank) local_rank[chunk + u * 64 + lane] = rank;
+                // the last lane of each key group publishes the new running count
+                if ((same >> lane) == 1ull) hist[key] = before + __popcll(same);
+            }
         }
-        if (valid) {
-            const int before = hist[key];
-            const int rank = before + __popcll(same & lt_mask);
-            if (local_rank) local_rank[j] = rank;
-            // the last lane of each key group publishes the new running count
-            if ((same >> lane) == 1ull) hist[key] = before + __popcll(same);
+    }
+}
+
+// Phase 3 for one wave: final position = rank within the wave's segment + global offset of
+// (wave, key); writes inv_sort_idx in place of the rank and scatters sort_idx.
+__device__ __forceinline__ void wave_scatter(const void *sel, int is_i64, int E, int64_t seg_begin, int64_t seg_end,
+                                             const int *offsets, const int *offsets2, int32_t *sort_idx,
+                                             int32_t *rank_io, int lane) {
+    for (int64_t chunk = seg_begin; chunk < seg_end; chunk += 64 * kSortChunk) {
+        int keys[kSortChunk], ranks[kSortChunk];
+#pragma unroll
+        for (int u = 0; u < kSortChunk; ++u) {
+            const int64_t j = chunk + u * 64 + lane;
+            int key = -1, rank = 0;
+            if (j < seg_end) {
+                const int64_t k64 = load_key(sel, is_i64, j);
+                key = (k64 >= 0 && k64 < E) ? (int)k64 : -1;
+                rank = rank_io[j];
+            }
+            keys[u] = key;
+            ranks[u] = rank;
+        }
+#pragma unroll
+        for (int u = 0; u < kSortChunk; ++u) {
+            const int64_t j = chunk + u * 64 + lane;
+            if (keys[u] >= 0) {
+                const int pos = ranks[u] + offsets[keys[u]] + (offsets2 ? offsets2[keys[u]] : 0);
+                rank_io[j] = pos;
+                if (sort_idx) sort_idx[pos] = (int32_t)j;
+            }
         }
     }
 }
@@ -206,17 +249,7 @@ __global__ __launch_bounds__(1024) void sort_single_kernel(const void *__restric
         }
     }
     __syncthreads();
-    for (int64_t base = sb; base < se; base += 64) {
-        const int64_t j = base + lane;
-        if (j < se) {
-            const int64_t k64 = load_key(sel, is_i64, j);
-            if (k64 >= 0 && k64 < E) {
-                const int pos = inv_sort_idx[j] + table[wave * E + (int)k64] + totals[(int)k64];
-                inv_sort_idx[j] = pos;
-                if (sort_idx) sort_idx[pos] = (int32_t)j;
-            }
-        }
-    }
+    wave_scatter(sel, is_i64, E, sb, se, table + wave * E, totals, sort_idx, inv_sort_idx, lane);
 }
 
 // Multi-workgroup path: count -> scan -> scatter, table in global workspace.
@@ -283,18 +316,166 @@ __global__ __launch_bounds__(256) void sort_scatter_kernel(const void *__restric
     if (wave >= n_waves) return;
     int64_t sb, se;
     segment_of(wave, n_waves, R, sb, se);
-    for (int64_t base = sb; base < se; base += 64) {
-        const int64_t j = base + lane;
-        if (j < se) {
+    wave_scatter(sel, is_i64, E, sb, se, table + (int64_t)wave * E, nullptr, sort_idx, inv_sort_idx, lane);
+}
+
+// ---- two-kernel sort (E <= 512) ------------------------------------------------------------
+//
+// Many short segments (256 keys per wave) instead of a few long ones: the ballot ranking of a
+// batch depends on the LDS histogram left by the batch before it, so a wave is a serial chain
+// and the parallelism has to come from the number of waves.  Workgroups of 16 waves.
+//   kernel 1: every wave counts its segment; the workgroup turns its 16 histograms into
+//             exclusive prefixes over its waves (table[wave][e]) and a workgroup total
+//             (wg_tot[block][e]).
+//   kernel 2: a workgroup reads the (small) wg_tot table, derives the global offset of each of
+//             its (wave, expert) pairs -- experts before e, workgroups before it, waves before
+//             it -- then ranks its keys again (cheaper than a round trip of the ranks through
+//             memory) and scatters.  Workgroup 0 also writes the counts.
+
+constexpr int kFastBatches = 4;   // 64-key batches per chunk: 256 keys
+constexpr int kFastWaves = 16;    // waves per workgroup
+constexpr int kFastMaxBlocks = 64;
+
+template <int NBATCH>
+__device__ __forceinline__ void wave_rank_chunk(const void *sel, int is_i64, int E, int key_bits, int64_t begin,
+                                                int64_t seg_end, int *hist, int (&keys)[NBATCH],
+                                                int (&ranks)[NBATCH], int lane) {
+    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+    for (int u = 0; u < NBATCH; ++u) {
+        const int64_t j = begin + u * 64 + lane;
+        int key = -1;
+        if (j < seg_end) {
             const int64_t k64 = load_key(sel, is_i64, j);
-            if (k64 >= 0 && k64 < E) {
-                const int pos = inv_sort_idx[j] + table[(int64_t)wave * E + (int)k64];
-                inv_sort_idx[j] = pos;
-                if (sort_idx) sort_idx[pos] = (int32_t)j;
+            key = (k64 >= 0 && k64 < E) ? (int)k64 : -1;
+        }
+        keys[u] = key;
+    }
+#pragma unroll
+    for (int u = 0; u < NBATCH; ++u) {
+        const int key = keys[u];
+        const bool valid = key >= 0;
+        uint64_t same = __ballot(valid);
+        for (int b = 0; b < key_bits; ++b) {
+            const uint64_t bal = __ballot((key >> b) & 1);
+            same &= ((key >> b) & 1) ? bal : ~bal;
+        }
+        int rank = 0;
+        if (valid) {
+            const int before = hist[key];
+            rank = before + __popcll(same & lt_mask);
+            if ((same >> lane) == 1ull) hist[key] = before + __popcll(same);
+        }
+        ranks[u] = rank;
+    }
+}
+
+__global__ __launch_bounds__(1024) void fast_count_kernel(const void *__restrict__ sel, int is_i64, int64_t R, int E,
+                                                          int key_bits, int n_waves, int32_t *__restrict__ table,
+                                                          int32_t *__restrict__ wg_tot) {
+    extern __shared__ int lds[];  // [16][E]
+    const int wib = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * kFastWaves + wib;
+    int *hist = lds + wib * E;
+    for (int i = lane; i < E; i += 64) hist[i] = 0;
+    if (wave < n_waves) {
+        int64_t sb, se;
+        segment_of(wave, n_waves, R, sb, se);
+        for (int64_t c = sb; c < se; c += 64 * kFastBatches) {
+            int keys[kFastBatches], ranks[kFastBatches];
+            wave_rank_chunk<kFastBatches>(sel, is_i64, E, key_bits, c, se, hist, keys, ranks, lane);
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        int run = 0;
+#pragma unroll
+        for (int w = 0; w < kFastWaves; ++w) {
+            const int cnt = lds[w * E + e];
+            lds[w * E + e] = run;
+            run += cnt;
+        }
+        wg_tot[blockIdx.x * E + e] = run;
+    }
+    __syncthreads();
+    if (wave < n_waves)
+        for (int i = lane; i < E; i += 64) table[(int64_t)wave * E + i] = hist[i];
+}
+
+__global__ __launch_bounds__(1024) void fast_scatter_kernel(const void *__restrict__ sel, int is_i64, int64_t R,
+                                                            int E, int key_bits, int n_waves, int n_blocks,
+                                                            const int32_t *__restrict__ table,
+                                                            const int32_t *__restrict__ wg_tot,
+                                                            int32_t *__restrict__ counts,
+                                                            int32_t *__restrict__ sort_idx,
+                                                            int32_t *__restrict__ inv_sort_idx) {
+    extern __shared__ int lds[];  // base [E], offsets [16][E], histograms [16][E]
+    int *base = lds;
+    int *offs = base + E;
+    int *hists = offs + kFastWaves * E;
+    const int tid = threadIdx.x, wib = tid >> 6, lane = tid & 63;
+    // base[e] = rows of experts before e + rows of e in workgroups before this one
+    for (int e = tid; e < E; e += blockDim.x) {
+        int total = 0, before = 0;
+        for (int blk = 0; blk < n_blocks; ++blk) {
+            const int v = wg_tot[blk * E + e];
+            if (blk < (int)blockIdx.x) before += v;
+            total += v;
+        }
+        base[e] = total;
+        offs[e] = before;  // parked in the first offsets row until the scan is done
+        if (blockIdx.x == 0) counts[e] = total;
+    }
+    __syncthreads();
+    if (sort_idx == nullptr && inv_sort_idx == nullptr) return;
+    if (wib == 0) {  // exclusive scan of the totals over the experts, plus the workgroup part
+        int carry = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int v = e < E ? base[e] : 0;
+            int inc = v;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int up = __shfl_up(inc, o);
+                if (lane >= o) inc += up;
             }
+            if (e < E) base[e] = carry + inc - v + offs[e];
+            carry += __shfl(inc, 63);
+        }
+    }
+    __syncthreads();
+    const int wave = blockIdx.x * kFastWaves + wib;
+    if (wave >= n_waves) return;
+    int *hist = hists + wib * E;
+    int *my_off = offs + wib * E;
+    for (int i = lane; i < E; i += 64) {
+        hist[i] = 0;
+        my_off[i] = base[i] + table[(int64_t)wave * E + i];
+    }
+    int64_t sb, se;
+    segment_of(wave, n_waves, R, sb, se);
+    for (int64_t c = sb; c < se; c += 64 * kFastBatches) {
+        int keys[kFastBatches], ranks[kFastBatches];
+        wave_rank_chunk<kFastBatches>(sel, is_i64, E, key_bits, c, se, hist, keys, ranks, lane);
+#pragma unroll
+        for (int u = 0; u < kFastBatches; ++u) {
+            if (keys[u] < 0) continue;
+            const int64_t j = c + u * 64 + lane;
+            const int pos = ranks[u] + my_off[keys[u]];
+            if (inv_sort_idx) inv_sort_idx[j] = pos;
+            if (sort_idx) sort_idx[pos] = (int32_t)j;
         }
     }
 }
+
+inline int fast_waves(int64_t R) {
+    int64_t w = (R + 64 * kFastBatches - 1) / (64 * kFastBatches);
+    if (w > kFastMaxBlocks * kFastWaves) w = kFastMaxBlocks * kFastWaves;
+    if (w < 1) w = 1;
+    return (int)w;
+}
+
+inline bool fast_sort_ok(int E) { return E <= 512; }  // (2 * 16 + 1) * E ints of LDS
 
 constexpr int64_t kSingleBlockMaxR = 65536;
 
@@ -317,6 +498,10 @@ int route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int E, i
 }
 
 size_t expert_sort_workspace(int64_t R, int E) {
+    if (fast_sort_ok(E)) {
+        const int n_waves = fast_waves(R);
+        return ((size_t)(n_waves + ceil_div(n_waves, kFastWaves)) * (size_t)E * 4 + 255) / 256 * 256;
+    }
     // table for the multi-workgroup path + a rank buffer used when inv_sort_idx is not requested
     const size_t table = R > kSingleBlockMaxR ? (size_t)multi_waves(R) * (size_t)E * 4 : 0;
     const size_t ranks = (size_t)(R > 0 ? R : 0) * 4;
@@ -328,6 +513,29 @@ int expert_sort(const void *sel, int is_i64, int64_t R, int E, int32_t *counts, 
     if (E > kSortMaxE) return MFL_ERR_UNSUPPORTED;
     int key_bits = 0;
     while ((1 << key_bits) < E) ++key_bits;
+    if (fast_sort_ok(E)) {
+        const int n_waves = fast_waves(R);
+        const int n_blocks = ceil_div(n_waves, kFastWaves);
+        if (workspace == nullptr || ws_bytes < (size_t)(n_waves + n_blocks) * E * 4) return MFL_ERR_WORKSPACE;
+        int32_t *table = (int32_t *)workspace;
+        int32_t *wg_tot = table + (size_t)n_waves * E;
+        const size_t lds1 = (size_t)kFastWaves * E * 4, lds2 = (size_t)(2 * kFastWaves + 1) * E * 4;
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute((const void *)fast_scatter_kernel,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 33 * 512 * 4);
+            if (e != hipSuccess) return (int)e;
+            attr_set = true;
+        }
+        fast_count_kernel<<<n_blocks, kFastWaves * 64, lds1, stream>>>(sel, is_i64, R, E, key_bits, n_waves, table,
+                                                                       wg_tot);
+        int rc = launch_status();
+        if (rc) return rc;
+        fast_scatter_kernel<<<n_blocks, kFastWaves * 64, lds2, stream>>>(sel, is_i64, R, E, key_bits, n_waves,
+                                                                         n_blocks, table, wg_tot, counts, sort_idx,
+                                                                         inv_sort_idx);
+        return launch_status();
+    }
     const size_t table_bytes = ((R > kSingleBlockMaxR ? (size_t)multi_waves(R) * (size_t)E * 4 : 0) + 255) / 256 * 256;
     int32_t *table = (int32_t *)workspace;
     int32_t *rank_buf = inv_sort_idx;

@@ -17,13 +17,15 @@ def _sort(s: torch.Tensor, E: int, want_idx: bool) -> Tuple[torch.Tensor, Option
     assert s.ndim == 1
     s = _lib.as_index_tensor(s).contiguous()
     R = s.numel()
-    counts = torch.empty(E, device=s.device, dtype=torch.int32)
+    ws_bytes = _lib.lib().mfl_expert_sort_workspace(R, E)
+    # one allocation for all int32 outputs and the scratch table (fewer allocator calls per layer)
+    n_out = E + (2 * R if want_idx else 0)
+    buf = torch.empty(n_out + (ws_bytes + 3) // 4 + 64, device=s.device, dtype=torch.int32)
+    counts = buf[:E]
     sort_idx = inv_sort_idx = None
     if want_idx:
-        sort_idx = torch.empty(R, device=s.device, dtype=torch.int32)
-        inv_sort_idx = torch.empty(R, device=s.device, dtype=torch.int32)
-    ws_bytes = _lib.lib().mfl_expert_sort_workspace(R, E)
-    ws = torch.empty(ws_bytes, device=s.device, dtype=torch.uint8)
+        sort_idx, inv_sort_idx = buf[E:E + R], buf[E + R:E + 2 * R]
+    ws = buf[(n_out + 63) // 64 * 64:]                      # 256-byte aligned offset into a 256-byte aligned block
     rc = _lib.lib().mfl_expert_sort(_lib.ptr(s), _lib.itype_code(s.dtype), R, E, _lib.ptr(counts), _lib.ptr(sort_idx),
                                     _lib.ptr(inv_sort_idx), _lib.ptr(ws), ws_bytes, _lib.stream())
     _lib.check(rc, "mfl_expert_sort")
