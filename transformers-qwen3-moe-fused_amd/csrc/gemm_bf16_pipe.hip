@@ -151,76 +151,27 @@ __device__ __forceinline__ int tile_rows_of(int m) {
     return t == 0 ? 0 : ceil_div(ceil_div(m, t), 32) * 32;
 }
 
-template <int BM>
-__device__ __forceinline__ int count_row_tiles(const void *m_sizes, int ms_i64, int E, int n_tiles_n, int lane) {
-    int total = 0;
-    for (int e0 = 0; e0 < E; e0 += 64) {
-        const int e = e0 + lane;
-        int t = e < E ? m_tiles_of<BM>(load_msize(m_sizes, ms_i64, e)) * n_tiles_n : 0;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off);
-        total += t;
-    }
-    return total;
-}
-
-struct RowTile {
-    int expert, i0, i_end, jt;
-};
-
-// (expert, first row, row bound, n-tile) of logical tile L < total.  Within an expert the
-// m-tiles of one n-tile are consecutive, so workgroups that share a slice of the weight matrix
-// run side by side.
-template <int BM>
-__device__ __forceinline__ RowTile locate_row_tile(const void *m_sizes, int ms_i64, int E, int n_tiles_n, int64_t R,
-                                                   int L, int lane) {
-    RowTile rt = {0, 0, 0, 0};
-    int tile_carry = 0, row_carry = 0;
-    for (int e0 = 0; e0 < E; e0 += 64) {
-        const int e = e0 + lane;
-        const int m = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
-        const int t = m_tiles_of<BM>(m) * n_tiles_n;
-        int tinc = t, minc = m;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int ot = __shfl_up(tinc, off), om = __shfl_up(minc, off);
-            if (lane >= off) {
-                tinc += ot;
-                minc += om;
-            }
-        }
-        const int tbeg = tile_carry + tinc - t;
-        const uint64_t hits = __ballot(L >= tbeg && L < tbeg + t);
-        if (hits) {
-            const int src = __ffsll((unsigned long long)hits) - 1;
-            const int local = L - __shfl(tbeg, src);
-            const int m_start = row_carry + __shfl(minc - m, src);
-            const int m_size = __shfl(m, src);
-            const int m_tiles = m_tiles_of<BM>(m_size);
-            const int rows = tile_rows_of<BM>(m_size);
-            rt.expert = e0 + src;
-            rt.i0 = m_start + (local % m_tiles) * rows;
-            rt.i_end = m_start + m_size;
-            if (rt.i_end > rt.i0 + rows) rt.i_end = rt.i0 + rows;
-            if ((int64_t)rt.i_end > R) rt.i_end = (int)R;
-            rt.jt = local / m_tiles;
-            return rt;
-        }
-        tile_carry += __shfl(tinc, 63);
-        row_carry += __shfl(minc, 63);
-    }
-    return rt;
-}
+constexpr int kMaxTableExperts = 512;  // per-expert prefix tables live in LDS
 
 template <int V>
 using IC = std::integral_constant<int, V>;
 
-template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODE, typename TO>
+// NF4 weights (forward only): b points at the packed bytes; byte i holds element 2i in its high
+// nibble and 2i+1 in its low one; value = code16[nibble] * absmax[element >> bs_shift], rounded
+// once to bf16.
+struct Nf4Params {
+    const float *code16;
+    const float *absmax;
+    int bs_shift;
+};
+
+template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODE, bool NF4, typename TO>
 __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *__restrict__ a,
                                                                   const bf16_t *__restrict__ b,
                                                                   const void *__restrict__ m_sizes, int ms_i64,
                                                                   TO *__restrict__ c, int64_t R, int N, int K, int E,
-                                                                  float alpha, int accumulate) {
+                                                                  float alpha, int accumulate, Nf4Params nf4) {
+    static_assert(!NF4 || (MODE == MODE_FWD && S == 2 && BK == 64), "NF4 weights: forward product, two stages");
     constexpr int BM = MB * 32, BN = NB * 32;
     constexpr int NW = WGM * WGN;
     constexpr bool A_RC = MODE != MODE_DW;
@@ -232,7 +183,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
     constexpr int KS = BK / 16;
     typedef Stage<BM, BK, A_RC> SA;
     typedef Stage<BN, BK, B_RC> SB;
-    constexpr int LA = SA::kWaveLoads / NW, LB = SB::kWaveLoads / NW;  // copies per wave per step
+    constexpr int LA = SA::kWaveLoads / NW, LB = NF4 ? 0 : SB::kWaveLoads / NW;  // copies per wave per step
     static_assert(SA::kWaveLoads % NW == 0 && SB::kWaveLoads % NW == 0, "copies must split over the waves");
     constexpr int LPW = LA + LB;
     constexpr int STAGE_BYTES = SA::kBytes + SB::kBytes;
@@ -249,16 +200,44 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
     fo_a.init(wm * 32, WGM * 32, lane);
     fo_b.init(wn * WTN, 32, lane);
 
-    // ---- tile range of this workgroup: XCD x owns logical tiles [x*chunk, (x+1)*chunk)
-    int total, tiles_n = 0, per_expert = 0;
-    if (MODE == MODE_DW) {
-        tiles_n = ceil_div(K, BN);
-        per_expert = ceil_div(N, BM) * tiles_n;
-        total = E * per_expert;
-    } else {
-        tiles_n = ceil_div(N, BN);
-        total = __builtin_amdgcn_readfirstlane(count_row_tiles<BM>(m_sizes, ms_i64, E, tiles_n, lane));
+    // ---- per-expert prefix tables in LDS, behind the stages and the NF4 code table (every wave
+    // computes them, wave 0 writes them): rows before expert e, and tiles before expert e
+    int *tab_rows = (int *)(smem + S * STAGE_BYTES + 64);
+    int *tab_tiles = tab_rows + (kMaxTableExperts + 1);
+    const int tiles_n = MODE == MODE_DW ? ceil_div(K, BN) : ceil_div(N, BN);
+    const int per_expert = MODE == MODE_DW ? ceil_div(N, BM) * tiles_n : 0;
+    {
+        int row_carry = 0, tile_carry = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int m = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
+            const int t = e >= E ? 0 : MODE == MODE_DW ? per_expert : m_tiles_of<BM>(m) * tiles_n;
+            int minc = m, tinc = t;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int om = __shfl_up(minc, off), ot = __shfl_up(tinc, off);
+                if (lane >= off) {
+                    minc += om;
+                    tinc += ot;
+                }
+            }
+            if (wave == 0 && e <= E) {  // entry E comes from the lane behind the last expert, or from below
+                tab_rows[e] = row_carry + minc - m;
+                tab_tiles[e] = tile_carry + tinc - t;
+            }
+            row_carry += __shfl(minc, 63);
+            tile_carry += __shfl(tinc, 63);
+        }
+        if (wave == 0 && lane == 0 && E % 64 == 0) {
+            tab_rows[E] = row_carry;
+            tab_tiles[E] = tile_carry;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
     }
+    const int total = __builtin_amdgcn_readfirstlane(tab_tiles[E]);
+
+    // ---- tile range of this workgroup: XCD x owns logical tiles [x*chunk, (x+1)*chunk)
     const int chunk = ceil_div(total, kXcd);
     const int xcd = blockIdx.x % kXcd;
     const int per_xcd = gridDim.x / kXcd;
@@ -271,37 +250,48 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         const unsigned char *a_tile;
         const unsigned char *b_tile;
         int lda, ldb;
-        int64_t ldc;
+        int64_t ldc, nf4_base = 0;
         TO *c_base;
         if (MODE == MODE_DW) {
             const int e = L / per_expert, local = L % per_expert;
-            int before = 0, mine = 0;
-            for (int e0 = 0; e0 <= e; e0 += 64) {
-                const int q = e0 + lane;
-                const int m = q < E ? load_msize(m_sizes, ms_i64, q) : 0;
-                int part = q < e ? m : 0;
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
-                before += part;
-                if (e - e0 < 64) mine = __shfl(m, e - e0);
-            }
             i0 = (local / tiles_n) * BM, i_end = N;
             j0 = (local % tiles_n) * BN, j_end = K;
-            r_begin = __builtin_amdgcn_readfirstlane(before), r_end = r_begin + __builtin_amdgcn_readfirstlane(mine);
+            r_begin = __builtin_amdgcn_readfirstlane(tab_rows[e]);
+            r_end = __builtin_amdgcn_readfirstlane(tab_rows[e + 1]);
             if ((int64_t)r_end > R) r_end = (int)R;
             if (r_begin > r_end) r_begin = r_end;
             lda = N, ldb = K, ldc = K;
             a_tile = (const unsigned char *)(a + (int64_t)r_begin * lda + i0);
             b_tile = (const unsigned char *)(b + (int64_t)r_begin * ldb + j0);
-            c_base = c + (int64_t)e * N * K;
+            c_base = c + (int64_t)(L / per_expert) * N * K;
         } else {
-            const RowTile rt = locate_row_tile<BM>(m_sizes, ms_i64, E, tiles_n, R, L, lane);
-            i0 = __builtin_amdgcn_readfirstlane(rt.i0), i_end = __builtin_amdgcn_readfirstlane(rt.i_end);
-            j0 = __builtin_amdgcn_readfirstlane(rt.jt) * BN, j_end = N;
-            const int expert = __builtin_amdgcn_readfirstlane(rt.expert);
+            // expert whose tile range holds L.  Within an expert the m-tiles of one n-tile are
+            // consecutive, so workgroups that share a slice of the weight matrix run side by side.
+            int expert = 0;
+            for (int e0 = 0; e0 < E; e0 += 64) {
+                const int e = e0 + lane < E ? e0 + lane : E - 1;
+                const uint64_t hits = __ballot(e0 + lane < E && L >= tab_tiles[e] && L < tab_tiles[e + 1]);
+                if (hits) {
+                    expert = e0 + __ffsll((unsigned long long)hits) - 1;
+                    break;
+                }
+            }
+            expert = __builtin_amdgcn_readfirstlane(expert);
+            const int m_start = __builtin_amdgcn_readfirstlane(tab_rows[expert]);
+            const int m_size = __builtin_amdgcn_readfirstlane(tab_rows[expert + 1]) - m_start;
+            const int local = L - __builtin_amdgcn_readfirstlane(tab_tiles[expert]);
+            const int m_tiles = m_tiles_of<BM>(m_size);
+            const int rows = tile_rows_of<BM>(m_size);
+            i0 = m_start + (local % m_tiles) * rows;
+            i_end = m_start + m_size;
+            if (i_end > i0 + rows) i_end = i0 + rows;
+            if ((int64_t)i_end > R) i_end = (int)R;
+            if (i0 > i_end) i0 = i_end;
+            j0 = (local / m_tiles) * BN, j_end = N;
             r_begin = 0, r_end = K;
             lda = K, ldc = N;
             a_tile = (const unsigned char *)(a + (int64_t)i0 * lda);
+            nf4_base = ((int64_t)expert * N + j0) * K;  // first element of the tile's weight rows
             if (B_RC) {
                 ldb = K;
                 b_tile = (const unsigned char *)(b + (int64_t)expert * N * K + (int64_t)j0 * ldb);
@@ -380,7 +370,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         for (int s = 0; s < S - 1; ++s)
             if (s < KT) issue(s);
 
-        // ---- reduction loop, instantiated per number of row blocks that are multiplied
+        // ---- reduction loop, instantiated per number of row blocks that are multiplied.  The
+        // MFMA operands are swapped (B first): the accumulator of a lane then holds, for output
+        // row lane % 32 of the block, the columns 8g + 4*(lane / 32) + {0..3}, g = 0..3.
         auto k_loop = [&](auto ta_tag) {
             constexpr int TA = decltype(ta_tag)::value;
             for (int kt = 0; kt < KT; ++kt) {
@@ -423,25 +415,111 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                     for (int t = 0; t < TA; ++t)
 #pragma unroll
                         for (int bj = 0; bj < TN; ++bj)
-                            acc[t][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks & 1][t], fb[ks & 1][bj],
+                            acc[t][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks & 1][bj], fa[ks & 1][t],
                                                                                  acc[t][bj], 0, 0, 0);
                 }
             }
         };
+        // ---- NF4 weights: packed words travel through registers two steps ahead and are decoded
+        // into the other stage while the current one is multiplied
+        constexpr int NT_ = NW * 64;
+        constexpr int CPT = NF4 ? (BN * BK / 8) / NT_ : 1;  // 16-byte LDS chunks (8 weights) per thread
+        static_assert(!NF4 || (BN * BK / 8) % NT_ == 0, "weight chunks must split over the threads");
+        float *lut = (float *)(smem + S * STAGE_BYTES);
+        auto nf4_load = [&](int kt, uint32_t(&w)[CPT], float(&am)[CPT]) {
+#pragma unroll
+            for (int u = 0; u < CPT; ++u) {
+                const int ch = tid + NT_ * u;
+                int row = ch >> 3;
+                if (row >= j_lim) row = j_lim - 1;
+                const int64_t el = nf4_base + (int64_t)row * K + kt * BK + (ch & 7) * 8;
+                w[u] = ((const uint32_t *)b)[el >> 3];
+                am[u] = nf4.absmax[el >> nf4.bs_shift];
+            }
+        };
+        auto nf4_decode = [&](int kt, const uint32_t(&w)[CPT], const float(&am)[CPT]) {
+            unsigned char *sb = smem + (kt % S) * STAGE_BYTES + SA::kBytes;
+#pragma unroll
+            for (int u = 0; u < CPT; ++u) {
+                const int ch = tid + NT_ * u;
+                const int row = ch >> 3, kc = ch & 7;
+                bf16x8 v;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t nib = (w[u] >> (8 * (j >> 1) + ((j & 1) ? 0 : 4))) & 15u;
+                    v[j] = (bf16_t)(lut[nib] * am[u]);
+                }
+                *(bf16x8 *)(sb + row * SB::kRowBytes + SB::swz(row, kc) * 16) = v;
+            }
+        };
+        auto k_loop_nf4 = [&](auto ta_tag) {
+            constexpr int TA = decltype(ta_tag)::value;
+            uint32_t w0[CPT], w1[CPT];
+            float am0[CPT], am1[CPT];
+            if (tid < 16) lut[tid] = nf4.code16[tid];
+            if (KT > 0) nf4_load(0, w0, am0);
+            if (KT > 1) nf4_load(1, w1, am1);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __builtin_amdgcn_s_barrier();  // the code table is in LDS
+            if (KT > 0) nf4_decode(0, w0, am0);
+            auto step = [&](int kt, uint32_t(&w_even)[CPT], float(&am_even)[CPT], uint32_t(&w_odd)[CPT],
+                            float(&am_odd)[CPT]) {
+                // on entry: w_odd holds step kt+1 (in flight or landed), w_even is free
+                wait_vmcnt<0>();
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // decoded weights of step kt are written
+                __builtin_amdgcn_s_barrier();
+                if (kt + 1 < KT) issue(kt + 1);
+                if (kt + 2 < KT) nf4_load(kt + 2, w_even, am_even);
+                if (kt + 1 < KT) nf4_decode(kt + 1, w_odd, am_odd);
+                const unsigned char *sa = smem + (kt % S) * STAGE_BYTES, *sb = sa + SA::kBytes;
+                bf16x8 fa[2][TA], fb[2][TN];
+#pragma unroll
+                for (int bj = 0; bj < TN; ++bj) fb[0][bj] = fo_b.load(sb, bj, 0);
+#pragma unroll
+                for (int t = 0; t < TA; ++t) fa[0][t] = fo_a.load(sa, t, 0);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    if (ks + 1 < KS) {
+#pragma unroll
+                        for (int bj = 0; bj < TN; ++bj) fb[(ks + 1) & 1][bj] = fo_b.load(sb, bj, ks + 1);
+#pragma unroll
+                        for (int t = 0; t < TA; ++t) fa[(ks + 1) & 1][t] = fo_a.load(sa, t, ks + 1);
+                    }
+#pragma unroll
+                    for (int t = 0; t < TA; ++t)
+#pragma unroll
+                        for (int bj = 0; bj < TN; ++bj)
+                            acc[t][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks & 1][bj], fa[ks & 1][t],
+                                                                                 acc[t][bj], 0, 0, 0);
+                }
+            };
+            for (int kt = 0; kt < KT; kt += 2) {
+                step(kt, w0, am0, w1, am1);
+                if (kt + 1 < KT) step(kt + 1, w1, am1, w0, am0);
+            }
+        };
         // a wave without valid rows still copies, and multiplies one block nobody stores
+        auto run = [&](auto ta_tag) {
+            if constexpr (NF4)
+                k_loop_nf4(ta_tag);
+            else
+                k_loop(ta_tag);
+        };
         if (TM == 1 || active <= 1)
-            k_loop(IC<1>{});
+            run(IC<1>{});
         else if (TM == 2 || active == 2)
-            k_loop(IC<(TM >= 2 ? 2 : 1)>{});
+            run(IC<(TM >= 2 ? 2 : 1)>{});
         else if (TM == 3 || active == 3)
-            k_loop(IC<(TM >= 3 ? 3 : 1)>{});
+            run(IC<(TM >= 3 ? 3 : 1)>{});
         else
-            k_loop(IC<TM>{});
+            run(IC<TM>{});
 
         // ---- epilogue
+        const int h = lane >> 5, rl = lane & 31;
         if (sizeof(TO) == 2 && !accumulate) {
-            // One 32-row block of the wave at a time: stage it in LDS as bf16, then write full
-            // rows, 16 bytes per lane, instead of 2-byte stores scattered over 32 rows.
+            // One 32-row block of the wave at a time: stage it in LDS as bf16 (8 bytes per lane and
+            // write), then store whole rows, 16 bytes per lane, instead of short stores scattered
+            // over 32 rows.
             __builtin_amdgcn_s_barrier();  // all waves are done reading the last stage
             constexpr int ROWB = WTN * 2 + 16;  // padded row, bytes
             constexpr int CPR = WTN / 8;        // 16-byte chunks per row
@@ -452,10 +530,14 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 #pragma unroll
                 for (int bj = 0; bj < TN; ++bj)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                        const int col = bj * 32 + (lane & 31);
-                        *(bf16_t *)(ep + row * ROWB + col * 2) = (bf16_t)(acc[t][bj][r] * alpha);
+                    for (int g = 0; g < 4; ++g) {
+                        union {
+                            bf16_t e[4];
+                            uint2_t v;
+                        } pk;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) pk.e[u] = (bf16_t)(acc[t][bj][4 * g + u] * alpha);
+                        *(uint2_t *)(ep + rl * ROWB + (bj * 32 + 8 * g + 4 * h) * 2) = pk.v;
                     }
                 // the same wave reads back what it wrote: LDS operations of one wave complete in order
                 const int row_base = i0 + (wm + WGM * t) * 32;
@@ -464,34 +546,31 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                     const int row = row_base + row_l;
                     const int col = j0 + wn * WTN + lcol;
                     if (row >= i_end || col >= j_end) continue;
-                    const uint4_t v = *(const uint4_t *)(ep + row_l * ROWB + lcol * 2);
-                    bf16_t *dst = (bf16_t *)c_base + (int64_t)row * ldc + col;
-                    if (col + 8 <= j_end) {
-                        *(uint4_t *)dst = v;
-                    } else {
-                        const bf16_t *pv = (const bf16_t *)&v;
-                        for (int u = 0; u < j_end - col; ++u) dst[u] = pv[u];
-                    }
+                    // the output width is a multiple of 8: a chunk is inside or outside as a whole
+                    *(uint4_t *)((bf16_t *)c_base + (int64_t)row * ldc + col) =
+                        *(const uint4_t *)(ep + row_l * ROWB + lcol * 2);
                 }
             }
         } else {
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
                 if (t >= active) continue;
+                const int row = i0 + (wm + WGM * t) * 32 + rl;
+                if (row >= i_end) continue;
 #pragma unroll
-                for (int bj = 0; bj < TN; ++bj) {
-                    const int col = j0 + wn * WTN + bj * 32 + (lane & 31);
-                    if (col >= j_end) continue;
+                for (int bj = 0; bj < TN; ++bj)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int row = i0 + (wm + WGM * t) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                        if (row >= i_end) continue;
+                    for (int g = 0; g < 4; ++g) {
+                        const int col = j0 + wn * WTN + bj * 32 + 8 * g + 4 * h;
                         TO *p = c_base + (int64_t)row * ldc + col;
-                        float v = alpha * acc[t][bj][r];
-                        if (accumulate) v += to_f32(*p);
-                        *p = from_f32<TO>(v);
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            if (col + u >= j_end) continue;
+                            float v = alpha * acc[t][bj][4 * g + u];
+                            if (accumulate) v += to_f32(p[u]);
+                            p[u] = from_f32<TO>(v);
+                        }
                     }
-                }
             }
         }
     }
@@ -499,18 +578,21 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 
 template <int MB, int NB, int BK, int S, int WGM, int WGN, typename TO>
 int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
-                int K, int E, float alpha, int accumulate, hipStream_t stream) {
+                int K, int E, float alpha, int accumulate, const Nf4Params *nf4, hipStream_t stream) {
     constexpr int NT = WGM * WGN * 64;
     constexpr int STAGE_BYTES = (MB + NB) * 32 * BK * 2;
     constexpr int EP_BYTES = WGM * WGN * 32 * ((NB / WGN) * 64 + 16);
-    constexpr int LDS_BYTES = S * STAGE_BYTES > EP_BYTES ? S * STAGE_BYTES : EP_BYTES;
+    static_assert(EP_BYTES <= S * STAGE_BYTES, "the output staging reuses the stages");
+    // stages | NF4 code table | two per-expert prefix tables
+    constexpr int LDS_BYTES = S * STAGE_BYTES + 64 + 2 * (kMaxTableExperts + 1) * 4;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS capacity of a CDNA4 compute unit");
     const bf16_t *pa = (const bf16_t *)a, *pb = (const bf16_t *)b;
     TO *pc = (TO *)c;
     const int grid = device_info().cu_count / kXcd * kXcd;  // one persistent workgroup per CU
-#define MFL_PIPE(MODE)                                                                                          \
+    const Nf4Params none = {nullptr, nullptr, 0};
+#define MFL_PIPE(MODE, NF4)                                                                                     \
     {                                                                                                           \
-        auto kern = gemm_pipe_kernel<MB, NB, BK, S, WGM, WGN, MODE, TO>;                                        \
+        auto kern = gemm_pipe_kernel<MB, NB, BK, S, WGM, WGN, MODE, NF4, TO>;                                   \
         static bool attr_set = false;                                                                           \
         if (!attr_set) {                                                                                        \
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,  \
@@ -518,11 +600,15 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
             if (e != hipSuccess) return (int)e;                                                                 \
             attr_set = true;                                                                                    \
         }                                                                                                       \
-        kern<<<grid, NT, LDS_BYTES, stream>>>(pa, pb, m_sizes, ms_i64, pc, R, N, K, E, alpha, accumulate);      \
+        kern<<<grid, NT, LDS_BYTES, stream>>>(pa, pb, m_sizes, ms_i64, pc, R, N, K, E, alpha, accumulate,       \
+                                              NF4 ? *nf4 : none);                                               \
     }
-    if (mode == MODE_FWD) MFL_PIPE(MODE_FWD)
-    else if (mode == MODE_DX) MFL_PIPE(MODE_DX)
-    else MFL_PIPE(MODE_DW)
+    if (nf4 != nullptr) {
+        if constexpr (S == 2 && BK == 64 && ((NB * 32 * BK / 8) % NT == 0)) MFL_PIPE(MODE_FWD, true)
+        else return MFL_ERR_UNSUPPORTED;
+    } else if (mode == MODE_FWD) MFL_PIPE(MODE_FWD, false)
+    else if (mode == MODE_DX) MFL_PIPE(MODE_DX, false)
+    else MFL_PIPE(MODE_DW, false)
 #undef MFL_PIPE
     return launch_status();
 }
@@ -531,26 +617,21 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
 
 int g_pipe_config = 0;
 
-int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
-                   int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream) {
-    if (g_pipe_config < 0) return MFL_ERR_UNSUPPORTED;
-    if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, 16)) return MFL_ERR_UNSUPPORTED;
-    if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
-    if (mode == MODE_FWD && (K % 64 != 0 || N % 8 != 0 || N < 8)) return MFL_ERR_UNSUPPORTED;
-    if (mode == MODE_DX && (K % 64 != 0 || N % 8 != 0 || N < 8)) return MFL_ERR_UNSUPPORTED;
-    if (mode == MODE_DW && (N % 8 != 0 || K % 8 != 0 || N < 8 || K < 8)) return MFL_ERR_UNSUPPORTED;
-    if (mode != MODE_DW && R <= 0) return MFL_OK;
+namespace {
+
+int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
+                  int K, int E, int out_dtype, float alpha, int accumulate, const Nf4Params *nf4, hipStream_t stream) {
 #define MFL_LAUNCH(MB, NB, BK, S, WGM, WGN)                                                                       \
     (out_dtype == MFL_BF16 ? launch_pipe<MB, NB, BK, S, WGM, WGN, bf16_t>(mode, a, b, m_sizes, ms_i64, c, R, N, K, \
-                                                                          E, alpha, accumulate, stream)           \
+                                                                          E, alpha, accumulate, nf4, stream)      \
                            : launch_pipe<MB, NB, BK, S, WGM, WGN, float>(mode, a, b, m_sizes, ms_i64, c, R, N, K, \
-                                                                         E, alpha, accumulate, stream))
+                                                                         E, alpha, accumulate, nf4, stream))
     // Tile table (row blocks, column blocks, BK, stages, waves along M, waves along N).  The default
     // per product was picked from timings at the Qwen3-30B-A3B expert shapes.
     // Row-grouped products: 320 x 192 tiles, i.e. every expert of up to 320 rows is one tile per
     // 192-column slice (4 slices of N = 768: 512 tiles, two per CU).  DW: square 256 x 256 tiles.
     int cfg = g_pipe_config;
-    if (cfg == 0) cfg = mode == MODE_DW ? 8 : 3;
+    if (cfg == 0 || nf4 != nullptr) cfg = mode == MODE_DW ? 8 : 3;
     switch (cfg) {
         case 1:
             return MFL_LAUNCH(4, 4, 64, 4, 2, 2);
@@ -560,12 +641,42 @@ int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, 
             return MFL_LAUNCH(10, 6, 64, 2, 4, 2);
         case 4:
             return MFL_LAUNCH(10, 4, 64, 2, 4, 2);
-        case 5:
-            return MFL_LAUNCH(10, 8, 64, 2, 2, 4);
         default:
             return MFL_LAUNCH(8, 8, 64, 2, 2, 4);
     }
 #undef MFL_LAUNCH
+}
+
+}  // namespace
+
+int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
+                   int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream) {
+    if (g_pipe_config < 0 || E > kMaxTableExperts) return MFL_ERR_UNSUPPORTED;
+    if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, 16)) return MFL_ERR_UNSUPPORTED;
+    if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
+    if (mode == MODE_FWD && (K % 64 != 0 || N % 8 != 0 || N < 8)) return MFL_ERR_UNSUPPORTED;
+    if (mode == MODE_DX && (K % 64 != 0 || N % 8 != 0 || N < 8)) return MFL_ERR_UNSUPPORTED;
+    if (mode == MODE_DW && (N % 8 != 0 || K % 8 != 0 || N < 8 || K < 8)) return MFL_ERR_UNSUPPORTED;
+    if (mode != MODE_DW && R <= 0) return MFL_OK;
+    return dispatch_pipe(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, nullptr, stream);
+}
+
+int gemm_nf4_pipe(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                  const void *m_sizes, int ms_i64, void *y, int64_t R, int N, int K, int E, int out_dtype,
+                  hipStream_t stream) {
+    if (g_pipe_config < 0 || E > kMaxTableExperts) return MFL_ERR_UNSUPPORTED;
+    int shift = 0;
+    while ((1 << shift) < blocksize) ++shift;
+    // a 16-byte LDS chunk (8 weights along K) must not straddle two absmax blocks
+    if (K % 64 != 0 || N % 8 != 0 || N < 8 || blocksize < 8) return MFL_ERR_UNSUPPORTED;
+    // With a handful of rows per expert the 128 x 128 tiles of the register-staged kernel spread
+    // the weight stream over more workgroups; measured cross-over near 32 rows per expert.
+    if (R < (int64_t)32 * E) return MFL_ERR_UNSUPPORTED;
+    if (!aligned(x, 16) || !aligned(wq, 4) || !aligned(y, 16)) return MFL_ERR_UNSUPPORTED;
+    if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
+    if (R <= 0) return MFL_OK;
+    const Nf4Params nf4 = {code16, absmax, shift};
+    return dispatch_pipe(MODE_FWD, x, wq, m_sizes, ms_i64, y, R, N, K, E, out_dtype, 1.0f, 0, &nf4, stream);
 }
 
 }  // namespace mfl
