@@ -66,7 +66,7 @@ def test_argument_errors_without_device_work():
     # per-wave and per-workgroup histograms: at least one count per expert, more rows never need less
     assert lib.mfl_expert_sort_workspace(32768, 128) >= 128 * 4
     assert lib.mfl_expert_sort_workspace(65536, 128) >= lib.mfl_expert_sort_workspace(32768, 128)
-    assert lib.mfl_expert_sort_workspace(1 << 20, 128) >= (1 << 20) * 4
+    assert lib.mfl_expert_sort_workspace(1 << 20, 128) >= lib.mfl_expert_sort_workspace(65536, 128)
 
 
 def test_python_wrappers_assert_on_cpu_tensors():
