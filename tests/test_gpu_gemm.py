@@ -43,6 +43,8 @@ SHAPES = [
     (257, 136, 264, 3),      # one row past a tile edge
     (64, 16, 2048, 128),     # LoRA A shape, most experts empty
     (64, 768, 16, 128),      # LoRA B shape
+    (2000, 200, 256, 3),     # experts of several row tiles each
+    (700, 64, 128, 600),     # more experts than the pipelined kernel's LDS tables hold
 ]
 
 

@@ -27,7 +27,10 @@ def _quantised(E, N, K, blocksize, seed):
 
 
 @pytest.mark.parametrize("R,N,K,E,blocksize", [(1024, 768, 2048, 128, 256), (1024, 768, 2048, 128, 64),
-                                               (128, 768, 2048, 128, 64), (300, 40, 72, 5, 8), (513, 136, 64, 3, 64)])
+                                               (128, 768, 2048, 128, 64), (300, 40, 72, 5, 8), (513, 136, 64, 3, 64),
+                                               # >= 32 rows per expert: the pipelined kernel, several row tiles
+                                               # per expert and many reduction steps
+                                               (8192, 768, 2048, 16, 64), (4096, 200, 512, 4, 128)])
 def test_fused_nf4_forward(R, N, K, E, blocksize):
     packed, state, w_deq = _quantised(E, N, K, blocksize, R + N)
     g = gen(R)
