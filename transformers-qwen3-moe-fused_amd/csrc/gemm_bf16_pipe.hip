@@ -201,50 +201,93 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
     fo_b.init(wn * WTN, 32, lane);
 
     // ---- per-expert prefix tables in LDS, behind the stages and the NF4 code table (every wave
-    // computes them, wave 0 writes them): rows before expert e, and tiles before expert e
+    // computes them, wave 0 writes them): rows, tiles and work before expert e.  The work of a
+    // tile is its number of reduction-side units (32-row blocks, or reduction steps in DW) plus a
+    // constant for what every tile costs whatever its height (streaming its weights, the epilogue).
     int *tab_rows = (int *)(smem + S * STAGE_BYTES + 64);
     int *tab_tiles = tab_rows + (kMaxTableExperts + 1);
+    int *tab_work = tab_tiles + (kMaxTableExperts + 1);
+    constexpr int kTileConstWork = MODE == MODE_DW ? 3 : 6;
+    auto tile_work = [&](int m) {
+        return (MODE == MODE_DW ? ceil_div(m, BK) : tile_rows_of<BM>(m) / 32) + kTileConstWork;
+    };
     const int tiles_n = MODE == MODE_DW ? ceil_div(K, BN) : ceil_div(N, BN);
     const int per_expert = MODE == MODE_DW ? ceil_div(N, BM) * tiles_n : 0;
     {
-        int row_carry = 0, tile_carry = 0;
+        int row_carry = 0, tile_carry = 0, work_carry = 0;
         for (int e0 = 0; e0 < E; e0 += 64) {
             const int e = e0 + lane;
             const int m = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
             const int t = e >= E ? 0 : MODE == MODE_DW ? per_expert : m_tiles_of<BM>(m) * tiles_n;
-            int minc = m, tinc = t;
+            const int w = t * tile_work(m);
+            int minc = m, tinc = t, winc = w;
 #pragma unroll
             for (int off = 1; off < 64; off <<= 1) {
-                const int om = __shfl_up(minc, off), ot = __shfl_up(tinc, off);
+                const int om = __shfl_up(minc, off), ot = __shfl_up(tinc, off), ow = __shfl_up(winc, off);
                 if (lane >= off) {
                     minc += om;
                     tinc += ot;
+                    winc += ow;
                 }
             }
             if (wave == 0 && e <= E) {  // entry E comes from the lane behind the last expert, or from below
                 tab_rows[e] = row_carry + minc - m;
                 tab_tiles[e] = tile_carry + tinc - t;
+                tab_work[e] = work_carry + winc - w;
             }
             row_carry += __shfl(minc, 63);
             tile_carry += __shfl(tinc, 63);
+            work_carry += __shfl(winc, 63);
         }
         if (wave == 0 && lane == 0 && E % 64 == 0) {
             tab_rows[E] = row_carry;
             tab_tiles[E] = tile_carry;
+            tab_work[E] = work_carry;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
     }
     const int total = __builtin_amdgcn_readfirstlane(tab_tiles[E]);
 
-    // ---- tile range of this workgroup: XCD x owns logical tiles [x*chunk, (x+1)*chunk)
-    const int chunk = ceil_div(total, kXcd);
+    // ---- tile range of this workgroup.  XCD x owns a contiguous run of logical tiles, so the
+    // tiles of one expert meet in one L2.  With few tiles per workgroup the runs hold equal
+    // numbers of tiles (one tile more on an XCD is a whole extra round there); with many, as
+    // under skewed routing, the runs hold equal work, and the strided deal within a run mixes
+    // tall and flat tiles over its workgroups.
     const int xcd = blockIdx.x % kXcd;
     const int per_xcd = gridDim.x / kXcd;
-    int L_end = (xcd + 1) * chunk;
+    int L_begin, L_end;
+    if (total < 3 * (int)gridDim.x) {
+        const int chunk = ceil_div(total, kXcd);
+        L_begin = xcd * chunk;
+        L_end = (xcd + 1) * chunk;
+    } else {
+        const int total_work = __builtin_amdgcn_readfirstlane(tab_work[E]);
+        // first tile whose work prefix reaches total_work * x / kXcd
+        auto boundary = [&](int x) {
+            if (x >= kXcd) return total;
+            const int target = (int)((int64_t)total_work * x / kXcd);
+            int found = total;
+            for (int e0 = 0; e0 < E; e0 += 64) {
+                const int e = e0 + lane < E ? e0 + lane : E - 1;
+                const int wb = tab_work[e], we = tab_work[e + 1];
+                const uint64_t hits = __ballot(e0 + lane < E && target >= wb && target < we);
+                if (hits) {
+                    const int src = __ffsll((unsigned long long)hits) - 1;
+                    const int ex = e0 + src;
+                    const int m = tab_rows[ex + 1] - tab_rows[ex];
+                    found = tab_tiles[ex] + (target - __shfl(wb, src)) / tile_work(m);
+                    break;
+                }
+            }
+            return __builtin_amdgcn_readfirstlane(found);
+        };
+        L_begin = boundary(xcd);
+        L_end = boundary(xcd + 1);
+    }
     if (L_end > total) L_end = total;
 
-    for (int L = xcd * chunk + blockIdx.x / kXcd; L < L_end; L += per_xcd) {
+    for (int L = L_begin + blockIdx.x / kXcd; L < L_end; L += per_xcd) {
         // ---- tile coordinates
         int i0, i_end, j0, j_end, r_begin, r_end;
         const unsigned char *a_tile;
@@ -583,8 +626,8 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
     constexpr int STAGE_BYTES = (MB + NB) * 32 * BK * 2;
     constexpr int EP_BYTES = WGM * WGN * 32 * ((NB / WGN) * 64 + 16);
     static_assert(EP_BYTES <= S * STAGE_BYTES, "the output staging reuses the stages");
-    // stages | NF4 code table | two per-expert prefix tables
-    constexpr int LDS_BYTES = S * STAGE_BYTES + 64 + 2 * (kMaxTableExperts + 1) * 4;
+    // stages | NF4 code table | three per-expert prefix tables
+    constexpr int LDS_BYTES = S * STAGE_BYTES + 64 + 3 * (kMaxTableExperts + 1) * 4;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS capacity of a CDNA4 compute unit");
     const bf16_t *pa = (const bf16_t *)a, *pb = (const bf16_t *)b;
     TO *pc = (TO *)c;
@@ -628,10 +671,11 @@ int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, i
                                                                          E, alpha, accumulate, nf4, stream))
     // Tile table (row blocks, column blocks, BK, stages, waves along M, waves along N).  The default
     // per product was picked from timings at the Qwen3-30B-A3B expert shapes.
-    // Row-grouped products: 320 x 192 tiles, i.e. every expert of up to 320 rows is one tile per
-    // 192-column slice (4 slices of N = 768: 512 tiles, two per CU).  DW: square 256 x 256 tiles.
+    // Row-grouped products at a few hundred rows per expert: 320 x 192 tiles, i.e. every expert of
+    // up to 320 rows is one tile per 192-column slice (4 slices of N = 768: 512 tiles, two per CU).
+    // From about 512 rows per expert on, and in DW: square 256 x 256 tiles (fewer bytes per flop).
     int cfg = g_pipe_config;
-    if (cfg == 0 || nf4 != nullptr) cfg = mode == MODE_DW ? 8 : 3;
+    if (cfg == 0 || nf4 != nullptr) cfg = (mode == MODE_DW || R >= (int64_t)512 * E) ? 8 : 3;
     switch (cfg) {
         case 1:
             return MFL_LAUNCH(4, 4, 64, 4, 2, 2);
