@@ -619,7 +619,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
     }
 }
 
-template <int MB, int NB, int BK, int S, int WGM, int WGN, typename TO>
+// MODES: bit 0 FWD (and NF4), bit 1 DX, bit 2 DW -- the products a tile configuration is built for.
+template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODES, typename TO>
 int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
                 int K, int E, float alpha, int accumulate, const Nf4Params *nf4, hipStream_t stream) {
     constexpr int NT = WGM * WGN * 64;
@@ -647,11 +648,18 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
                                               NF4 ? *nf4 : none);                                               \
     }
     if (nf4 != nullptr) {
-        if constexpr (S == 2 && BK == 64 && ((NB * 32 * BK / 8) % NT == 0)) MFL_PIPE(MODE_FWD, true)
+        if constexpr ((MODES & 1) && S == 2 && BK == 64 && ((NB * 32 * BK / 8) % NT == 0)) MFL_PIPE(MODE_FWD, true)
         else return MFL_ERR_UNSUPPORTED;
-    } else if (mode == MODE_FWD) MFL_PIPE(MODE_FWD, false)
-    else if (mode == MODE_DX) MFL_PIPE(MODE_DX, false)
-    else MFL_PIPE(MODE_DW, false)
+    } else if (mode == MODE_FWD) {
+        if constexpr (MODES & 1) MFL_PIPE(MODE_FWD, false)
+        else return MFL_ERR_UNSUPPORTED;
+    } else if (mode == MODE_DX) {
+        if constexpr (MODES & 2) MFL_PIPE(MODE_DX, false)
+        else return MFL_ERR_UNSUPPORTED;
+    } else {
+        if constexpr (MODES & 4) MFL_PIPE(MODE_DW, false)
+        else return MFL_ERR_UNSUPPORTED;
+    }
 #undef MFL_PIPE
     return launch_status();
 }
@@ -664,29 +672,42 @@ namespace {
 
 int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
                   int K, int E, int out_dtype, float alpha, int accumulate, const Nf4Params *nf4, hipStream_t stream) {
-#define MFL_LAUNCH(MB, NB, BK, S, WGM, WGN)                                                                       \
-    (out_dtype == MFL_BF16 ? launch_pipe<MB, NB, BK, S, WGM, WGN, bf16_t>(mode, a, b, m_sizes, ms_i64, c, R, N, K, \
-                                                                          E, alpha, accumulate, nf4, stream)      \
-                           : launch_pipe<MB, NB, BK, S, WGM, WGN, float>(mode, a, b, m_sizes, ms_i64, c, R, N, K, \
-                                                                         E, alpha, accumulate, nf4, stream))
-    // Tile table (row blocks, column blocks, BK, stages, waves along M, waves along N).  The default
-    // per product was picked from timings at the Qwen3-30B-A3B expert shapes.
+#define MFL_LAUNCH(MB, NB, BK, S, WGM, WGN, MODES)                                                              \
+    (out_dtype == MFL_BF16                                                                                     \
+         ? launch_pipe<MB, NB, BK, S, WGM, WGN, MODES, bf16_t>(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, alpha, \
+                                                               accumulate, nf4, stream)                        \
+         : launch_pipe<MB, NB, BK, S, WGM, WGN, MODES, float>(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, alpha,  \
+                                                              accumulate, nf4, stream))
+    // Tile table (row blocks, column blocks, BK, stages, waves along M, waves along N, products).
+    // The default per product was picked from timings at the Qwen3-30B-A3B expert shapes.
     // Row-grouped products at a few hundred rows per expert: 320 x 192 tiles, i.e. every expert of
     // up to 320 rows is one tile per 192-column slice (4 slices of N = 768: 512 tiles, two per CU).
     // From about 512 rows per expert on, and in DW: square 256 x 256 tiles (fewer bytes per flop).
+    // Rank-r LoRA products (one side of the output at most 64 wide) are bound by streaming the
+    // wide operand: small stages, many of them, so that a CU keeps 100 KiB and more in flight.
     int cfg = g_pipe_config;
-    if (cfg == 0 || nf4 != nullptr) cfg = (mode == MODE_DW || R >= (int64_t)512 * E) ? 8 : 3;
+    if (cfg == 0 || nf4 != nullptr) {
+        if (mode == MODE_DW)
+            cfg = (N <= 64 || K <= 64) ? 11 : 8;
+        else
+            cfg = (N <= 64 && nf4 == nullptr) ? 10 : R >= (int64_t)512 * E ? 8 : 3;
+    }
     switch (cfg) {
         case 1:
-            return MFL_LAUNCH(4, 4, 64, 4, 2, 2);
+            return MFL_LAUNCH(4, 4, 64, 4, 2, 2, 7);
         case 2:
-            return MFL_LAUNCH(8, 4, 64, 3, 4, 2);
+            return MFL_LAUNCH(8, 4, 64, 3, 4, 2, 7);
         case 3:
-            return MFL_LAUNCH(10, 6, 64, 2, 4, 2);
+            return MFL_LAUNCH(10, 6, 64, 2, 4, 2, 7);
         case 4:
-            return MFL_LAUNCH(10, 4, 64, 2, 4, 2);
+            return MFL_LAUNCH(10, 4, 64, 2, 4, 2, 7);
+        case 10:  // thin output of a row-grouped product: 128 rows x 64 columns, 6 stages of 24 KiB
+            return MFL_LAUNCH(4, 2, 64, 6, 4, 1, 3);
+        case 11:  // dW with a thin side: 64 x 64 tiles (an expert's reduction is spread over as many
+                  // workgroups as its wide side has 64-column slices), 8 stages of 16 KiB
+            return MFL_LAUNCH(2, 2, 64, 8, 2, 2, 4);
         default:
-            return MFL_LAUNCH(8, 8, 64, 2, 2, 4);
+            return MFL_LAUNCH(8, 8, 64, 2, 2, 4, 7);
     }
 #undef MFL_LAUNCH
 }
