@@ -194,6 +194,38 @@ def main() -> int:
                                        "fused_packed_gbs": round(packed_bytes / us_f / 1e3, 1),
                                        "fused_tflops": round(2.0 * tokens * TOPK * INTER * HIDDEN / us_f / 1e6, 1)}
         extra["nf4_gate_proj"] = nf4
+        del packed, qstate, x5
+        # config 4: rank-16 LoRA on gate_proj, 8192 tokens, Zipf(1.2)-skewed top-8 routing (65536 rows):
+        # the frozen base product and the five thin products of one forward + backward
+        T4, R4, RANK = 8192, 8192 * TOPK, 16
+        bias = (torch.randperm(E, device=dev).float() + 1).pow(-1.2).log()
+        _, _, s4 = softmax_topk_raw(torch.randn((T4, E), device=dev) + bias, TOPK, True, torch.bfloat16)
+        ms4, _, _ = get_expert_counts_and_idx(s4.view(-1), E)
+        x4 = torch.randn((R4, HIDDEN), device=dev, dtype=torch.bfloat16)
+        dy4 = torch.randn((R4, INTER), device=dev, dtype=torch.bfloat16)
+        la = torch.randn((E, RANK, HIDDEN), device=dev, dtype=torch.bfloat16) * 0.01
+        lb = torch.randn((E, INTER, RANK), device=dev, dtype=torch.bfloat16) * 0.01
+        u4 = grouped_gemm_forward(x4, la, ms4)
+        y4 = grouped_gemm_forward(x4, ws[0], ms4)
+        t4 = grouped_gemm_forward_transposed(dy4, lb, ms4)
+        flop4 = 2.0 * R4 * INTER * HIDDEN
+        lora = {"rows": R4, "largest_expert_rows": int(ms4.max().item()), "smallest_expert_rows": int(ms4.min().item())}
+        for name, fn, stream_bytes in (
+                ("base_fwd", lambda i: grouped_gemm_forward(x4, ws[0], ms4), None),
+                ("base_dx", lambda i: grouped_gemm_forward_transposed(dy4, ws[0].view(E, INTER, HIDDEN), ms4), None),
+                ("lora_a_fwd", lambda i: grouped_gemm_forward(x4, la, ms4), R4 * HIDDEN * 2),
+                ("lora_b_fwd_accumulate", lambda i: grouped_gemm_forward(u4, lb, ms4, out=y4, alpha=2.0, accumulate=True),
+                 2 * R4 * INTER * 2),
+                ("lora_dy_b", lambda i: grouped_gemm_forward_transposed(dy4, lb, ms4), R4 * INTER * 2),
+                ("lora_da", lambda i: grouped_gemm_backward_dw(x4, t4, ms4, torch.bfloat16), R4 * HIDDEN * 2),
+                ("lora_db", lambda i: grouped_gemm_backward_dw(u4, dy4, ms4, torch.bfloat16), R4 * INTER * 2)):
+            us = _event_us(fn, 20, 3, stream)
+            lora[name] = {"us": round(us, 1)}
+            if stream_bytes is None:
+                lora[name]["tflops"] = round(flop4 / us / 1e6, 1)
+            else:
+                lora[name]["wide_operand_gbs"] = round(stream_bytes / us / 1e3, 1)
+        extra["lora_rank16_zipf_config4"] = lora
         out["extra"] = extra
 
     if not args.no_cpu_baseline:

@@ -23,7 +23,7 @@
 // past the last row cost no MFMA and there is no branch inside the loop.
 //
 // Shapes this kernel takes (the caller falls back to gemm_bf16_mfma.hip otherwise):
-//   FWD, DX: K % BK == 0, N % 8 == 0.   DW: N % 8 == 0, K % 8 == 0.
+//   N % 8 == 0, K % 8 == 0 (NF4 weights: K % BK == 0).
 // Rows or columns past a tile's valid range are loaded from a clamped (valid) address and never
 // stored; in DW the rows of the last, partial reduction step are zeroed in LDS before use.
 #include <type_traits>
@@ -155,6 +155,10 @@ constexpr int kMaxTableExperts = 512;  // per-expert prefix tables live in LDS
 
 template <int V>
 using IC = std::integral_constant<int, V>;
+
+// Source of the 16-byte chunks that lie past the end of a reduction-contiguous row in the last,
+// partial reduction step (K not a multiple of BK).
+__device__ uint4_t g_zero_chunk = {0u, 0u, 0u, 0u};
 
 // NF4 weights (forward only): b points at the packed bytes; byte i holds element 2i in its high
 // nibble and 2i+1 in its low one; value = code16[nibble] * absmax[element >> bs_shift], rounded
@@ -365,28 +369,48 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             unsigned char *st = smem + (kt % S) * STAGE_BYTES;
             const unsigned char *pa = a_tile + kt * step_a;
             const unsigned char *pb = b_tile + kt * step_b;
-            // In DW the last step may be partial: lanes whose row lies past the end re-read the
-            // last valid row; those rows are zeroed in LDS before use.
-            const bool tail = MODE == MODE_DW && (kt + 1) * BK > red;
+            // The last step may be partial.  Reduction-strided operand: lanes whose row lies past
+            // the end re-read the last valid row (in DW those rows of A are zeroed in LDS before
+            // use; in DX they meet zeros of A).  Reduction-contiguous operand: chunks past the
+            // end of the row are copied from a chunk of zeros.
+            const bool tail = (kt + 1) * BK > red;
+            if (!tail) {
+#pragma unroll
+                for (int q = 0; q < LA; ++q)
+                    __builtin_amdgcn_global_load_lds((global_void_ptr)(pa + lane_off[q]),
+                                                     (lds_void_ptr)(st + (wave * LA + q) * 1024), 16, 0, 0);
+#pragma unroll
+                for (int q = 0; q < LB; ++q)
+                    __builtin_amdgcn_global_load_lds((global_void_ptr)(pb + lane_off[LA + q]),
+                                                     (lds_void_ptr)(st + SA::kBytes + (wave * LB + q) * 1024), 16, 0, 0);
+                return;
+            }
 #pragma unroll
             for (int q = 0; q < LA; ++q) {
-                uint32_t o = lane_off[q];
-                if (!A_RC && tail) {
-                    const int row = SA::row_of(wave * LA + q, lane) + kt * BK;
-                    if (row >= red) o -= (uint32_t)(row - (red - 1)) * (uint32_t)lda * 2u;
+                const int load = wave * LA + q;
+                const unsigned char *p = pa + lane_off[q];
+                if (A_RC) {
+                    const int c = SA::swz(SA::row_of(load, lane), SA::phys_of(load, lane));
+                    if (kt * BK + c * 8 >= red) p = (const unsigned char *)&g_zero_chunk;
+                } else {
+                    const int row = SA::row_of(load, lane) + kt * BK;
+                    if (row >= red) p -= (int64_t)(row - (red - 1)) * lda * 2;
                 }
-                __builtin_amdgcn_global_load_lds((global_void_ptr)(pa + o), (lds_void_ptr)(st + (wave * LA + q) * 1024),
-                                                 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((global_void_ptr)p, (lds_void_ptr)(st + load * 1024), 16, 0, 0);
             }
 #pragma unroll
             for (int q = 0; q < LB; ++q) {
-                uint32_t o = lane_off[LA + q];
-                if (!B_RC && tail) {
-                    const int row = SB::row_of(wave * LB + q, lane) + kt * BK;
-                    if (row >= red) o -= (uint32_t)(row - (red - 1)) * (uint32_t)ldb * 2u;
+                const int load = wave * LB + q;
+                const unsigned char *p = pb + lane_off[LA + q];
+                if (B_RC) {
+                    const int c = SB::swz(SB::row_of(load, lane), SB::phys_of(load, lane));
+                    if (kt * BK + c * 8 >= red) p = (const unsigned char *)&g_zero_chunk;
+                } else {
+                    const int row = SB::row_of(load, lane) + kt * BK;
+                    if (row >= red) p -= (int64_t)(row - (red - 1)) * ldb * 2;
                 }
-                __builtin_amdgcn_global_load_lds((global_void_ptr)(pb + o),
-                                                 (lds_void_ptr)(st + SA::kBytes + (wave * LB + q) * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((global_void_ptr)p, (lds_void_ptr)(st + SA::kBytes + load * 1024), 16,
+                                                 0, 0);
             }
         };
 
@@ -594,6 +618,45 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                         *(const uint4_t *)(ep + row_l * ROWB + lcol * 2);
                 }
             }
+        } else if (sizeof(TO) == 2) {
+            // accumulate into a bf16 output: the products are staged in fp32, the old values are
+            // read as whole rows, and the sum is rounded once
+            __builtin_amdgcn_s_barrier();  // all waves are done reading the last stage
+            constexpr int ROWF = WTN * 4 + 16;  // padded row of floats, bytes
+            constexpr int CPR = WTN / 8;        // 16-byte output chunks per row
+            static_assert(NW * 32 * ROWF <= S * STAGE_BYTES, "fp32 output staging must fit in the stages");
+            unsigned char *ep = smem + wave * (32 * ROWF);
+#pragma unroll
+            for (int t = 0; t < TM; ++t) {
+                if (t >= active) continue;
+#pragma unroll
+                for (int bj = 0; bj < TN; ++bj)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        floatx4 v;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) v[u] = acc[t][bj][4 * g + u] * alpha;
+                        *(floatx4 *)(ep + rl * ROWF + (bj * 32 + 8 * g + 4 * h) * 4) = v;
+                    }
+                const int row_base = i0 + (wm + WGM * t) * 32;
+                for (int q = lane; q < 32 * CPR; q += 64) {
+                    const int row_l = q / CPR, lcol = (q % CPR) * 8;
+                    const int row = row_base + row_l;
+                    const int col = j0 + wn * WTN + lcol;
+                    if (row >= i_end || col >= j_end) continue;
+                    bf16x8 *dst = (bf16x8 *)((bf16_t *)c_base + (int64_t)row * ldc + col);
+                    const bf16x8 old = *dst;
+                    const floatx4 lo = *(const floatx4 *)(ep + row_l * ROWF + lcol * 4);
+                    const floatx4 hi = *(const floatx4 *)(ep + row_l * ROWF + lcol * 4 + 16);
+                    bf16x8 out;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        out[u] = (bf16_t)(lo[u] + (float)old[u]);
+                        out[4 + u] = (bf16_t)(hi[u] + (float)old[4 + u]);
+                    }
+                    *dst = out;
+                }
+            }
         } else {
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
@@ -719,8 +782,7 @@ int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, 
     if (g_pipe_config < 0 || E > kMaxTableExperts) return MFL_ERR_UNSUPPORTED;
     if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, 16)) return MFL_ERR_UNSUPPORTED;
     if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
-    if (mode == MODE_FWD && (K % 64 != 0 || N % 8 != 0 || N < 8)) return MFL_ERR_UNSUPPORTED;
-    if (mode == MODE_DX && (K % 64 != 0 || N % 8 != 0 || N < 8)) return MFL_ERR_UNSUPPORTED;
+    if (mode != MODE_DW && (K % 8 != 0 || K < 8 || N % 8 != 0 || N < 8)) return MFL_ERR_UNSUPPORTED;
     if (mode == MODE_DW && (N % 8 != 0 || K % 8 != 0 || N < 8 || K < 8)) return MFL_ERR_UNSUPPORTED;
     if (mode != MODE_DW && R <= 0) return MFL_OK;
     return dispatch_pipe(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, nullptr, stream);
