@@ -488,56 +488,64 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             }
         };
         // ---- NF4 weights: packed words travel through registers two steps ahead and are decoded
-        // into the other stage while the current one is multiplied
+        // into the other stage while the current one is multiplied.  A thread owns half a row of
+        // the weight stage: 32 weights = 16 packed bytes (one load) = four 16-byte LDS chunks.
+        // The 16 fp32 codes sit in LDS: whatever the nibbles, a wave's lookups fall in 16 different
+        // banks (a 256-entry table of code pairs, one lookup per byte, was 2x slower: bank conflicts).
         constexpr int NT_ = NW * 64;
-        constexpr int CPT = NF4 ? (BN * BK / 8) / NT_ : 1;  // 16-byte LDS chunks (8 weights) per thread
-        static_assert(!NF4 || (BN * BK / 8) % NT_ == 0, "weight chunks must split over the threads");
+        static_assert(!NF4 || BN * 2 <= NT_, "one thread per half row of the weight stage");
         float *lut = (float *)(smem + S * STAGE_BYTES);
-        auto nf4_load = [&](int kt, uint32_t(&w)[CPT], float(&am)[CPT]) {
+        const bool nf4_on = tid < BN * 2;
+        const int nf4_row = tid >> 1, nf4_half = tid & 1;
+        struct Nf4Regs {
+            uint4_t w;
+            float am[4];
+        };
+        auto nf4_load = [&](int kt, Nf4Regs &r) {
+            if (!nf4_on) return;
+            int row = nf4_row;
+            if (row >= j_lim) row = j_lim - 1;
+            const int64_t el = nf4_base + (int64_t)row * K + kt * BK + nf4_half * 32;
+            r.w = *(const uint4_t *)((const unsigned char *)b + (el >> 1));
+            if (nf4.bs_shift >= 5) {
+                r.am[0] = nf4.absmax[el >> nf4.bs_shift];
+            } else {
 #pragma unroll
-            for (int u = 0; u < CPT; ++u) {
-                const int ch = tid + NT_ * u;
-                int row = ch >> 3;
-                if (row >= j_lim) row = j_lim - 1;
-                const int64_t el = nf4_base + (int64_t)row * K + kt * BK + (ch & 7) * 8;
-                w[u] = ((const uint32_t *)b)[el >> 3];
-                am[u] = nf4.absmax[el >> nf4.bs_shift];
+                for (int u = 0; u < 4; ++u) r.am[u] = nf4.absmax[(el + 8 * u) >> nf4.bs_shift];
             }
         };
-        auto nf4_decode = [&](int kt, const uint32_t(&w)[CPT], const float(&am)[CPT]) {
-            unsigned char *sb = smem + (kt % S) * STAGE_BYTES + SA::kBytes;
+        auto nf4_decode = [&](int kt, const Nf4Regs &r) {
+            if (!nf4_on) return;
+            unsigned char *sb = smem + (kt % S) * STAGE_BYTES + SA::kBytes + nf4_row * SB::kRowBytes;
 #pragma unroll
-            for (int u = 0; u < CPT; ++u) {
-                const int ch = tid + NT_ * u;
-                const int row = ch >> 3, kc = ch & 7;
+            for (int u = 0; u < 4; ++u) {
+                const float am = nf4.bs_shift >= 5 ? r.am[0] : r.am[u];
                 bf16x8 v;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const uint32_t nib = (w[u] >> (8 * (j >> 1) + ((j & 1) ? 0 : 4))) & 15u;
-                    v[j] = (bf16_t)(lut[nib] * am[u]);
+                    const uint32_t nib = (r.w[u] >> (8 * (j >> 1) + ((j & 1) ? 0 : 4))) & 15u;
+                    v[j] = (bf16_t)(lut[nib] * am);
                 }
-                *(bf16x8 *)(sb + row * SB::kRowBytes + SB::swz(row, kc) * 16) = v;
+                *(bf16x8 *)(sb + SB::swz(nf4_row, nf4_half * 4 + u) * 16) = v;
             }
         };
         auto k_loop_nf4 = [&](auto ta_tag) {
             constexpr int TA = decltype(ta_tag)::value;
-            uint32_t w0[CPT], w1[CPT];
-            float am0[CPT], am1[CPT];
+            Nf4Regs r0, r1;
             if (tid < 16) lut[tid] = nf4.code16[tid];
-            if (KT > 0) nf4_load(0, w0, am0);
-            if (KT > 1) nf4_load(1, w1, am1);
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            if (KT > 0) nf4_load(0, r0);
+            if (KT > 1) nf4_load(1, r1);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();  // the code table is in LDS
-            if (KT > 0) nf4_decode(0, w0, am0);
-            auto step = [&](int kt, uint32_t(&w_even)[CPT], float(&am_even)[CPT], uint32_t(&w_odd)[CPT],
-                            float(&am_odd)[CPT]) {
-                // on entry: w_odd holds step kt+1 (in flight or landed), w_even is free
+            if (KT > 0) nf4_decode(0, r0);
+            auto step = [&](int kt, Nf4Regs &r_even, Nf4Regs &r_odd) {
+                // on entry: r_odd holds step kt+1 (in flight or landed), r_even is free
                 wait_vmcnt<0>();
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // decoded weights of step kt are written
                 __builtin_amdgcn_s_barrier();
                 if (kt + 1 < KT) issue(kt + 1);
-                if (kt + 2 < KT) nf4_load(kt + 2, w_even, am_even);
-                if (kt + 1 < KT) nf4_decode(kt + 1, w_odd, am_odd);
+                if (kt + 2 < KT) nf4_load(kt + 2, r_even);
+                if (kt + 1 < KT) nf4_decode(kt + 1, r_odd);
                 const unsigned char *sa = smem + (kt % S) * STAGE_BYTES, *sb = sa + SA::kBytes;
                 bf16x8 fa[2][TA], fb[2][TN];
 #pragma unroll
@@ -561,8 +569,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 }
             };
             for (int kt = 0; kt < KT; kt += 2) {
-                step(kt, w0, am0, w1, am1);
-                if (kt + 1 < KT) step(kt + 1, w1, am1, w0, am0);
+                step(kt, r0, r1);
+                if (kt + 1 < KT) step(kt + 1, r1, r0);
             }
         };
         // a wave without valid rows still copies, and multiplies one block nobody stores
@@ -711,7 +719,7 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
                                               NF4 ? *nf4 : none);                                               \
     }
     if (nf4 != nullptr) {
-        if constexpr ((MODES & 1) && S == 2 && BK == 64 && ((NB * 32 * BK / 8) % NT == 0)) MFL_PIPE(MODE_FWD, true)
+        if constexpr ((MODES & 1) && S == 2 && BK == 64 && NB * 64 <= NT) MFL_PIPE(MODE_FWD, true)
         else return MFL_ERR_UNSUPPORTED;
     } else if (mode == MODE_FWD) {
         if constexpr (MODES & 1) MFL_PIPE(MODE_FWD, false)
