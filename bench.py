@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the moe_fused_linear hot path on one MI355X.
 
-A step is one forward grouped GEMM over one synthetic batch at BASELINE config 2
+A step is one forward grouped GEMM over one synthetic batch at benchmark configuration 2
 (Qwen3-30B-A3B gate_proj: 128 experts, weight (128, 768, 2048) bf16, 4096 tokens routed
 top-8 -> 32768 rows sorted by expert).  Inputs are resident in HBM before the timed region.
 One JSON line is printed; dX / dW at config 3 and the bandwidth-bound neighbours are reported

@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Writes tests/golden/config1.npz: BASELINE config 1 (seed 0; 8 experts, 64 -> 128 features,
+"""Writes tests/golden/config1.npz: benchmark configuration 1 (seed 0; 8 experts, 64 -> 128 features,
 256 tokens routed top-2 -> 512 rows) with expected outputs.
 
 The reference holds no golden vectors for this path, and every function on it reduces to a

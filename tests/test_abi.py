@@ -84,7 +84,7 @@ def test_python_wrappers_assert_on_cpu_tensors():
 
 def test_naive_trio_runs_on_cpu():
     """The reference's naive functions are plain torch and define the semantics on any device
-    (functional.py:7-61): checked here against the oracle on BASELINE config 1 sizes."""
+    (functional.py:7-61): checked here against the oracle on benchmark configuration 1 sizes."""
     import numpy as np
     import torch
 

@@ -1,4 +1,4 @@
-"""BASELINE config 1 against the committed fixture tests/golden/config1.npz (made by
+"""benchmark configuration 1 against the committed fixture tests/golden/config1.npz (made by
 tests/golden/make_golden.py from float64 library routines): the oracle on the CPU, and the
 HIP path on the GPU."""
 import os

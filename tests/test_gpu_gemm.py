@@ -1,7 +1,7 @@
 """GPU parity of the grouped GEMM (fwd / dX / dW) against the CPU oracle, through the C ABI
 (the Python wrappers are thin ctypes calls).  Shapes follow the reference's own scripts
 (test_moe_fused_linear.py:19-23: 1024 x 2048 -> 768, 128 experts; the tiny model's odd sizes
-3 / 16 / 11 experts from test_model.py:29-40) plus BASELINE configs 1-3."""
+3 / 16 / 11 experts from test_model.py:29-40) plus the benchmark configurations 1-3."""
 import numpy as np
 import pytest
 import torch
@@ -35,7 +35,7 @@ def _tol(dtype):
 
 SHAPES = [
     # R, N, K, E
-    (512, 128, 64, 8),       # BASELINE config 1 sizes
+    (512, 128, 64, 8),       # benchmark configuration 1 sizes
     (1024, 768, 2048, 128),  # the reference's test shape
     (91, 3, 16, 11),         # tiny model: gate/up (moe_intermediate 3, hidden 16, 11 experts)
     (91, 16, 3, 11),         # tiny model: down
@@ -138,7 +138,7 @@ def test_wrapper_asserts_like_the_reference():
         grouped_gemm_forward(torch.zeros((2, 8), dtype=torch.bfloat16, device=DEV), w, ms.float())
 
 
-# ---- BASELINE configs 2 and 3 at full size: oracle on a sample + size-independent properties
+# ---- benchmark configurations 2 and 3 at full size: oracle on a sample + size-independent properties
 
 def _config23(seed):
     g = gen(seed)

@@ -131,7 +131,7 @@ def test_lora_layer_init_and_scaling():
 
 
 def test_lora_config4_rank16_zipf_bf16():
-    """BASELINE config 4 at reduced hidden size for the oracle: rank-16 fused-format LoRA,
+    """benchmark configuration 4 at reduced hidden size for the oracle: rank-16 fused-format LoRA,
     Zipf(1.2)-skewed top-8 routing, forward + backward in bf16."""
     E, k, T, H, I, r = 128, 8, 1024, 256, 96, 16
     g = gen(44)
