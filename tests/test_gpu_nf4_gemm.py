@@ -30,7 +30,9 @@ def _quantised(E, N, K, blocksize, seed):
                                                (128, 768, 2048, 128, 64), (300, 40, 72, 5, 8), (513, 136, 64, 3, 64),
                                                # >= 32 rows per expert: the pipelined kernel, several row tiles
                                                # per expert and many reduction steps
-                                               (8192, 768, 2048, 16, 64), (4096, 200, 512, 4, 128)])
+                                               (8192, 768, 2048, 16, 64), (4096, 200, 512, 4, 128),
+                                               # small quantisation blocks on the pipelined kernel
+                                               (2048, 64, 128, 2, 16), (1500, 72, 192, 3, 8)])
 def test_fused_nf4_forward(R, N, K, E, blocksize):
     packed, state, w_deq = _quantised(E, N, K, blocksize, R + N)
     g = gen(R)
