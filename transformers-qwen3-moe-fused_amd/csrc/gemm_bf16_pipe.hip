@@ -761,7 +761,9 @@ int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, i
         if (mode == MODE_DW)
             cfg = (N <= 64 || K <= 64) ? 11 : 8;
         else
-            cfg = (N <= 64 && nf4 == nullptr) ? 10 : R >= (int64_t)512 * E ? 8 : 3;
+            cfg = (N <= 64 && nf4 == nullptr) ? 10
+                  : (R <= (int64_t)32 * E && nf4 == nullptr) ? 15
+                  : R >= (int64_t)512 * E ? 8 : 3;
     }
     switch (cfg) {
         case 1:
@@ -772,6 +774,9 @@ int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, i
             return MFL_LAUNCH(10, 6, 64, 2, 4, 2, 7);
         case 4:
             return MFL_LAUNCH(10, 4, 64, 2, 4, 2, 7);
+        case 15:  // a few rows per expert (decode): the weights are all the traffic; flat 64 x 128 tiles,
+                  // 6 stages of 24 KiB
+            return MFL_LAUNCH(2, 4, 64, 6, 2, 4, 3);
         case 10:  // thin output of a row-grouped product: 128 rows x 64 columns, 6 stages of 24 KiB
             return MFL_LAUNCH(4, 2, 64, 6, 4, 1, 3);
         case 11:  // dW with a thin side: 64 x 64 tiles (an expert's reduction is spread over as many
