@@ -226,6 +226,28 @@ def main() -> int:
             else:
                 lora[name]["wide_operand_gbs"] = round(stream_bytes / us / 1e3, 1)
         extra["lora_rank16_zipf_config4"] = lora
+        del x4, dy4, u4, y4, t4
+        # config 5: the whole sparse block (router -> top-k -> sort -> gather -> gate/up -> SiLU-mul -> down ->
+        # weighted combine) with NF4 experts, forward only, module calls as a user makes them
+        from types import SimpleNamespace
+        from qwen3_moe_fused.modular_qwen3_moe_fused import Qwen3MoeFusedSparseMoeBlock
+        from qwen3_moe_fused.quantize.layer import MoeFusedLinear4bit
+        cfg5 = SimpleNamespace(num_experts=E, num_experts_per_tok=TOPK, norm_topk_prob=True, hidden_size=HIDDEN,
+                               moe_intermediate_size=INTER, hidden_act="silu")
+        blk = Qwen3MoeFusedSparseMoeBlock(cfg5).to(torch.bfloat16)
+        with torch.no_grad():
+            blk.gate.weight.copy_(torch.randn(blk.gate.weight.shape) * 0.02)
+            for name, (fin, fout), wsrc in (("gate_proj", (HIDDEN, INTER), ws[0]), ("up_proj", (HIDDEN, INTER), ws[1]),
+                                            ("down_proj", (INTER, HIDDEN), ws[2].view(E, HIDDEN, INTER))):
+                setattr(blk, name, MoeFusedLinear4bit(fin, fout, E, weight=wsrc, quant_type="nf4", blocksize=64))
+        blk = blk.to(dev)
+        block = {}
+        with torch.no_grad():
+            for tokens in (16, 256, 16384):
+                h5 = torch.randn((1, tokens, HIDDEN), device=dev, dtype=torch.bfloat16)
+                us = _event_us(lambda i: blk(h5), 20 if tokens > 1000 else 50, 3, stream)
+                block[f"tokens_{tokens}"] = {"us": round(us, 1), "tokens_per_s": round(tokens / us * 1e6)}
+        extra["nf4_sparse_block_fwd_config5"] = block
         out["extra"] = extra
 
     if not args.no_cpu_baseline:
