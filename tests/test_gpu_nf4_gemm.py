@@ -32,7 +32,10 @@ def _quantised(E, N, K, blocksize, seed):
                                                # per expert and many reduction steps
                                                (8192, 768, 2048, 16, 64), (4096, 200, 512, 4, 128),
                                                # small quantisation blocks on the pipelined kernel
-                                               (2048, 64, 128, 2, 16), (1500, 72, 192, 3, 8)])
+                                               (2048, 64, 128, 2, 16), (1500, 72, 192, 3, 8),
+                                               # decode-sized batches (register-decode kernel), small blocks, a
+                                               # column count that is not a multiple of 32
+                                               (60, 64, 128, 3, 16), (90, 72, 256, 5, 8), (200, 200, 192, 9, 32)])
 def test_fused_nf4_forward(R, N, K, E, blocksize):
     packed, state, w_deq = _quantised(E, N, K, blocksize, R + N)
     g = gen(R)

@@ -130,7 +130,10 @@ int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, cons
     if (!wq || !code16 || !absmax || !m_sizes || (R > 0 && (!x || !y))) return MFL_ERR_NULL;
     if (R == 0) return MFL_OK;
     if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
-    int rc = gemm_nf4_pipe(x, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E,
+    int rc = gemm_nf4_decode(x, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E,
+                             out_dtype, (hipStream_t)stream);
+    if (rc != MFL_ERR_UNSUPPORTED) return rc;
+    rc = gemm_nf4_pipe(x, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E,
                            out_dtype, (hipStream_t)stream);
     if (rc != MFL_ERR_UNSUPPORTED) return rc;
     return gemm_nf4_mfma(x, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E, out_dtype,

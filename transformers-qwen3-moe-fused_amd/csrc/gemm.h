@@ -20,6 +20,12 @@ int gemm_bf16_mfma(int mode, const void *a, const void *b, const void *m_sizes, 
 int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
                    int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream);
 
+// Forward with NF4 weights for decode-sized batches (at most 32 rows per expert on average):
+// weights decoded in registers, no LDS stage.
+int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                    const void *m_sizes, int ms_i64, void *y, int64_t R, int N, int K, int E, int out_dtype,
+                    hipStream_t stream);
+
 // Pipelined forward with NF4 weights decoded into LDS one step ahead of the multiply.
 int gemm_nf4_pipe(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
                   const void *m_sizes, int ms_i64, void *y, int64_t R, int N, int K, int E, int out_dtype,

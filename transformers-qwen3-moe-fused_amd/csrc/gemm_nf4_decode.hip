@@ -1,0 +1,209 @@
+// Fused NF4 grouped GEMM for decode-sized batches (a few rows per expert): the packed weights are
+// all the traffic, so the kernel is built around streaming them.
+//
+// A workgroup (4 waves) owns 32 rows of one expert and 4 * CB * 32 output columns; every wave owns
+// CB 32-column blocks and works alone: no LDS stage, no barrier in the reduction loop.
+//   * v_mfma_f32_32x32x16_bf16 takes from lane l of its first operand 8 reduction elements of
+//     column l % 32 (group l / 32): 8 weights = one packed dword.  The reduction index is
+//     permuted (the same way for both operands, which leaves the sum unchanged) so that a lane
+//     owns 32 consecutive weights of its column per 64-wide step: ONE 16-byte load per lane and
+//     step feeds 4 MFMAs.  The weights are decoded in registers (16-entry code table in LDS,
+//     code * absmax in fp32, one rounding to bf16) straight into the fragment layout.
+//   * the rows come the same way: lane l holds 32 consecutive elements of row l % 32 (64 bytes).
+//   * loads run DEPTH steps ahead in registers, and two or three workgroups share a CU: tens of
+//     KiB of packed weights in flight per CU.
+// The accumulator of a lane holds output row l % 32, columns 8g + 4*(l / 32) + {0..3}.
+#include "common.h"
+#include "gemm.h"
+
+namespace mfl {
+
+namespace {
+
+constexpr int kDepth = 4;  // steps in flight
+
+template <int CB, typename TO>
+__global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restrict__ x, const uint8_t *__restrict__ wq,
+                                                         const float *__restrict__ code16,
+                                                         const float *__restrict__ absmax, int bs_shift,
+                                                         const void *__restrict__ m_sizes, int ms_i64,
+                                                         TO *__restrict__ y, int64_t R, int N, int K, int E,
+                                                         int tiles_n) {
+    __shared__ float lut[16];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+    if (tid < 16) lut[tid] = code16[tid];
+
+    // ---- which 32 rows: row tile blockIdx.x / tiles_n in the order of the experts
+    const int ct = blockIdx.x % tiles_n, rt = blockIdx.x / tiles_n;
+    int expert = -1, m_start = 0, m_size = 0, t_begin = 0;
+    {
+        int row_carry = 0, tile_carry = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int m = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
+            const int t = ceil_div(m, 32);
+            int minc = m, tinc = t;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int om = __shfl_up(minc, off), ot = __shfl_up(tinc, off);
+                if (lane >= off) {
+                    minc += om;
+                    tinc += ot;
+                }
+            }
+            const int tb = tile_carry + tinc - t;
+            const uint64_t hits = __ballot(rt >= tb && rt < tb + t);
+            if (hits) {
+                const int src = __ffsll((unsigned long long)hits) - 1;
+                expert = e0 + src;
+                m_start = row_carry + __shfl(minc - m, src);
+                m_size = __shfl(m, src);
+                t_begin = __shfl(tb, src);
+                break;
+            }
+            row_carry += __shfl(minc, 63);
+            tile_carry += __shfl(tinc, 63);
+        }
+    }
+    __syncthreads();  // the code table is in LDS (every wave of the workgroup takes the same path below)
+    if (expert < 0) return;
+    expert = __builtin_amdgcn_readfirstlane(expert);
+    const int i0 = __builtin_amdgcn_readfirstlane(m_start) + (rt - __builtin_amdgcn_readfirstlane(t_begin)) * 32;
+    int i_end = __builtin_amdgcn_readfirstlane(m_start) + __builtin_amdgcn_readfirstlane(m_size);
+    if ((int64_t)i_end > R) i_end = (int)R;
+    const int rows = i_end - i0 < 32 ? i_end - i0 : 32;
+    if (rows <= 0) return;
+
+    // ---- this lane's sources
+    const int j0 = (ct * 4 + wave) * CB * 32;  // first column of the wave
+    int64_t w_el[CB];                          // first weight of the lane in step 0, per column block
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        int col = j0 + cb * 32 + n;
+        if (col >= N) col = N - 1;  // loaded, multiplied, never stored
+        w_el[cb] = ((int64_t)expert * N + col) * K + h * 32;
+    }
+    const bf16_t *x_row = x + (int64_t)(i0 + (n < rows ? n : rows - 1)) * K + h * 32;
+    const int KT = K / 64;
+
+    struct Step {
+        uint4_t w[CB];
+        float am[CB][4];
+        uint4_t xs[4];
+    };
+    auto load = [&](int kt, Step &s) {
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            const int64_t el = w_el[cb] + (int64_t)kt * 64;
+            s.w[cb] = *(const uint4_t *)(wq + (el >> 1));
+            if (bs_shift >= 5) {
+                s.am[cb][0] = absmax[el >> bs_shift];
+            } else {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) s.am[cb][u] = absmax[(el + 8 * u) >> bs_shift];
+            }
+        }
+        const uint4_t *px = (const uint4_t *)(x_row + kt * 64);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) s.xs[u] = px[u];
+    };
+
+    floatx16 acc[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[cb][r] = 0.f;
+
+    auto multiply = [&](const Step &s) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            union {
+                uint4_t u;
+                bf16x8 v;
+            } xa;
+            xa.u = s.xs[ks];
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                const uint32_t w = s.w[cb][ks];
+                const float am = bs_shift >= 5 ? s.am[cb][0] : s.am[cb][ks];
+                bf16x8 wf;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t nib = (w >> (8 * (j >> 1) + ((j & 1) ? 0 : 4))) & 15u;
+                    wf[j] = (bf16_t)(lut[nib] * am);
+                }
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xa.v, acc[cb], 0, 0, 0);
+            }
+        }
+    };
+
+    Step st[kDepth];  // st[j] holds a step congruent to j modulo kDepth
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d)
+        if (d < KT) load(d, st[d]);
+    for (int kt = 0; kt < KT; kt += kDepth) {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            if (kt + d < KT) {
+                multiply(st[d]);
+                if (kt + d + kDepth < KT) load(kt + d + kDepth, st[d]);
+            }
+        }
+    }
+
+    // ---- output: lane = row n, 4 consecutive columns per group
+    if (n < rows) {
+        TO *y_row = y + (int64_t)(i0 + n) * N;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int col = j0 + cb * 32 + 8 * g + 4 * h;
+                if (col >= N) continue;  // N is a multiple of 8: a group of 4 is inside or outside as a whole
+                if (sizeof(TO) == 2) {
+                    union {
+                        bf16_t e[4];
+                        uint2_t v;
+                    } pk;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) pk.e[u] = (bf16_t)acc[cb][4 * g + u];
+                    *(uint2_t *)((bf16_t *)y_row + col) = pk.v;
+                } else {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) y_row[col + u] = from_f32<TO>(acc[cb][4 * g + u]);
+                }
+            }
+    }
+}
+
+}  // namespace
+
+int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                    const void *m_sizes, int ms_i64, void *y, int64_t R, int N, int K, int E, int out_dtype,
+                    hipStream_t stream) {
+    // decode-sized batches only: with more rows per expert every 32-row tile decodes the weights again
+    if (R > (int64_t)32 * E || R <= 0) return R <= 0 ? MFL_OK : MFL_ERR_UNSUPPORTED;
+    int shift = 0;
+    while ((1 << shift) < blocksize) ++shift;
+    if (K % 64 != 0 || N % 8 != 0 || N < 8 || blocksize < 8) return MFL_ERR_UNSUPPORTED;
+    if (!aligned(x, 16) || !aligned(wq, 16) || !aligned(y, 16)) return MFL_ERR_UNSUPPORTED;
+    if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
+    constexpr int CB = 1;  // 128 columns per workgroup: the most workgroups per expert (two blocks per wave: slower)
+    const int tiles_n = ceil_div(N, 4 * CB * 32);
+    const int64_t row_tiles = R / 32 + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / 32)
+    const int64_t grid = row_tiles * tiles_n;
+    if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
+    if (out_dtype == MFL_BF16)
+        nf4_decode_kernel<CB, bf16_t><<<(unsigned)grid, 256, 0, stream>>>((const bf16_t *)x, wq, code16, absmax, shift,
+                                                                         m_sizes, ms_i64, (bf16_t *)y, R, N, K, E,
+                                                                         tiles_n);
+    else
+        nf4_decode_kernel<CB, float><<<(unsigned)grid, 256, 0, stream>>>((const bf16_t *)x, wq, code16, absmax, shift,
+                                                                        m_sizes, ms_i64, (float *)y, R, N, K, E,
+                                                                        tiles_n);
+    return launch_status();
+}
+
+}  // namespace mfl
