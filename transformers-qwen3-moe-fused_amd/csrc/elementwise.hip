@@ -118,13 +118,22 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const T *src, const in
     const bool scaled = row_scale != nullptr;
     const float sc = scaled ? to_f32(row_scale[j]) : 1.0f;
     if (vec_ok) {
-        for (int c = lane * V; c < H; c += 64 * V) {
-            Vec<T> v = ld_vec(s + c);
-            if (scaled) {
+        // four vectors per lane in flight before the first store
+        constexpr int U = 4;
+        for (int c0 = lane * V; c0 < H; c0 += 64 * V * U) {
+            Vec<T> v[U];
 #pragma unroll
-                for (int u = 0; u < V; ++u) v.v[u] = from_f32<T>(to_f32(v.v[u]) * sc);
+            for (int q = 0; q < U; ++q)
+                if (c0 + q * 64 * V < H) v[q] = ld_vec(s + c0 + q * 64 * V);
+#pragma unroll
+            for (int q = 0; q < U; ++q) {
+                if (c0 + q * 64 * V >= H) continue;
+                if (scaled) {
+#pragma unroll
+                    for (int u = 0; u < V; ++u) v[q].v[u] = from_f32<T>(to_f32(v[q].v[u]) * sc);
+                }
+                st_vec(d + c0 + q * 64 * V, v[q]);
             }
-            st_vec(d + c, v);
         }
     } else {
         for (int c = lane; c < H; c += 64) d[c] = scaled ? from_f32<T>(to_f32(s[c]) * sc) : s[c];
@@ -146,11 +155,24 @@ __global__ __launch_bounds__(256) void combine_rows_kernel(const T *src, const i
             float acc[V];
 #pragma unroll
             for (int u = 0; u < V; ++u) acc[u] = 0.f;
-            for (int j = 0; j < k; ++j) {
-                const float w = weights ? to_f32(weights[t * k + j]) : 1.0f;
-                Vec<T> v = ld_vec(src + (int64_t)p[j] * H + c);
+            // the selected rows are read eight at a time before they are added (in order: the sum
+            // is the same as one row after the other)
+            constexpr int U = 8;
+            for (int j0 = 0; j0 < k; j0 += U) {
+                Vec<T> v[U];
+                float w[U];
 #pragma unroll
-                for (int u = 0; u < V; ++u) acc[u] = fmaf(to_f32(v.v[u]), w, acc[u]);
+                for (int q = 0; q < U; ++q) {
+                    if (j0 + q >= k) continue;
+                    w[q] = weights ? to_f32(weights[t * k + j0 + q]) : 1.0f;
+                    v[q] = ld_vec(src + (int64_t)p[j0 + q] * H + c);
+                }
+#pragma unroll
+                for (int q = 0; q < U; ++q) {
+                    if (j0 + q >= k) continue;
+#pragma unroll
+                    for (int u = 0; u < V; ++u) acc[u] = fmaf(to_f32(v[q].v[u]), w[q], acc[u]);
+                }
             }
             Vec<T> o;
 #pragma unroll
