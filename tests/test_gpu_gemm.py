@@ -189,3 +189,50 @@ def test_config3_down_proj_backward_full_size():
     ref = dyd.float().t() @ xd.float()
     check_close(total, to_np32(ref), 2e-2, 2e-2 * float(ref.abs().max()), "sum_e dW == dy^T x")
     assert torch.equal(grouped_gemm_backward_dw(xd, dyd, msd, torch.bfloat16), dw)
+
+
+# ---- randomised shapes: every tile configuration and edge path of the bf16 kernels
+def _random_case(seed):
+    rng = np.random.default_rng(seed)
+    E = int(rng.choice([1, 2, 3, 5, 8, 17, 40]))
+    N = int(rng.choice([8, 16, 24, 64, 72, 136, 200, 256, 384, 520]))
+    K = int(rng.choice([8, 16, 64, 72, 128, 192, 264, 512]))
+    kind = int(rng.integers(0, 4))
+    if kind == 0:      # a few rows per expert (decode-sized), many experts empty
+        m = rng.integers(0, 6, size=E) * (rng.random(E) < 0.6)
+    elif kind == 1:    # a few hundred rows per expert
+        m = rng.integers(100, 400, size=E)
+    elif kind == 2:    # skewed: one expert holds most rows, several tiles of it
+        m = rng.integers(0, 40, size=E)
+        m[int(rng.integers(0, E))] += int(rng.integers(700, 1500))
+    else:              # tile edges
+        m = rng.choice([0, 1, 31, 32, 33, 255, 256, 257, 319, 320, 321], size=E)
+    m = np.minimum(m, max(1, 6000 // E)).astype(np.int64)
+    return E, N, K, torch.from_numpy(m)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_match_oracle_bf16(seed):
+    E, N, K, ms = _random_case(seed)
+    R = int(ms.sum())
+    x, w, dy, _, _ = _case(9000 + seed, R, N, K, E, torch.bfloat16, m_sizes=ms)
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    xd, wd, dyd, msd = x.to(DEV), w.to(DEV), dy.to(DEV), ms.to(DEV)
+    what = f"seed {seed}: E={E} N={N} K={K} m_sizes={ms.tolist()}"
+
+    y = grouped_gemm_forward(xd, wd, msd)
+    exp_y = oracle.linear_fwd(to_np32(x), to_np32(w), sel)
+    check_close(y, exp_y, 1e-2, 1e-2, "fwd " + what)
+    # y2 = 0.5 * product + y, rounded once
+    y2 = y.clone()
+    grouped_gemm_forward(xd, wd, msd, out=y2, alpha=0.5, accumulate=True)
+    check_close(y2, 0.5 * exp_y + to_np32(y), 1e-2, 1e-2, "fwd accumulate " + what)
+
+    dx = grouped_gemm_forward_transposed(dyd, wd, msd)
+    check_close(dx, oracle.linear_bwd_input(to_np32(dy), to_np32(w), sel), 1e-2, 1e-2, "dx " + what)
+
+    dw = grouped_gemm_backward_dw(xd, dyd, msd, torch.bfloat16)
+    exp_dw = oracle.linear_bwd_weight(to_np32(dy), to_np32(x), sel, E)
+    check_close(dw, exp_dw, 1e-2, 1e-2 * max(1.0, np.abs(exp_dw).max()), "dw " + what)
+    for e in (ms == 0).nonzero().flatten().tolist():
+        assert torch.count_nonzero(dw[e]).item() == 0, "experts without rows must get exact zeros"

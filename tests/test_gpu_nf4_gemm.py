@@ -48,3 +48,34 @@ def test_fused_nf4_forward(R, N, K, E, blocksize):
     # the unfused route (dequantise, then bf16 GEMM) sees the same bf16 weights
     y2 = grouped_gemm_forward(x.to(DEV), dequantize_nf4(packed, state, torch.bfloat16), ms.to(DEV))
     check_close(y, to_np32(y2), 1e-2, 1e-2, "fused vs dequant-then-GEMM")
+
+
+def _random_nf4_case(seed):
+    rng = np.random.default_rng(seed)
+    E = int(rng.choice([1, 3, 6, 20]))
+    N = int(rng.choice([8, 40, 64, 136, 256, 392]))
+    K = int(rng.choice([64, 72, 128, 192, 512]))
+    blocksize = int(rng.choice([8, 16, 32, 64, 128]))
+    while (N * K) % blocksize:  # a quantisation block must not straddle two experts
+        blocksize //= 2
+    kind = int(rng.integers(0, 3))
+    if kind == 0:      # decode-sized
+        m = rng.integers(0, 20, size=E)
+    elif kind == 1:    # a few hundred rows per expert
+        m = rng.integers(60, 400, size=E)
+    else:              # one large expert
+        m = rng.integers(0, 30, size=E)
+        m[int(rng.integers(0, E))] += int(rng.integers(600, 1200))
+    return E, N, K, blocksize, torch.from_numpy(m.astype(np.int64))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_fused_nf4(seed):
+    E, N, K, blocksize, ms = _random_nf4_case(seed)
+    R = int(ms.sum())
+    packed, state, w_deq = _quantised(E, N, K, blocksize, 700 + seed)
+    x = randn((R, K), gen(800 + seed), 1.0, torch.bfloat16)
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    y = grouped_gemm_forward_4bit(x.to(DEV), packed, state, ms.to(DEV))
+    check_close(y, oracle.linear_fwd(to_np32(x), w_deq, sel),
+                what=f"seed {seed}: E={E} N={N} K={K} blocksize={blocksize} m_sizes={ms.tolist()}")
