@@ -83,6 +83,48 @@ int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, cons
                      int blocksize, const void *m_sizes, int m_sizes_dtype, void *y, int64_t R,
                      int N, int K, int E, int in_dtype, int out_dtype, void *stream);
 
+/* ---- forward products fused with their neighbours in the sparse MLP block ---------
+ * The reference names these fusions as future work (modular_qwen3_moe_fused.py:100-101,105).
+ * Each call returns MFL_ERR_UNSUPPORTED, with nothing enqueued, for a request the pipelined
+ * kernels do not take (element type other than bf16, N or K not a multiple of 8, NF4 with
+ * K % 64 != 0 or blocksize < 8, more than 512 experts, pointers not 16-byte aligned, a
+ * source matrix of 4 GiB or more); the caller then runs the separate entry points. */
+
+/* y = grouped_gemm_forward(x, w, m_sizes) with x[m, :] = x_src[row_idx[m] / idx_div, :]:
+ * the rows are gathered while they are copied into the kernel's staging memory, x is never
+ * written.  x_src (src_rows, K); row_idx (R,) int32 with values in [0, src_rows * idx_div).
+ * Replaces modular_qwen3_moe_fused.py:95-103 followed by forward.py:116-160. */
+int mfl_gemm_fwd_gather(const void *x_src, int64_t src_rows, const int32_t *row_idx, int idx_div,
+                        const void *w, const void *m_sizes, int m_sizes_dtype, void *y, int64_t R,
+                        int N, int K, int E, int in_dtype, int out_dtype, void *stream);
+
+/* The same with NF4 weights (see mfl_gemm_fwd_nf4). */
+int mfl_gemm_fwd_nf4_gather(const void *x_src, int64_t src_rows, const int32_t *row_idx,
+                            int idx_div, const uint8_t *wq, const float *code16,
+                            const float *absmax, int blocksize, const void *m_sizes,
+                            int m_sizes_dtype, void *y, int64_t R, int N, int K, int E,
+                            int in_dtype, int out_dtype, void *stream);
+
+/* h = silu(e) * g with e = grouped_gemm_forward(x, w_gate), g = grouped_gemm_forward(x, w_up),
+ * in one kernel: x is read once, e and g stay in registers.  Rounding is that of the separate
+ * calls (e and g to bf16, silu in fp32 to bf16, product to bf16), so h is bit-identical to
+ * mfl_gemm_fwd x 2 + mfl_silu_mul_fwd.  e_out / g_out (R,N), where not NULL, receive e and g
+ * (a training step needs them for the backward pass).  row_idx may be NULL: x is then (R,K)
+ * and src_rows, idx_div are ignored; otherwise rows are gathered as in mfl_gemm_fwd_gather.
+ * Replaces modular_qwen3_moe_fused.py:105-108 (gate_proj, up_proj, silu_mul). */
+int mfl_glu_fwd(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div,
+                const void *w_gate, const void *w_up, const void *m_sizes, int m_sizes_dtype,
+                void *h, void *e_out, void *g_out, int64_t R, int N, int K, int E, int dtype,
+                void *stream);
+
+/* The same with NF4 weights, each matrix with its own quantisation state. */
+int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div,
+                    const uint8_t *wq_gate, const float *code16_gate, const float *absmax_gate,
+                    int blocksize_gate, const uint8_t *wq_up, const float *code16_up,
+                    const float *absmax_up, int blocksize_up, const void *m_sizes,
+                    int m_sizes_dtype, void *h, void *e_out, void *g_out, int64_t R, int N, int K,
+                    int E, int dtype, void *stream);
+
 /* ---- NF4 / blockwise dequantisation ----------------------------------------------- */
 
 /* out[i] = code16[nibble(i)] * absmax[i / blocksize], i < n (n even).  Stands in for the

@@ -1,0 +1,144 @@
+"""Forward products fused with their neighbours (gathered rows; gate/up/SiLU in one kernel)
+against the oracle, and bit for bit against the separate kernels they stand in for."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from util import check_close, gen, m_sizes_uniform, randn, to_np32
+
+pytestmark = pytest.mark.gpu
+
+from qwen3_moe_fused.grouped_gemm.forward import grouped_gemm_forward  # noqa: E402
+from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_4bit  # noqa: E402
+from qwen3_moe_fused.grouped_gemm.fused import (grouped_gemm_forward_4bit_gathered,  # noqa: E402
+                                                grouped_gemm_forward_gathered, grouped_glu_forward,
+                                                grouped_glu_forward_4bit)
+from qwen3_moe_fused.kernels.silu_mul import silu_mul_forward  # noqa: E402
+from qwen3_moe_fused.quantize.nf4 import Nf4QuantState, nf4_code  # noqa: E402
+
+DEV = "cuda"
+
+
+def _routing(T, E, k, seed):
+    """k distinct experts per token; returns (m_sizes int32, sort_idx int32) of the stable sort."""
+    g = gen(seed)
+    sel = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).reshape(-1)
+    counts, sort_idx, _ = oracle.expert_counts_and_idx(sel.numpy(), E)
+    return torch.from_numpy(counts.astype(np.int32)), torch.from_numpy(sort_idx.astype(np.int32)), sel.numpy()
+
+
+def _quantised(E, N, K, blocksize, seed):
+    w = randn((E, N, K), gen(seed), 0.05)
+    q, absmax = oracle.nf4_quant(w.numpy(), blocksize)
+    w_deq = oracle.round_bf16(oracle.nf4_dequant(q, absmax, blocksize)).reshape(E, N, K)
+    state = Nf4QuantState(absmax=torch.from_numpy(absmax).to(DEV), shape=(E, N, K), code=nf4_code(DEV),
+                          blocksize=blocksize, dtype=torch.bfloat16)
+    return torch.from_numpy(q).view(-1, 1).to(DEV), state, w_deq
+
+
+def _oracle_glu(xg, wg, wu, sel_sorted):
+    """e, g rounded to bf16, then the SiLU-mul with the reference's rounding chain."""
+    e = oracle.round_bf16(oracle.linear_fwd(xg, wg, sel_sorted))
+    g = oracle.round_bf16(oracle.linear_fwd(xg, wu, sel_sorted))
+    h = oracle.from_bf16_bits(oracle.silu_mul_fwd_bf16(oracle.to_bf16_bits(e), oracle.to_bf16_bits(g)))
+    return h, e, g
+
+
+# (tokens, experts, selected, N, K): tile-sized, ragged, decode-sized, one expert, many rows per expert
+GATHER_CASES = [(512, 16, 4, 192, 256), (300, 5, 2, 72, 136), (8, 32, 4, 256, 128), (700, 1, 1, 64, 64),
+                (2048, 4, 2, 392, 192), (64, 128, 8, 768, 2048)]
+
+
+@pytest.mark.parametrize("T,E,k,N,K", GATHER_CASES)
+def test_gathered_forward_matches_oracle_and_explicit_gather(T, E, k, N, K):
+    ms, sort_idx, sel = _routing(T, E, k, T + N)
+    x = randn((T, K), gen(T), 1.0, torch.bfloat16)
+    w = randn((E, N, K), gen(N), 0.05, torch.bfloat16)
+    rows = sort_idx.numpy() // k
+    y = grouped_gemm_forward_gathered(x.to(DEV), sort_idx.to(DEV), k, w.to(DEV), ms.to(DEV))
+    check_close(y, oracle.linear_fwd(to_np32(x)[rows], to_np32(w), np.sort(sel, kind="stable")), what="gathered fwd")
+    y2 = grouped_gemm_forward(x[rows.astype(np.int64)].contiguous().to(DEV), w.to(DEV), ms.to(DEV))
+    assert torch.equal(y, y2), "gather folded into the operand load must not change a bit"
+
+
+@pytest.mark.parametrize("T,E,k,N,K,blocksize", [(512, 16, 4, 192, 256, 64), (40, 20, 2, 136, 128, 16),
+                                                 (1024, 4, 2, 264, 192, 32), (16, 128, 8, 768, 2048, 64)])
+def test_gathered_nf4_forward(T, E, k, N, K, blocksize):
+    ms, sort_idx, sel = _routing(T, E, k, T + N)
+    x = randn((T, K), gen(T), 1.0, torch.bfloat16)
+    packed, state, w_deq = _quantised(E, N, K, blocksize, N + K)
+    rows = sort_idx.numpy() // k
+    y = grouped_gemm_forward_4bit_gathered(x.to(DEV), sort_idx.to(DEV), k, packed, state, ms.to(DEV))
+    check_close(y, oracle.linear_fwd(to_np32(x)[rows], w_deq, np.sort(sel, kind="stable")), what="gathered nf4 fwd")
+    y2 = grouped_gemm_forward_4bit(x[rows.astype(np.int64)].contiguous().to(DEV), packed, state, ms.to(DEV))
+    assert torch.equal(y, y2)
+
+
+@pytest.mark.parametrize("gathered", [False, True])
+@pytest.mark.parametrize("T,E,k,N,K", GATHER_CASES)
+def test_glu_forward(T, E, k, N, K, gathered):
+    ms, sort_idx, sel = _routing(T, E, k, T + N + 1)
+    x = randn((T, K), gen(T), 1.0, torch.bfloat16)
+    wg = randn((E, N, K), gen(N), 0.05, torch.bfloat16)
+    wu = randn((E, N, K), gen(N + 1), 0.05, torch.bfloat16)
+    rows = (sort_idx.numpy() // k).astype(np.int64)
+    xg = x[rows].contiguous()
+    if gathered:
+        h, e, g = grouped_glu_forward(x.to(DEV), wg.to(DEV), wu.to(DEV), ms.to(DEV), sort_idx.to(DEV), k,
+                                      return_products=True)
+    else:
+        h, e, g = grouped_glu_forward(xg.to(DEV), wg.to(DEV), wu.to(DEV), ms.to(DEV), return_products=True)
+    h_ref, e_ref, g_ref = _oracle_glu(to_np32(xg), to_np32(wg), to_np32(wu), np.sort(sel, kind="stable"))
+    check_close(e, e_ref, what="gate product")
+    check_close(g, g_ref, what="up product")
+    # the oracle's e and g may differ from the kernel's by a bf16 ulp, and silu(e) * g carries that on
+    check_close(h, h_ref, 2e-2, 2e-2, what="glu")
+    # bit for bit: the separate kernels
+    e2 = grouped_gemm_forward(xg.to(DEV), wg.to(DEV), ms.to(DEV))
+    g2 = grouped_gemm_forward(xg.to(DEV), wu.to(DEV), ms.to(DEV))
+    assert torch.equal(e, e2) and torch.equal(g, g2)
+    assert torch.equal(h, silu_mul_forward(e2, g2))
+    # without the products
+    h3 = grouped_glu_forward(xg.to(DEV), wg.to(DEV), wu.to(DEV), ms.to(DEV))
+    assert torch.equal(h, h3)
+
+
+@pytest.mark.parametrize("T,E,k,N,K,bs_g,bs_u", [(512, 16, 4, 192, 256, 64, 64), (40, 20, 2, 136, 128, 16, 32),
+                                                 (1024, 4, 2, 264, 192, 32, 8), (16, 128, 8, 768, 2048, 64, 64),
+                                                 (256, 128, 8, 768, 2048, 64, 64)])
+def test_glu_nf4_forward(T, E, k, N, K, bs_g, bs_u):
+    ms, sort_idx, sel = _routing(T, E, k, T + N + 2)
+    x = randn((T, K), gen(T), 1.0, torch.bfloat16)
+    pg, sg, wg_deq = _quantised(E, N, K, bs_g, N + K)
+    pu, su, wu_deq = _quantised(E, N, K, bs_u, N + K + 1)
+    rows = (sort_idx.numpy() // k).astype(np.int64)
+    xg = x[rows].contiguous()
+    h, e, g = grouped_glu_forward_4bit(x.to(DEV), pg, sg, pu, su, ms.to(DEV), sort_idx.to(DEV), k,
+                                       return_products=True)
+    h_ref, e_ref, g_ref = _oracle_glu(to_np32(xg), wg_deq, wu_deq, np.sort(sel, kind="stable"))
+    check_close(e, e_ref, what="gate product")
+    check_close(g, g_ref, what="up product")
+    check_close(h, h_ref, 2e-2, 2e-2, what="glu")
+    e2 = grouped_gemm_forward_4bit(xg.to(DEV), pg, sg, ms.to(DEV))
+    g2 = grouped_gemm_forward_4bit(xg.to(DEV), pu, su, ms.to(DEV))
+    assert torch.equal(e, e2) and torch.equal(g, g2)
+    assert torch.equal(h, silu_mul_forward(e2, g2))
+    h3 = grouped_glu_forward_4bit(xg.to(DEV), pg, sg, pu, su, ms.to(DEV))
+    assert torch.equal(h, h3)
+
+
+def test_unsupported_requests_fall_back_to_the_separate_kernels():
+    # fp32 and a width that is not a multiple of 8: no fused kernel, same results
+    T, E, k, N, K = 64, 3, 2, 12, 20
+    ms, sort_idx, sel = _routing(T, E, k, 5)
+    x = randn((T, K), gen(1), 1.0)
+    wg, wu = randn((E, N, K), gen(2), 0.1), randn((E, N, K), gen(3), 0.1)
+    rows = (sort_idx.numpy() // k).astype(np.int64)
+    y = grouped_gemm_forward_gathered(x.to(DEV), sort_idx.to(DEV), k, wg.to(DEV), ms.to(DEV))
+    ref = oracle.linear_fwd(to_np32(x)[rows], to_np32(wg), np.sort(sel, kind="stable"))
+    check_close(y, ref, 1e-4, 1e-4, "fp32 gathered fwd")
+    h = grouped_glu_forward(x.to(DEV), wg.to(DEV), wu.to(DEV), ms.to(DEV), sort_idx.to(DEV), k)
+    e = oracle.linear_fwd(to_np32(x)[rows], to_np32(wg), np.sort(sel, kind="stable"))
+    g = oracle.linear_fwd(to_np32(x)[rows], to_np32(wu), np.sort(sel, kind="stable"))
+    check_close(h, oracle.silu_mul_fwd_f32(e, g), 1e-4, 1e-4, "fp32 glu")

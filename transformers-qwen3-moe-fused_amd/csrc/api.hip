@@ -140,6 +140,91 @@ int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, cons
                          (hipStream_t)stream);
 }
 
+/* ---- forward products fused with their neighbours in the sparse MLP block ---- */
+
+namespace {
+
+int check_fused(int64_t src_rows, const int32_t *row_idx, int idx_div, const void *m_sizes, int ms_dtype, int64_t R,
+                int N, int K, int E, int in_dtype, int out_dtype) {
+    if (R < 0 || N <= 0 || K <= 0 || E <= 0 || R > 0x7fffffff) return MFL_ERR_SHAPE;
+    if (row_idx != nullptr && (idx_div <= 0 || src_rows <= 0)) return MFL_ERR_SHAPE;
+    if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || !itype_ok(ms_dtype)) return MFL_ERR_DTYPE;
+    if (!m_sizes) return MFL_ERR_NULL;
+    return MFL_OK;
+}
+
+}  // namespace
+
+int mfl_gemm_fwd_gather(const void *x_src, int64_t src_rows, const int32_t *row_idx, int idx_div, const void *w,
+                        const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K, int E, int in_dtype,
+                        int out_dtype, void *stream) {
+    int rc = check_fused(src_rows, row_idx, idx_div, m_sizes, m_sizes_dtype, R, N, K, E, in_dtype, out_dtype);
+    if (rc) return rc;
+    if (R > 0 && (!x_src || !row_idx || !w || !y)) return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    const GemmFusion fu = {row_idx, idx_div, src_rows, nullptr, nullptr, nullptr, 0, nullptr, nullptr};
+    return gemm_bf16_pipe(MODE_FWD, x_src, w, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E, out_dtype, 1.0f, 0,
+                          (hipStream_t)stream, &fu);
+}
+
+int mfl_gemm_fwd_nf4_gather(const void *x_src, int64_t src_rows, const int32_t *row_idx, int idx_div, const uint8_t *wq,
+                            const float *code16, const float *absmax, int blocksize, const void *m_sizes,
+                            int m_sizes_dtype, void *y, int64_t R, int N, int K, int E, int in_dtype, int out_dtype,
+                            void *stream) {
+    int rc = check_fused(src_rows, row_idx, idx_div, m_sizes, m_sizes_dtype, R, N, K, E, in_dtype, out_dtype);
+    if (rc) return rc;
+    if (blocksize < 2 || (blocksize & (blocksize - 1)) != 0) return MFL_ERR_SHAPE;
+    if (K % 2 != 0 || ((int64_t)E * N * K) % blocksize != 0) return MFL_ERR_SHAPE;
+    if (!wq || !code16 || !absmax || (R > 0 && (!x_src || !row_idx || !y))) return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    const GemmFusion fu = {row_idx, idx_div, src_rows, nullptr, nullptr, nullptr, 0, nullptr, nullptr};
+    const int ms_i64 = m_sizes_dtype == MFL_I64;
+    rc = gemm_nf4_decode(x_src, wq, code16, absmax, blocksize, m_sizes, ms_i64, y, R, N, K, E, out_dtype,
+                         (hipStream_t)stream, &fu);
+    if (rc != MFL_ERR_UNSUPPORTED) return rc;
+    return gemm_nf4_pipe(x_src, wq, code16, absmax, blocksize, m_sizes, ms_i64, y, R, N, K, E, out_dtype,
+                         (hipStream_t)stream, &fu);
+}
+
+int mfl_glu_fwd(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div, const void *w_gate,
+                const void *w_up, const void *m_sizes, int m_sizes_dtype, void *h, void *e_out, void *g_out, int64_t R,
+                int N, int K, int E, int dtype, void *stream) {
+    int rc = check_fused(src_rows, row_idx, idx_div, m_sizes, m_sizes_dtype, R, N, K, E, dtype, dtype);
+    if (rc) return rc;
+    if (R > 0 && (!x || !w_gate || !w_up || !h)) return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    const GemmFusion fu = {row_idx, idx_div, src_rows, w_up, nullptr, nullptr, 0, e_out, g_out};
+    return gemm_bf16_pipe(MODE_FWD, x, w_gate, m_sizes, m_sizes_dtype == MFL_I64, h, R, N, K, E, MFL_BF16, 1.0f, 0,
+                          (hipStream_t)stream, &fu);
+}
+
+int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div, const uint8_t *wq_gate,
+                    const float *code16_gate, const float *absmax_gate, int blocksize_gate, const uint8_t *wq_up,
+                    const float *code16_up, const float *absmax_up, int blocksize_up, const void *m_sizes,
+                    int m_sizes_dtype, void *h, void *e_out, void *g_out, int64_t R, int N, int K, int E, int dtype,
+                    void *stream) {
+    int rc = check_fused(src_rows, row_idx, idx_div, m_sizes, m_sizes_dtype, R, N, K, E, dtype, dtype);
+    if (rc) return rc;
+    for (int bs : {blocksize_gate, blocksize_up}) {
+        if (bs < 2 || (bs & (bs - 1)) != 0 || ((int64_t)E * N * K) % bs != 0) return MFL_ERR_SHAPE;
+    }
+    if (K % 2 != 0) return MFL_ERR_SHAPE;
+    if (!wq_gate || !code16_gate || !absmax_gate || !wq_up || !code16_up || !absmax_up || (R > 0 && (!x || !h)))
+        return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    const GemmFusion fu = {row_idx, idx_div, src_rows, wq_up, code16_up, absmax_up, blocksize_up, e_out, g_out};
+    const int ms_i64 = m_sizes_dtype == MFL_I64;
+    rc = gemm_nf4_decode(x, wq_gate, code16_gate, absmax_gate, blocksize_gate, m_sizes, ms_i64, h, R, N, K, E, MFL_BF16,
+                         (hipStream_t)stream, &fu);
+    if (rc != MFL_ERR_UNSUPPORTED) return rc;
+    return gemm_nf4_pipe(x, wq_gate, code16_gate, absmax_gate, blocksize_gate, m_sizes, ms_i64, h, R, N, K, E, MFL_BF16,
+                         (hipStream_t)stream, &fu);
+}
+
 int mfl_nf4_dequant(const uint8_t *wq, const float *code16, const float *absmax, int blocksize, void *out, int64_t n,
                     int out_dtype, void *stream) {
     if (n < 0 || n % 2 != 0 || blocksize < 2 || n % blocksize != 0) return MFL_ERR_SHAPE;

@@ -32,6 +32,18 @@ __device__ __forceinline__ T from_f32(float v) {
     return (T)v;  // bf16/f16: one round-to-nearest-even (v_cvt_pk_bf16_f32 on gfx950)
 }
 
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// h = silu(e) * g with the rounding chain of the reference (qwen3_moe_fused/kernels/silu_mul.py:34-39):
+// silu in fp32, rounded to the storage type, then the product in the storage type.
+template <typename T>
+__device__ __forceinline__ T silu_fwd_one(T e, T g) {
+    const float e32 = to_f32(e);
+    if (sizeof(T) == 4) return from_f32<T>((e32 * sigmoid_f32(e32)) * to_f32(g));
+    const T f = from_f32<T>(e32 * sigmoid_f32(e32));
+    return from_f32<T>(to_f32(f) * to_f32(g));
+}
+
 __device__ __forceinline__ int load_msize(const void *m_sizes, int is_i64, int e) {
     return is_i64 ? (int)((const int64_t *)m_sizes)[e] : ((const int32_t *)m_sizes)[e];
 }

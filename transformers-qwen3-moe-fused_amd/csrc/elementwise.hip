@@ -25,17 +25,7 @@ __device__ __forceinline__ void st_vec(T *p, const Vec<T> &r) {
     *(uint4_t *)p = *(const uint4_t *)r.v;
 }
 
-__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
-
 // ---------------------------------------------------------------- SiLU-mul
-
-template <typename T>
-__device__ __forceinline__ T silu_fwd_one(T e, T g) {
-    const float e32 = to_f32(e);
-    if (sizeof(T) == 4) return from_f32<T>((e32 * sigmoid_f32(e32)) * to_f32(g));
-    const T f = from_f32<T>(e32 * sigmoid_f32(e32));
-    return from_f32<T>(to_f32(f) * to_f32(g));
-}
 
 template <typename T>
 __device__ __forceinline__ void silu_bwd_one(T dh, T e, T g, T &h, T &de, T &dg) {

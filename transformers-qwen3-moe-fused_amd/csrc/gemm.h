@@ -15,21 +15,37 @@ int gemm_generic(int mode, const void *a, const void *b, const void *m_sizes, in
 int gemm_bf16_mfma(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
                    int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream);
 
+// What a forward product can take over from its neighbours in the sparse MLP block.
+struct GemmFusion {
+    // gather: row i of the left operand is row row_idx[i] / idx_div of a (src_rows, K) matrix
+    const int32_t *row_idx;
+    int idx_div;
+    int64_t src_rows;
+    // gated linear unit: w2 is a second weight matrix of the same shape (the up projection, w being
+    // the gate projection); the output is silu(x w^T) * (x w2^T); e_out / g_out, where not null,
+    // receive the two products.  With NF4 weights w2 comes with its own quantisation state.
+    const void *w2;
+    const float *code16_2, *absmax_2;
+    int blocksize_2;
+    void *e_out, *g_out;
+};
+
 // Pipelined bf16 MFMA kernels (direct global->LDS copies, multi-stage) for aligned shapes.
 // Returns MFL_ERR_UNSUPPORTED for the rest.
 int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
-                   int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream);
+                   int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream,
+                   const GemmFusion *fusion = nullptr);
 
 // Forward with NF4 weights for decode-sized batches (at most 32 rows per expert on average):
 // weights decoded in registers, no LDS stage.
 int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
                     const void *m_sizes, int ms_i64, void *y, int64_t R, int N, int K, int E, int out_dtype,
-                    hipStream_t stream);
+                    hipStream_t stream, const GemmFusion *fusion = nullptr);
 
 // Pipelined forward with NF4 weights decoded into LDS one step ahead of the multiply.
 int gemm_nf4_pipe(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
                   const void *m_sizes, int ms_i64, void *y, int64_t R, int N, int K, int E, int out_dtype,
-                  hipStream_t stream);
+                  hipStream_t stream, const GemmFusion *fusion = nullptr);
 
 // bf16 MFMA forward with NF4 weights decoded in the K loop.
 int gemm_nf4_mfma(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,

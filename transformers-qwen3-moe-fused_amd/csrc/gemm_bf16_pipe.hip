@@ -169,14 +169,36 @@ struct Nf4Params {
     int bs_shift;
 };
 
-template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODE, bool NF4, typename TO>
+// Fusions of the forward product with its neighbours in the sparse MLP block.
+//   Gather: row i of A is row row_idx[i] / idx_div of `a` (the replicate-and-sort of the tokens
+//   never materialises).
+//   GLU: two weight matrices b (gate) and b2 (up) of the same shape; the output is
+//   silu(A b^T) * (A b2^T), rounded like the separate kernels round (each product to bf16, silu
+//   in fp32 to bf16, product to bf16); the two products are stored too where c_e / c_g are given.
+struct FwdFusion {
+    const int32_t *row_idx;
+    int idx_div;
+    const void *b2;
+    Nf4Params nf4_2;
+    void *c_e, *c_g;
+};
+
+template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODE, bool NF4, bool GLU, typename TO>
 __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *__restrict__ a,
                                                                   const bf16_t *__restrict__ b,
                                                                   const void *__restrict__ m_sizes, int ms_i64,
                                                                   TO *__restrict__ c, int64_t R, int N, int K, int E,
-                                                                  float alpha, int accumulate, Nf4Params nf4) {
+                                                                  float alpha, int accumulate, Nf4Params nf4,
+                                                                  FwdFusion fu) {
     static_assert(!NF4 || (MODE == MODE_FWD && S == 2 && BK == 64), "NF4 weights: forward product, two stages");
+    static_assert(!GLU || (MODE == MODE_FWD && WGN % 2 == 0 && sizeof(TO) == 2 && BK == 64),
+                  "GLU: forward product, bf16 output, the waves along N split in a gate half and an up half");
     constexpr int BM = MB * 32, BN = NB * 32;
+    // GLU: the weight stage holds BNH rows of the gate matrix and the same BNH rows of the up
+    // matrix.  Wave column wn < WGN/2 multiplies gate rows, wn >= WGN/2 the up rows of the same
+    // output columns as wave wn - WGN/2.
+    constexpr int BNH = GLU ? BN / 2 : BN;  // output columns of a tile
+    constexpr int HW = GLU ? WGN / 2 : WGN;
     constexpr int NW = WGM * WGN;
     constexpr bool A_RC = MODE != MODE_DW;
     constexpr bool B_RC = MODE == MODE_FWD;
@@ -203,19 +225,23 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
     FragOffsets<BN, BK, B_RC, TN> fo_b;
     fo_a.init(wm * 32, WGM * 32, lane);
     fo_b.init(wn * WTN, 32, lane);
+    // GLU: weight-stage row -> (matrix, column of the tile).  A copy fills 8 whole stage rows and
+    // WTN is a multiple of 32, so the matrix is the same for all lanes of a copy.
+    auto glu_up = [](int stage_row) { return (stage_row / WTN) / HW; };
+    auto glu_col = [](int stage_row) { return ((stage_row / WTN) % HW) * WTN + stage_row % WTN; };
 
-    // ---- per-expert prefix tables in LDS, behind the stages and the NF4 code table (every wave
+    // ---- per-expert prefix tables in LDS, behind the stages and the NF4 code tables (every wave
     // computes them, wave 0 writes them): rows, tiles and work before expert e.  The work of a
     // tile is its number of reduction-side units (32-row blocks, or reduction steps in DW) plus a
     // constant for what every tile costs whatever its height (streaming its weights, the epilogue).
-    int *tab_rows = (int *)(smem + S * STAGE_BYTES + 64);
+    int *tab_rows = (int *)(smem + S * STAGE_BYTES + 128);
     int *tab_tiles = tab_rows + (kMaxTableExperts + 1);
     int *tab_work = tab_tiles + (kMaxTableExperts + 1);
     constexpr int kTileConstWork = MODE == MODE_DW ? 3 : 6;
     auto tile_work = [&](int m) {
         return (MODE == MODE_DW ? ceil_div(m, BK) : tile_rows_of<BM>(m) / 32) + kTileConstWork;
     };
-    const int tiles_n = MODE == MODE_DW ? ceil_div(K, BN) : ceil_div(N, BN);
+    const int tiles_n = MODE == MODE_DW ? ceil_div(K, BN) : ceil_div(N, BNH);
     const int per_expert = MODE == MODE_DW ? ceil_div(N, BM) * tiles_n : 0;
     {
         int row_carry = 0, tile_carry = 0, work_carry = 0;
@@ -296,6 +322,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         int i0, i_end, j0, j_end, r_begin, r_end;
         const unsigned char *a_tile;
         const unsigned char *b_tile;
+        const unsigned char *b2_tile = nullptr;
         int lda, ldb;
         int64_t ldc, nf4_base = 0;
         TO *c_base;
@@ -334,7 +361,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             if (i_end > i0 + rows) i_end = i0 + rows;
             if ((int64_t)i_end > R) i_end = (int)R;
             if (i0 > i_end) i0 = i_end;
-            j0 = (local / m_tiles) * BN, j_end = N;
+            j0 = (local / m_tiles) * BNH, j_end = N;
             r_begin = 0, r_end = K;
             lda = K, ldc = N;
             a_tile = (const unsigned char *)(a + (int64_t)i0 * lda);
@@ -342,6 +369,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             if (B_RC) {
                 ldb = K;
                 b_tile = (const unsigned char *)(b + (int64_t)expert * N * K + (int64_t)j0 * ldb);
+                if (GLU) b2_tile = (const unsigned char *)((const bf16_t *)fu.b2 + (int64_t)expert * N * K + (int64_t)j0 * ldb);
             } else {
                 ldb = N;
                 b_tile = (const unsigned char *)(b + (int64_t)expert * N * K + j0);
@@ -351,7 +379,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         const int red = r_end - r_begin;
         const int KT = ceil_div(red, BK);
         const int i_lim = i_end - i0 < BM ? i_end - i0 : BM;  // valid rows (or columns) of A from the tile origin
-        const int j_lim = j_end - j0 < BN ? j_end - j0 : BN;
+        const int j_lim = j_end - j0 < BNH ? j_end - j0 : BNH;
 
         // per-lane 32-bit source offsets of this wave's copies (tile origin, reduction step 0);
         // the step advances a wave-uniform base pointer
@@ -359,9 +387,33 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 #pragma unroll
         for (int q = 0; q < LA; ++q)
             lane_off[q] = (uint32_t)lane_src_offset<BM, BK, A_RC>(wave * LA + q, lane, lda, i_lim);
+        if (MODE == MODE_FWD && fu.row_idx != nullptr) {
+            // gathered rows: offsets from the start of the source matrix (the host checked that
+            // it is smaller than 4 GiB)
 #pragma unroll
-        for (int q = 0; q < LB; ++q)
-            lane_off[LA + q] = (uint32_t)lane_src_offset<BN, BK, B_RC>(wave * LB + q, lane, ldb, j_lim);
+            for (int q = 0; q < LA; ++q) {
+                const int load = wave * LA + q;
+                const int row = SA::row_of(load, lane);
+                const int ch = SA::swz(row, SA::phys_of(load, lane));
+                const int i = row < i_lim ? row : i_lim - 1;
+                const uint32_t src = (uint32_t)fu.row_idx[i0 + i] / (uint32_t)fu.idx_div;
+                lane_off[q] = (src * (uint32_t)lda + ch * 8) * 2;
+            }
+            a_tile = (const unsigned char *)a;
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q) {
+            if (GLU) {
+                const int load = wave * LB + q;
+                const int row = SB::row_of(load, lane);
+                const int ch = SB::swz(row, SB::phys_of(load, lane));
+                int col = glu_col(row);
+                if (col >= j_lim) col = j_lim - 1;
+                lane_off[LA + q] = (uint32_t)(((int64_t)col * ldb + ch * 8) * 2);
+            } else {
+                lane_off[LA + q] = (uint32_t)lane_src_offset<BN, BK, B_RC>(wave * LB + q, lane, ldb, j_lim);
+            }
+        }
         const int64_t step_a = A_RC ? (int64_t)BK * 2 : (int64_t)BK * lda * 2;
         const int64_t step_b = B_RC ? (int64_t)BK * 2 : (int64_t)BK * ldb * 2;
 
@@ -369,6 +421,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             unsigned char *st = smem + (kt % S) * STAGE_BYTES;
             const unsigned char *pa = a_tile + kt * step_a;
             const unsigned char *pb = b_tile + kt * step_b;
+            const unsigned char *pb2 = GLU ? b2_tile + kt * step_b : pb;
+            // weight matrix of the wave's q-th copy (wave-uniform)
+            auto b_src = [&](int q) { return GLU && glu_up((wave * LB + q) * (64 / SB::kChunksPerRow)) ? pb2 : pb; };
             // The last step may be partial.  Reduction-strided operand: lanes whose row lies past
             // the end re-read the last valid row (in DW those rows of A are zeroed in LDS before
             // use; in DX they meet zeros of A).  Reduction-contiguous operand: chunks past the
@@ -381,7 +436,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                                                      (lds_void_ptr)(st + (wave * LA + q) * 1024), 16, 0, 0);
 #pragma unroll
                 for (int q = 0; q < LB; ++q)
-                    __builtin_amdgcn_global_load_lds((global_void_ptr)(pb + lane_off[LA + q]),
+                    __builtin_amdgcn_global_load_lds((global_void_ptr)(b_src(q) + lane_off[LA + q]),
                                                      (lds_void_ptr)(st + SA::kBytes + (wave * LB + q) * 1024), 16, 0, 0);
                 return;
             }
@@ -401,7 +456,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 #pragma unroll
             for (int q = 0; q < LB; ++q) {
                 const int load = wave * LB + q;
-                const unsigned char *p = pb + lane_off[LA + q];
+                const unsigned char *p = b_src(q) + lane_off[LA + q];
                 if (B_RC) {
                     const int c = SB::swz(SB::row_of(load, lane), SB::phys_of(load, lane));
                     if (kt * BK + c * 8 >= red) p = (const unsigned char *)&g_zero_chunk;
@@ -497,21 +552,28 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         float *lut = (float *)(smem + S * STAGE_BYTES);
         const bool nf4_on = tid < BN * 2;
         const int nf4_row = tid >> 1, nf4_half = tid & 1;
+        // GLU: the thread's stage row belongs to the gate or to the up matrix, each with its own
+        // packed bytes, absmax, block size and code table
+        const bool nf4_up = GLU && glu_up(nf4_row);
+        const unsigned char *nf4_w = (const unsigned char *)(nf4_up ? fu.b2 : (const void *)b);
+        const float *nf4_am = nf4_up ? fu.nf4_2.absmax : nf4.absmax;
+        const int nf4_shift = nf4_up ? fu.nf4_2.bs_shift : nf4.bs_shift;
+        const float *nf4_lut = lut + (nf4_up ? 16 : 0);
         struct Nf4Regs {
             uint4_t w;
             float am[4];
         };
         auto nf4_load = [&](int kt, Nf4Regs &r) {
             if (!nf4_on) return;
-            int row = nf4_row;
+            int row = GLU ? glu_col(nf4_row) : nf4_row;
             if (row >= j_lim) row = j_lim - 1;
             const int64_t el = nf4_base + (int64_t)row * K + kt * BK + nf4_half * 32;
-            r.w = *(const uint4_t *)((const unsigned char *)b + (el >> 1));
-            if (nf4.bs_shift >= 5) {
-                r.am[0] = nf4.absmax[el >> nf4.bs_shift];
+            r.w = *(const uint4_t *)(nf4_w + (el >> 1));
+            if (nf4_shift >= 5) {
+                r.am[0] = nf4_am[el >> nf4_shift];
             } else {
 #pragma unroll
-                for (int u = 0; u < 4; ++u) r.am[u] = nf4.absmax[(el + 8 * u) >> nf4.bs_shift];
+                for (int u = 0; u < 4; ++u) r.am[u] = nf4_am[(el + 8 * u) >> nf4_shift];
             }
         };
         auto nf4_decode = [&](int kt, const Nf4Regs &r) {
@@ -519,12 +581,12 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             unsigned char *sb = smem + (kt % S) * STAGE_BYTES + SA::kBytes + nf4_row * SB::kRowBytes;
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                const float am = nf4.bs_shift >= 5 ? r.am[0] : r.am[u];
+                const float am = nf4_shift >= 5 ? r.am[0] : r.am[u];
                 bf16x8 v;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const uint32_t nib = (r.w[u] >> (8 * (j >> 1) + ((j & 1) ? 0 : 4))) & 15u;
-                    v[j] = (bf16_t)(lut[nib] * am);
+                    v[j] = (bf16_t)(nf4_lut[nib] * am);
                 }
                 *(bf16x8 *)(sb + SB::swz(nf4_row, nf4_half * 4 + u) * 16) = v;
             }
@@ -533,6 +595,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             constexpr int TA = decltype(ta_tag)::value;
             Nf4Regs r0, r1;
             if (tid < 16) lut[tid] = nf4.code16[tid];
+            if (GLU && tid >= 16 && tid < 32) lut[tid] = fu.nf4_2.code16[tid - 16];
             if (KT > 0) nf4_load(0, r0);
             if (KT > 1) nf4_load(1, r1);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -591,7 +654,57 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 
         // ---- epilogue
         const int h = lane >> 5, rl = lane & 31;
-        if (sizeof(TO) == 2 && !accumulate) {
+        if constexpr (GLU) {
+            // Each wave stages its 32-row block of one product in LDS as bf16; the wave that holds
+            // the other product of the same rows and columns does the same; then each of the two
+            // takes 16 of the 32 rows, reads both products back as whole 16-byte chunks, and
+            // stores silu(gate) * up (and the products themselves where the caller wants them).
+            __builtin_amdgcn_s_barrier();  // all waves are done reading the last stage
+            constexpr int ROWB = WTN * 2 + 16;  // padded row, bytes
+            constexpr int CPR = WTN / 8;        // 16-byte chunks per row
+            const int up = wn / HW, cw = wn % HW;
+            unsigned char *ep = smem + wave * (32 * ROWB);
+            const unsigned char *ep_e = smem + (wm * WGN + cw) * (32 * ROWB);
+            const unsigned char *ep_g = smem + (wm * WGN + cw + HW) * (32 * ROWB);
+#pragma unroll
+            for (int t = 0; t < TM; ++t) {
+                if (t < active) {
+#pragma unroll
+                    for (int bj = 0; bj < TN; ++bj)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            union {
+                                bf16_t e[4];
+                                uint2_t v;
+                            } pk;
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) pk.e[u] = (bf16_t)acc[t][bj][4 * g + u];
+                            *(uint2_t *)(ep + rl * ROWB + (bj * 32 + 8 * g + 4 * h) * 2) = pk.v;
+                        }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();  // both products of the block are staged
+                if (t < active) {
+                    for (int q = lane; q < 16 * CPR; q += 64) {
+                        const int row_l = 16 * up + q / CPR, lcol = (q % CPR) * 8;
+                        const int row = i0 + (wm + WGM * t) * 32 + row_l;
+                        const int col = j0 + cw * WTN + lcol;
+                        if (row >= i_end || col >= j_end) continue;
+                        const bf16x8 e8 = *(const bf16x8 *)(ep_e + row_l * ROWB + lcol * 2);
+                        const bf16x8 g8 = *(const bf16x8 *)(ep_g + row_l * ROWB + lcol * 2);
+                        bf16x8 h8;
+#pragma unroll
+                        for (int u = 0; u < 8; ++u) h8[u] = silu_fwd_one<bf16_t>(e8[u], g8[u]);
+                        const int64_t o = (int64_t)row * ldc + col;
+                        *(bf16x8 *)((bf16_t *)c_base + o) = h8;
+                        if (fu.c_e) *(bf16x8 *)((bf16_t *)fu.c_e + o) = e8;
+                        if (fu.c_g) *(bf16x8 *)((bf16_t *)fu.c_g + o) = g8;
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();  // the staging areas are free again
+            }
+        } else if (sizeof(TO) == 2 && !accumulate) {
             // One 32-row block of the wave at a time: stage it in LDS as bf16 (8 bytes per lane and
             // write), then store whole rows, 16 bytes per lane, instead of short stores scattered
             // over 32 rows.
@@ -693,21 +806,26 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 // MODES: bit 0 FWD (and NF4), bit 1 DX, bit 2 DW -- the products a tile configuration is built for.
 template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODES, typename TO>
 int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
-                int K, int E, float alpha, int accumulate, const Nf4Params *nf4, hipStream_t stream) {
+                int K, int E, float alpha, int accumulate, const Nf4Params *nf4, const FwdFusion *fusion,
+                hipStream_t stream) {
     constexpr int NT = WGM * WGN * 64;
     constexpr int STAGE_BYTES = (MB + NB) * 32 * BK * 2;
     constexpr int EP_BYTES = WGM * WGN * 32 * ((NB / WGN) * 64 + 16);
     static_assert(EP_BYTES <= S * STAGE_BYTES, "the output staging reuses the stages");
-    // stages | NF4 code table | three per-expert prefix tables
-    constexpr int LDS_BYTES = S * STAGE_BYTES + 64 + 3 * (kMaxTableExperts + 1) * 4;
+    // stages | two NF4 code tables | three per-expert prefix tables
+    constexpr int LDS_BYTES = S * STAGE_BYTES + 128 + 3 * (kMaxTableExperts + 1) * 4;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS capacity of a CDNA4 compute unit");
     const bf16_t *pa = (const bf16_t *)a, *pb = (const bf16_t *)b;
     TO *pc = (TO *)c;
     const int grid = device_info().cu_count / kXcd * kXcd;  // one persistent workgroup per CU
     const Nf4Params none = {nullptr, nullptr, 0};
-#define MFL_PIPE(MODE, NF4)                                                                                     \
+    const FwdFusion no_fusion = {nullptr, 1, nullptr, none, nullptr, nullptr};
+    const FwdFusion fu = fusion ? *fusion : no_fusion;
+    const bool glu = fu.b2 != nullptr;
+    if ((glu || fu.row_idx) && mode != MODE_FWD) return MFL_ERR_UNSUPPORTED;
+#define MFL_PIPE(MODE, NF4, GLU)                                                                                \
     {                                                                                                           \
-        auto kern = gemm_pipe_kernel<MB, NB, BK, S, WGM, WGN, MODE, NF4, TO>;                                   \
+        auto kern = gemm_pipe_kernel<MB, NB, BK, S, WGM, WGN, MODE, NF4, GLU, TO>;                              \
         static bool attr_set = false;                                                                           \
         if (!attr_set) {                                                                                        \
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,  \
@@ -716,19 +834,32 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
             attr_set = true;                                                                                    \
         }                                                                                                       \
         kern<<<grid, NT, LDS_BYTES, stream>>>(pa, pb, m_sizes, ms_i64, pc, R, N, K, E, alpha, accumulate,       \
-                                              NF4 ? *nf4 : none);                                               \
+                                              NF4 ? *nf4 : none, fu);                                           \
     }
-    if (nf4 != nullptr) {
-        if constexpr ((MODES & 1) && S == 2 && BK == 64 && NB * 64 <= NT) MFL_PIPE(MODE_FWD, true)
+    // MODES bit 3: the configuration is also built with the GLU epilogue (bf16 output only)
+    constexpr bool GLU_OK = (MODES & 8) && WGN % 2 == 0 && sizeof(TO) == 2 && BK == 64;
+    if (glu) {
+        if constexpr (GLU_OK) {
+            if (nf4 != nullptr) {
+                if constexpr (S == 2 && NB * 64 <= NT) MFL_PIPE(MODE_FWD, true, true)
+                else return MFL_ERR_UNSUPPORTED;
+            } else {
+                MFL_PIPE(MODE_FWD, false, true)
+            }
+        } else {
+            return MFL_ERR_UNSUPPORTED;
+        }
+    } else if (nf4 != nullptr) {
+        if constexpr ((MODES & 1) && S == 2 && BK == 64 && NB * 64 <= NT) MFL_PIPE(MODE_FWD, true, false)
         else return MFL_ERR_UNSUPPORTED;
     } else if (mode == MODE_FWD) {
-        if constexpr (MODES & 1) MFL_PIPE(MODE_FWD, false)
+        if constexpr (MODES & 1) MFL_PIPE(MODE_FWD, false, false)
         else return MFL_ERR_UNSUPPORTED;
     } else if (mode == MODE_DX) {
-        if constexpr (MODES & 2) MFL_PIPE(MODE_DX, false)
+        if constexpr (MODES & 2) MFL_PIPE(MODE_DX, false, false)
         else return MFL_ERR_UNSUPPORTED;
     } else {
-        if constexpr (MODES & 4) MFL_PIPE(MODE_DW, false)
+        if constexpr (MODES & 4) MFL_PIPE(MODE_DW, false, false)
         else return MFL_ERR_UNSUPPORTED;
     }
 #undef MFL_PIPE
@@ -742,13 +873,14 @@ int g_pipe_config = 0;
 namespace {
 
 int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
-                  int K, int E, int out_dtype, float alpha, int accumulate, const Nf4Params *nf4, hipStream_t stream) {
+                  int K, int E, int out_dtype, float alpha, int accumulate, const Nf4Params *nf4,
+                  const FwdFusion *fusion, hipStream_t stream) {
 #define MFL_LAUNCH(MB, NB, BK, S, WGM, WGN, MODES)                                                              \
     (out_dtype == MFL_BF16                                                                                     \
          ? launch_pipe<MB, NB, BK, S, WGM, WGN, MODES, bf16_t>(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, alpha, \
-                                                               accumulate, nf4, stream)                        \
+                                                               accumulate, nf4, fusion, stream)                \
          : launch_pipe<MB, NB, BK, S, WGM, WGN, MODES, float>(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, alpha,  \
-                                                              accumulate, nf4, stream))
+                                                              accumulate, nf4, fusion, stream))
     // Tile table (row blocks, column blocks, BK, stages, waves along M, waves along N, products).
     // The default per product was picked from timings at the Qwen3-30B-A3B expert shapes.
     // Row-grouped products at a few hundred rows per expert: 320 x 192 tiles, i.e. every expert of
@@ -756,8 +888,12 @@ int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, i
     // From about 512 rows per expert on, and in DW: square 256 x 256 tiles (fewer bytes per flop).
     // Rank-r LoRA products (one side of the output at most 64 wide) are bound by streaming the
     // wide operand: small stages, many of them, so that a CU keeps 100 KiB and more in flight.
+    // Products with the GLU epilogue (bit 3): the configurations whose waves along N split in two halves.
+    const bool glu = fusion != nullptr && fusion->b2 != nullptr;
     int cfg = g_pipe_config;
-    if (cfg == 0 || nf4 != nullptr) {
+    if (glu && (cfg == 0 || nf4 != nullptr)) {
+        cfg = R >= (int64_t)512 * E ? 8 : (R <= (int64_t)32 * E && nf4 == nullptr) ? 15 : 3;
+    } else if (cfg == 0 || nf4 != nullptr) {
         if (mode == MODE_DW)
             cfg = (N <= 64 || K <= 64) ? 11 : 8;
         else
@@ -771,39 +907,79 @@ int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, i
         case 2:
             return MFL_LAUNCH(8, 4, 64, 3, 4, 2, 7);
         case 3:
-            return MFL_LAUNCH(10, 6, 64, 2, 4, 2, 7);
+            return MFL_LAUNCH(10, 6, 64, 2, 4, 2, 15);
         case 4:
             return MFL_LAUNCH(10, 4, 64, 2, 4, 2, 7);
         case 15:  // a few rows per expert (decode): the weights are all the traffic; flat 64 x 128 tiles,
                   // 6 stages of 24 KiB
-            return MFL_LAUNCH(2, 4, 64, 6, 2, 4, 3);
+            return MFL_LAUNCH(2, 4, 64, 6, 2, 4, 11);
         case 10:  // thin output of a row-grouped product: 128 rows x 64 columns, 6 stages of 24 KiB
             return MFL_LAUNCH(4, 2, 64, 6, 4, 1, 3);
         case 11:  // dW with a thin side: 64 x 64 tiles (an expert's reduction is spread over as many
                   // workgroups as its wide side has 64-column slices), 8 stages of 16 KiB
             return MFL_LAUNCH(2, 2, 64, 8, 2, 2, 4);
         default:
-            return MFL_LAUNCH(8, 8, 64, 2, 2, 4, 7);
+            return MFL_LAUNCH(8, 8, 64, 2, 2, 4, 15);
     }
 #undef MFL_LAUNCH
 }
 
 }  // namespace
 
+namespace {
+
+// Checks the fusion request of a forward product and translates it for the kernel.
+// Returns MFL_ERR_UNSUPPORTED for what the pipelined kernels do not take.
+int make_fusion(const GemmFusion *f, int K, bool nf4, FwdFusion *out) {
+    *out = FwdFusion{nullptr, 1, nullptr, Nf4Params{nullptr, nullptr, 0}, nullptr, nullptr};
+    if (f == nullptr) return MFL_OK;
+    if (f->row_idx != nullptr) {
+        // the kernel addresses the source rows with 32-bit byte offsets
+        if (f->idx_div <= 0 || f->src_rows <= 0 || f->src_rows * (int64_t)K * 2 > 0xffffffffll)
+            return MFL_ERR_UNSUPPORTED;
+        out->row_idx = f->row_idx;
+        out->idx_div = f->idx_div;
+    }
+    if (f->w2 != nullptr) {
+        out->b2 = f->w2;
+        out->c_e = f->e_out;
+        out->c_g = f->g_out;
+        if (!aligned(f->w2, nf4 ? 4 : 16) || !aligned(f->e_out, 16) || !aligned(f->g_out, 16)) return MFL_ERR_UNSUPPORTED;
+        if (nf4) {
+            int shift = 0;
+            while ((1 << shift) < f->blocksize_2) ++shift;
+            if (f->blocksize_2 < 8 || f->code16_2 == nullptr || f->absmax_2 == nullptr) return MFL_ERR_UNSUPPORTED;
+            out->nf4_2 = Nf4Params{f->code16_2, f->absmax_2, shift};
+        }
+    }
+    return MFL_OK;
+}
+
+}  // namespace
+
 int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
-                   int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream) {
+                   int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream,
+                   const GemmFusion *fusion) {
     if (g_pipe_config < 0 || E > kMaxTableExperts) return MFL_ERR_UNSUPPORTED;
     if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, 16)) return MFL_ERR_UNSUPPORTED;
     if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
     if (mode != MODE_DW && (K % 8 != 0 || K < 8 || N % 8 != 0 || N < 8)) return MFL_ERR_UNSUPPORTED;
     if (mode == MODE_DW && (N % 8 != 0 || K % 8 != 0 || N < 8 || K < 8)) return MFL_ERR_UNSUPPORTED;
+    FwdFusion fu;
+    if (fusion != nullptr) {
+        if (mode != MODE_FWD) return MFL_ERR_UNSUPPORTED;
+        if (fusion->w2 != nullptr && (out_dtype != MFL_BF16 || accumulate || alpha != 1.0f)) return MFL_ERR_UNSUPPORTED;
+        const int rc = make_fusion(fusion, K, false, &fu);
+        if (rc) return rc;
+    }
     if (mode != MODE_DW && R <= 0) return MFL_OK;
-    return dispatch_pipe(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, nullptr, stream);
+    return dispatch_pipe(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, nullptr,
+                         fusion ? &fu : nullptr, stream);
 }
 
 int gemm_nf4_pipe(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
                   const void *m_sizes, int ms_i64, void *y, int64_t R, int N, int K, int E, int out_dtype,
-                  hipStream_t stream) {
+                  hipStream_t stream, const GemmFusion *fusion) {
     if (g_pipe_config < 0 || E > kMaxTableExperts) return MFL_ERR_UNSUPPORTED;
     int shift = 0;
     while ((1 << shift) < blocksize) ++shift;
@@ -811,12 +987,19 @@ int gemm_nf4_pipe(const void *x, const uint8_t *wq, const float *code16, const f
     if (K % 64 != 0 || N % 8 != 0 || N < 8 || blocksize < 8) return MFL_ERR_UNSUPPORTED;
     // With a handful of rows per expert the 128 x 128 tiles of the register-staged kernel spread
     // the weight stream over more workgroups; measured cross-over near 32 rows per expert.
-    if (R < (int64_t)32 * E) return MFL_ERR_UNSUPPORTED;
+    if (R < (int64_t)32 * E && fusion == nullptr) return MFL_ERR_UNSUPPORTED;
     if (!aligned(x, 16) || !aligned(wq, 4) || !aligned(y, 16)) return MFL_ERR_UNSUPPORTED;
     if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
+    FwdFusion fu;
+    if (fusion != nullptr) {
+        if (fusion->w2 != nullptr && out_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+        const int rc = make_fusion(fusion, K, true, &fu);
+        if (rc) return rc;
+    }
     if (R <= 0) return MFL_OK;
     const Nf4Params nf4 = {code16, absmax, shift};
-    return dispatch_pipe(MODE_FWD, x, wq, m_sizes, ms_i64, y, R, N, K, E, out_dtype, 1.0f, 0, &nf4, stream);
+    return dispatch_pipe(MODE_FWD, x, wq, m_sizes, ms_i64, y, R, N, K, E, out_dtype, 1.0f, 0, &nf4,
+                         fusion ? &fu : nullptr, stream);
 }
 
 }  // namespace mfl

@@ -1,8 +1,8 @@
 // Fused NF4 grouped GEMM for decode-sized batches (a few rows per expert): the packed weights are
 // all the traffic, so the kernel is built around streaming them.
 //
-// A workgroup (4 waves) owns 32 rows of one expert and 4 * CB * 32 output columns; every wave owns
-// CB 32-column blocks and works alone: no LDS stage, no barrier in the reduction loop.
+// A workgroup (4 waves) owns 32 rows of one expert and 128 output columns; every wave owns one
+// 32-column block and works alone: no LDS stage, no barrier in the reduction loop.
 //   * v_mfma_f32_32x32x16_bf16 takes from lane l of its first operand 8 reduction elements of
 //     column l % 32 (group l / 32): 8 weights = one packed dword.  The reduction index is
 //     permuted (the same way for both operands, which leaves the sum unchanged) so that a lane
@@ -13,6 +13,12 @@
 //   * loads run DEPTH steps ahead in registers, and two or three workgroups share a CU: tens of
 //     KiB of packed weights in flight per CU.
 // The accumulator of a lane holds output row l % 32, columns 8g + 4*(l / 32) + {0..3}.
+//
+// Two fusions with the neighbours of the product in the sparse MLP block:
+//   * gathered rows: row i of x is row row_idx[i] / idx_div of the token matrix;
+//   * gated linear unit: the wave multiplies the same rows with the same columns of a second
+//     weight matrix (gate = first, up = second) and stores silu(gate) * up, rounded the way the
+//     separate kernels round.
 #include "common.h"
 #include "gemm.h"
 
@@ -22,18 +28,28 @@ namespace {
 
 constexpr int kDepth = 4;  // steps in flight
 
-template <int CB, typename TO>
-__global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restrict__ x, const uint8_t *__restrict__ wq,
-                                                         const float *__restrict__ code16,
-                                                         const float *__restrict__ absmax, int bs_shift,
+struct Nf4Matrix {
+    const uint8_t *wq;
+    const float *code16;
+    const float *absmax;
+    int bs_shift;
+};
+
+template <bool GLU, typename TO>
+__global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restrict__ x,
+                                                         const int32_t *__restrict__ row_idx, int idx_div,
+                                                         Nf4Matrix w0, Nf4Matrix w1,
                                                          const void *__restrict__ m_sizes, int ms_i64,
-                                                         TO *__restrict__ y, int64_t R, int N, int K, int E,
+                                                         TO *__restrict__ y, TO *__restrict__ e_out,
+                                                         TO *__restrict__ g_out, int64_t R, int N, int K, int E,
                                                          int tiles_n) {
-    __shared__ float lut[16];
+    constexpr int CB = GLU ? 2 : 1;  // products per wave: block cb uses weight matrix cb
+    __shared__ float lut[16 * CB];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
-    if (tid < 16) lut[tid] = code16[tid];
+    if (tid < 16) lut[tid] = w0.code16[tid];
+    if (GLU && tid >= 16 && tid < 32) lut[tid] = w1.code16[tid - 16];
 
     // ---- which 32 rows: row tile blockIdx.x / tiles_n in the order of the experts
     const int ct = blockIdx.x % tiles_n, rt = blockIdx.x / tiles_n;
@@ -77,16 +93,20 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
     if (rows <= 0) return;
 
     // ---- this lane's sources
-    const int j0 = (ct * 4 + wave) * CB * 32;  // first column of the wave
-    int64_t w_el[CB];                          // first weight of the lane in step 0, per column block
-#pragma unroll
-    for (int cb = 0; cb < CB; ++cb) {
-        int col = j0 + cb * 32 + n;
+    const int j0 = (ct * 4 + wave) * 32;  // first column of the wave
+    int64_t w_el;                         // first weight of the lane in step 0
+    {
+        int col = j0 + n;
         if (col >= N) col = N - 1;  // loaded, multiplied, never stored
-        w_el[cb] = ((int64_t)expert * N + col) * K + h * 32;
+        w_el = ((int64_t)expert * N + col) * K + h * 32;
     }
-    const bf16_t *x_row = x + (int64_t)(i0 + (n < rows ? n : rows - 1)) * K + h * 32;
+    int64_t src_row = i0 + (n < rows ? n : rows - 1);
+    if (row_idx != nullptr) src_row = (uint32_t)row_idx[src_row] / (uint32_t)idx_div;
+    const bf16_t *x_row = x + src_row * K + h * 32;
     const int KT = K / 64;
+    const uint8_t *wq_of[2] = {w0.wq, w1.wq};
+    const float *am_of[2] = {w0.absmax, w1.absmax};
+    const int shift_of[2] = {w0.bs_shift, w1.bs_shift};
 
     struct Step {
         uint4_t w[CB];
@@ -96,13 +116,13 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
     auto load = [&](int kt, Step &s) {
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
-            const int64_t el = w_el[cb] + (int64_t)kt * 64;
-            s.w[cb] = *(const uint4_t *)(wq + (el >> 1));
-            if (bs_shift >= 5) {
-                s.am[cb][0] = absmax[el >> bs_shift];
+            const int64_t el = w_el + (int64_t)kt * 64;
+            s.w[cb] = *(const uint4_t *)(wq_of[cb] + (el >> 1));
+            if (shift_of[cb] >= 5) {
+                s.am[cb][0] = am_of[cb][el >> shift_of[cb]];
             } else {
 #pragma unroll
-                for (int u = 0; u < 4; ++u) s.am[cb][u] = absmax[(el + 8 * u) >> bs_shift];
+                for (int u = 0; u < 4; ++u) s.am[cb][u] = am_of[cb][(el + 8 * u) >> shift_of[cb]];
             }
         }
         const uint4_t *px = (const uint4_t *)(x_row + kt * 64);
@@ -127,12 +147,12 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 const uint32_t w = s.w[cb][ks];
-                const float am = bs_shift >= 5 ? s.am[cb][0] : s.am[cb][ks];
+                const float am = shift_of[cb] >= 5 ? s.am[cb][0] : s.am[cb][ks];
                 bf16x8 wf;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const uint32_t nib = (w >> (8 * (j >> 1) + ((j & 1) ? 0 : 4))) & 15u;
-                    wf[j] = (bf16_t)(lut[nib] * am);
+                    wf[j] = (bf16_t)(lut[16 * cb + nib] * am);
                 }
                 acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xa.v, acc[cb], 0, 0, 0);
             }
@@ -155,26 +175,38 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
 
     // ---- output: lane = row n, 4 consecutive columns per group
     if (n < rows) {
-        TO *y_row = y + (int64_t)(i0 + n) * N;
+        const int64_t o_row = (int64_t)(i0 + n) * N;
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
+        for (int g = 0; g < 4; ++g) {
+            const int col = j0 + 8 * g + 4 * h;
+            if (col >= N) continue;  // N is a multiple of 8: a group of 4 is inside or outside as a whole
+            if constexpr (GLU) {
+                union {
+                    bf16_t e[4];
+                    uint2_t v;
+                } pe, pg, ph;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int col = j0 + cb * 32 + 8 * g + 4 * h;
-                if (col >= N) continue;  // N is a multiple of 8: a group of 4 is inside or outside as a whole
-                if (sizeof(TO) == 2) {
-                    union {
-                        bf16_t e[4];
-                        uint2_t v;
-                    } pk;
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) pk.e[u] = (bf16_t)acc[cb][4 * g + u];
-                    *(uint2_t *)((bf16_t *)y_row + col) = pk.v;
-                } else {
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) y_row[col + u] = from_f32<TO>(acc[cb][4 * g + u]);
+                for (int u = 0; u < 4; ++u) {
+                    pe.e[u] = (bf16_t)acc[0][4 * g + u];
+                    pg.e[u] = (bf16_t)acc[1][4 * g + u];
+                    ph.e[u] = silu_fwd_one<bf16_t>(pe.e[u], pg.e[u]);
                 }
+                *(uint2_t *)((bf16_t *)y + o_row + col) = ph.v;
+                if (e_out) *(uint2_t *)((bf16_t *)e_out + o_row + col) = pe.v;
+                if (g_out) *(uint2_t *)((bf16_t *)g_out + o_row + col) = pg.v;
+            } else if (sizeof(TO) == 2) {
+                union {
+                    bf16_t e[4];
+                    uint2_t v;
+                } pk;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) pk.e[u] = (bf16_t)acc[0][4 * g + u];
+                *(uint2_t *)((bf16_t *)y + o_row + col) = pk.v;
+            } else {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) y[o_row + col + u] = from_f32<TO>(acc[0][4 * g + u]);
             }
+        }
     }
 }
 
@@ -182,7 +214,7 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
 
 int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
                     const void *m_sizes, int ms_i64, void *y, int64_t R, int N, int K, int E, int out_dtype,
-                    hipStream_t stream) {
+                    hipStream_t stream, const GemmFusion *fusion) {
     // decode-sized batches only: with more rows per expert every 32-row tile decodes the weights again
     if (R > (int64_t)32 * E || R <= 0) return R <= 0 ? MFL_OK : MFL_ERR_UNSUPPORTED;
     int shift = 0;
@@ -190,19 +222,46 @@ int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const
     if (K % 64 != 0 || N % 8 != 0 || N < 8 || blocksize < 8) return MFL_ERR_UNSUPPORTED;
     if (!aligned(x, 16) || !aligned(wq, 16) || !aligned(y, 16)) return MFL_ERR_UNSUPPORTED;
     if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
-    constexpr int CB = 1;  // 128 columns per workgroup: the most workgroups per expert (two blocks per wave: slower)
-    const int tiles_n = ceil_div(N, 4 * CB * 32);
+    const Nf4Matrix w0 = {wq, code16, absmax, shift};
+    Nf4Matrix w1 = w0;
+    const int32_t *row_idx = nullptr;
+    int idx_div = 1;
+    void *e_out = nullptr, *g_out = nullptr;
+    bool glu = false;
+    if (fusion != nullptr) {
+        if (fusion->row_idx != nullptr) {
+            if (fusion->idx_div <= 0 || fusion->src_rows <= 0) return MFL_ERR_UNSUPPORTED;
+            row_idx = fusion->row_idx;
+            idx_div = fusion->idx_div;
+        }
+        if (fusion->w2 != nullptr) {
+            int shift2 = 0;
+            while ((1 << shift2) < fusion->blocksize_2) ++shift2;
+            if (out_dtype != MFL_BF16 || fusion->blocksize_2 < 8 || !fusion->code16_2 || !fusion->absmax_2 ||
+                !aligned(fusion->w2, 16) || !aligned(fusion->e_out, 8) || !aligned(fusion->g_out, 8))
+                return MFL_ERR_UNSUPPORTED;
+            glu = true;
+            w1 = Nf4Matrix{(const uint8_t *)fusion->w2, fusion->code16_2, fusion->absmax_2, shift2};
+            e_out = fusion->e_out;
+            g_out = fusion->g_out;
+        }
+    }
+    // 128 columns per workgroup: the most workgroups per expert (two blocks per wave: slower)
+    const int tiles_n = ceil_div(N, 128);
     const int64_t row_tiles = R / 32 + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / 32)
     const int64_t grid = row_tiles * tiles_n;
     if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
-    if (out_dtype == MFL_BF16)
-        nf4_decode_kernel<CB, bf16_t><<<(unsigned)grid, 256, 0, stream>>>((const bf16_t *)x, wq, code16, absmax, shift,
-                                                                         m_sizes, ms_i64, (bf16_t *)y, R, N, K, E,
-                                                                         tiles_n);
+    const bf16_t *px = (const bf16_t *)x;
+    if (glu)
+        nf4_decode_kernel<true, bf16_t><<<(unsigned)grid, 256, 0, stream>>>(
+            px, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out, R, N, K, E,
+            tiles_n);
+    else if (out_dtype == MFL_BF16)
+        nf4_decode_kernel<false, bf16_t><<<(unsigned)grid, 256, 0, stream>>>(
+            px, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (bf16_t *)y, nullptr, nullptr, R, N, K, E, tiles_n);
     else
-        nf4_decode_kernel<CB, float><<<(unsigned)grid, 256, 0, stream>>>((const bf16_t *)x, wq, code16, absmax, shift,
-                                                                        m_sizes, ms_i64, (float *)y, R, N, K, E,
-                                                                        tiles_n);
+        nf4_decode_kernel<false, float><<<(unsigned)grid, 256, 0, stream>>>(
+            px, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (float *)y, nullptr, nullptr, R, N, K, E, tiles_n);
     return launch_status();
 }
 

@@ -33,6 +33,12 @@ _SIGNATURES = {
     "mfl_gemm_dx": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "mfl_gemm_dw": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "mfl_gemm_fwd_nf4": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
+    "mfl_gemm_fwd_gather": (_i, [_vp, _i64, _vp, _i, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
+    "mfl_gemm_fwd_nf4_gather": (_i, [_vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i,
+                                     _vp]),
+    "mfl_glu_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp]),
+    "mfl_glu_fwd_nf4": (_i, [_vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _i64,
+                             _i, _i, _i, _i, _vp]),
     "mfl_nf4_dequant": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _vp]),
     "mfl_dequant_blockwise_u8": (_i, [_vp, _vp, _vp, _i, _f, _vp, _i64, _vp]),
     "mfl_nf4_quant": (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _vp]),

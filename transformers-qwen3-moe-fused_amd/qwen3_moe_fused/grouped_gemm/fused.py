@@ -1,0 +1,159 @@
+"""Forward products fused with their neighbours in the sparse MLP block.
+
+The reference keeps these steps apart and names both fusions as possible
+(qwen3_moe_fused/modular_qwen3_moe_fused.py:100-101 "fuse a sort and a MoeFusedLinear layer",
+:105 "fuse gate_h and up_h"):
+
+* gathered rows: ``y = grouped_gemm_forward(x_src[row_idx // idx_div], w, m_sizes)`` without
+  writing the gathered matrix (with ``row_idx = sort_idx``, ``idx_div = num_selected`` this is the
+  replicate-and-sort of :95-103 folded into the GEMM's operand load);
+* gated linear unit: ``silu(x @ w_gate^T) * (x @ w_up^T)`` in one kernel (:106-108), with the
+  rounding steps of the separate kernels, so the result is bit-identical to them.
+
+Each wrapper calls the fused entry point and, when the library answers that it has no fused
+kernel for the request (status ``UNSUPPORTED``: odd sizes, fp32, ...), runs the separate HIP
+kernels instead.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from ..kernels.routing import _gather as gather_kernel
+from ..kernels.silu_mul import silu_mul_forward
+from ..quantize.nf4 import resolve_absmax
+from ._common import check_operands, is_int_tensor
+from .forward import grouped_gemm_forward
+from .forward_4bit import grouped_gemm_forward_4bit
+
+UNSUPPORTED = -6  # MFL_ERR_UNSUPPORTED
+
+
+def _gather(x_src: torch.Tensor, row_idx: torch.Tensor, idx_div: int) -> torch.Tensor:
+    return gather_kernel(x_src, row_idx, idx_div, None)
+
+
+def _check_gather(x_src: torch.Tensor, row_idx: Optional[torch.Tensor], idx_div: int) -> int:
+    """Number of rows of the (virtual) left operand."""
+    assert x_src.ndim == 2
+    if row_idx is None:
+        return x_src.shape[0]
+    assert row_idx.dtype == torch.int32 and row_idx.ndim == 1 and row_idx.is_contiguous()
+    assert row_idx.device == x_src.device and idx_div >= 1
+    return row_idx.numel()
+
+
+def _nf4_args(w_quant: torch.Tensor, state, x: torch.Tensor, k: int):
+    assert state.quant_type == "nf4"
+    blocksize = int(state.blocksize)
+    assert blocksize > 0 and blocksize & (blocksize - 1) == 0, "blocksize must be a power of two"
+    code = state.code
+    assert code.dtype == torch.float32
+    absmax = resolve_absmax(state)
+    for t in (w_quant, code, absmax):
+        assert t.device == x.device and t.is_contiguous()
+    assert is_int_tensor(w_quant) and len(state.shape) == 3
+    experts, n, k_w = state.shape
+    assert k_w == k and k % 2 == 0
+    total = experts * n * k
+    assert total % blocksize == 0 and w_quant.numel() == total // 2 and absmax.numel() == total // blocksize
+    return code, absmax, blocksize, experts, n
+
+
+def grouped_gemm_forward_gathered(x_src: torch.Tensor, row_idx: torch.Tensor, idx_div: int, w: torch.Tensor,
+                                  m_sizes: torch.Tensor, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``grouped_gemm_forward(x_src[row_idx // idx_div], w, m_sizes, dtype)``."""
+    check_operands(m_sizes, x_src, w)
+    rows = _check_gather(x_src, row_idx, idx_div)
+    assert w.ndim == 3
+    experts, n, k = w.shape
+    assert x_src.shape[1] == k and m_sizes.numel() == experts
+    y = torch.empty((rows, n), device=x_src.device, dtype=x_src.dtype if dtype is None else dtype)
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_gemm_fwd_gather(_lib.ptr(x_src), x_src.shape[0], _lib.ptr(row_idx), idx_div, _lib.ptr(w),
+                                        _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(y), rows, n, k, experts,
+                                        _lib.dtype_code(x_src.dtype), _lib.dtype_code(y.dtype), _lib.stream())
+    if rc == UNSUPPORTED:
+        return grouped_gemm_forward(_gather(x_src, row_idx, idx_div), w, m_sizes, dtype)
+    _lib.check(rc, "mfl_gemm_fwd_gather")
+    return y
+
+
+def grouped_gemm_forward_4bit_gathered(x_src: torch.Tensor, row_idx: torch.Tensor, idx_div: int,
+                                       w_quant: torch.Tensor, w_quant_state, m_sizes: torch.Tensor,
+                                       dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``grouped_gemm_forward_4bit(x_src[row_idx // idx_div], w_quant, w_quant_state, m_sizes, dtype)``."""
+    assert x_src.is_cuda and x_src.is_contiguous() and m_sizes.is_contiguous() and is_int_tensor(m_sizes)
+    rows = _check_gather(x_src, row_idx, idx_div)
+    k = x_src.shape[1]
+    code, absmax, blocksize, experts, n = _nf4_args(w_quant, w_quant_state, x_src, k)
+    assert m_sizes.numel() == experts
+    y = torch.empty((rows, n), device=x_src.device, dtype=x_src.dtype if dtype is None else dtype)
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_gemm_fwd_nf4_gather(_lib.ptr(x_src), x_src.shape[0], _lib.ptr(row_idx), idx_div,
+                                            _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), blocksize,
+                                            _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(y), rows, n, k, experts,
+                                            _lib.dtype_code(x_src.dtype), _lib.dtype_code(y.dtype), _lib.stream())
+    if rc == UNSUPPORTED:
+        return grouped_gemm_forward_4bit(_gather(x_src, row_idx, idx_div), w_quant, w_quant_state, m_sizes, dtype)
+    _lib.check(rc, "mfl_gemm_fwd_nf4_gather")
+    return y
+
+
+def grouped_glu_forward(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, m_sizes: torch.Tensor,
+                        row_idx: Optional[torch.Tensor] = None, idx_div: int = 1,
+                        return_products: bool = False):
+    """``h = silu(e) * g`` with ``e = grouped_gemm_forward(xg, w_gate, m_sizes)``,
+    ``g = grouped_gemm_forward(xg, w_up, m_sizes)`` and ``xg = x`` or, with ``row_idx``,
+    ``x[row_idx // idx_div]``.  Returns ``h`` or ``(h, e, g)``."""
+    check_operands(m_sizes, x, w_gate, w_up)
+    rows = _check_gather(x, row_idx, idx_div)
+    assert w_gate.ndim == 3 and w_up.shape == w_gate.shape
+    experts, n, k = w_gate.shape
+    assert x.shape[1] == k and m_sizes.numel() == experts
+    h = torch.empty((rows, n), device=x.device, dtype=x.dtype)
+    e = torch.empty_like(h) if return_products else None
+    g = torch.empty_like(h) if return_products else None
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_glu_fwd(_lib.ptr(x), x.shape[0], _lib.ptr(row_idx), idx_div, _lib.ptr(w_gate), _lib.ptr(w_up),
+                                _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(h), _lib.ptr(e), _lib.ptr(g), rows, n,
+                                k, experts, _lib.dtype_code(x.dtype), _lib.stream())
+    if rc == UNSUPPORTED:
+        xg = x if row_idx is None else _gather(x, row_idx, idx_div)
+        e = grouped_gemm_forward(xg, w_gate, m_sizes)
+        g = grouped_gemm_forward(xg, w_up, m_sizes)
+        h = silu_mul_forward(e, g)
+    else:
+        _lib.check(rc, "mfl_glu_fwd")
+    return (h, e, g) if return_products else h
+
+
+def grouped_glu_forward_4bit(x: torch.Tensor, gate_quant: torch.Tensor, gate_state, up_quant: torch.Tensor, up_state,
+                             m_sizes: torch.Tensor, row_idx: Optional[torch.Tensor] = None, idx_div: int = 1,
+                             return_products: bool = False):
+    """``grouped_glu_forward`` with NF4 gate and up weights, each with its own quant state."""
+    assert x.is_cuda and x.is_contiguous() and m_sizes.is_contiguous() and is_int_tensor(m_sizes)
+    rows = _check_gather(x, row_idx, idx_div)
+    k = x.shape[1]
+    code_g, absmax_g, bs_g, experts, n = _nf4_args(gate_quant, gate_state, x, k)
+    code_u, absmax_u, bs_u, experts_u, n_u = _nf4_args(up_quant, up_state, x, k)
+    assert (experts_u, n_u) == (experts, n) and m_sizes.numel() == experts
+    h = torch.empty((rows, n), device=x.device, dtype=x.dtype)
+    e = torch.empty_like(h) if return_products else None
+    g = torch.empty_like(h) if return_products else None
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_glu_fwd_nf4(_lib.ptr(x), x.shape[0], _lib.ptr(row_idx), idx_div,
+                                    _lib.ptr(gate_quant), _lib.ptr(code_g), _lib.ptr(absmax_g), bs_g,
+                                    _lib.ptr(up_quant), _lib.ptr(code_u), _lib.ptr(absmax_u), bs_u,
+                                    _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(h), _lib.ptr(e), _lib.ptr(g), rows,
+                                    n, k, experts, _lib.dtype_code(x.dtype), _lib.stream())
+    if rc == UNSUPPORTED:
+        xg = x if row_idx is None else _gather(x, row_idx, idx_div)
+        e = grouped_gemm_forward_4bit(xg, gate_quant, gate_state, m_sizes)
+        g = grouped_gemm_forward_4bit(xg, up_quant, up_state, m_sizes)
+        h = silu_mul_forward(e, g)
+    else:
+        _lib.check(rc, "mfl_glu_fwd_nf4")
+    return (h, e, g) if return_products else h
