@@ -27,20 +27,25 @@ def _ulp_diff_bf16(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
     return np.abs(key(a_bits) - key(b_bits))
 
 
+def _two_roundings_close(d: np.ndarray) -> None:
+    """bf16 steps between two results of `round(round(silu(e)) * x)`: at most two, and rarely any."""
+    assert d.max() <= 2
+    assert (d > 1).sum() <= max(1, 1e-5 * d.size) and (d > 0).sum() <= max(2, 1e-3 * d.size)
+
+
 @pytest.mark.parametrize("shape", [(32768, 768), (91, 3), (1, 1), (1000, 7)])
 def test_silu_mul_bf16(shape):
     g = gen(shape[0])
     e, gg, dh = (randn(shape, g, 2.0, torch.bfloat16) for _ in range(3))
     h = silu_mul_forward(e.to(DEV), gg.to(DEV))
     h_ref = oracle.silu_mul_fwd_bf16(_bits(e), _bits(gg))
-    # same rounding chain; exp() may differ by an ulp between CPU and GPU, which can move a
-    # bf16 result by at most one step
-    d = _ulp_diff_bf16(_bits(h), h_ref)
-    assert d.max() <= 1 and (d > 0).mean() < 1e-3
+    # same rounding chain; the sigmoid differs by a few fp32 ulps between CPU and GPU, which now
+    # and then moves silu(e) by one bf16 step, and the rounding of the product can add one more
+    _two_roundings_close(_ulp_diff_bf16(_bits(h), h_ref))
     de, dg = silu_mul_backward(dh.to(DEV), e.to(DEV), gg.to(DEV))
     h_r, de_r, dg_r = oracle.silu_mul_bwd_bf16(_bits(dh), _bits(e), _bits(gg))
     assert _ulp_diff_bf16(_bits(de), de_r).max() <= 2 and (_ulp_diff_bf16(_bits(de), de_r) > 0).mean() < 5e-3
-    assert _ulp_diff_bf16(_bits(dg), dg_r).max() <= 1
+    _two_roundings_close(_ulp_diff_bf16(_bits(dg), dg_r))  # dg = silu(e) * dh: two roundings, like h
     # in-place variant: (dh, e, g) <- (h, de, dg)
     a, b, c = dh.to(DEV).clone(), e.to(DEV).clone(), gg.to(DEV).clone()
     silu_mul_backward_inplace(a, b, c)

@@ -261,3 +261,55 @@ def test_4bit_layer_and_fast_lora_on_nf4_base():
     check_close(y1, to_np32(y2), 2e-2, 2e-2, "fast_lora nf4 vs dense")
     for a, b, n in zip(g_q, g_d, ("dx", "dAg", "dBg", "dAu", "dBu", "dAw", "dBw")):
         check_close(a, to_np32(b), 2e-2, 2e-2 * float(b.abs().max() + 1e-12), n)
+
+
+def _grads_close(a, b, what):
+    a, b = a.float(), b.float()
+    err = (a - b).abs().max().item() / max(b.abs().max().item(), 1e-30)
+    assert err <= 2e-2, f"{what}: normalised max error {err:.3e}"
+
+
+@pytest.mark.parametrize("T,E,k,H,I", [(384, 16, 4, 256, 96), (40, 64, 8, 128, 64)])
+def test_fused_front_of_block_matches_module_by_module_path(T, E, k, H, I):
+    cfg = _config(E, k, H, I)
+    blk = _block(cfg, torch.bfloat16, 11).to(DEV)
+    hidden = randn((1, T, H), gen(T), 1.0, torch.bfloat16).to(DEV)
+    gout = randn((1, T, H), gen(T + 1), 1.0, torch.bfloat16).to(DEV)
+    results = []
+    for fuse in (True, False):
+        blk.fuse_front = fuse
+        blk.zero_grad(set_to_none=True)
+        h = hidden.clone().requires_grad_()
+        out, logits = blk(h)
+        out.backward(gout)
+        results.append((out.detach(), h.grad, {n: p.grad.clone() for n, p in blk.named_parameters()}))
+    (o1, g1, p1), (o2, g2, p2) = results
+    assert torch.equal(o1, o2), "same kernels' arithmetic, same roundings"
+    _grads_close(g1, g2, "d hidden")
+    for n in p1:
+        _grads_close(p1[n], p2[n], n)
+    # inference: no products are kept, same output
+    blk.fuse_front = True
+    with torch.no_grad():
+        o3, _ = blk(hidden)
+    assert torch.equal(o3, o1)
+
+
+def test_fused_front_of_block_with_4bit_projections():
+    T, E, k, H, I = 96, 8, 2, 128, 64
+    cfg = _config(E, k, H, I)
+    blk = _block(cfg, torch.bfloat16, 13)
+    for name, (i, o) in {"gate_proj": (H, I), "up_proj": (H, I), "down_proj": (I, H)}.items():
+        setattr(blk, name, MoeFusedLinear4bit(i, o, E, weight=getattr(blk, name).weight, quant_type="nf4"))
+    blk = blk.to(DEV)
+    hidden = randn((1, T, H), gen(3), 1.0, torch.bfloat16).to(DEV)
+    gout = randn((1, T, H), gen(4), 1.0, torch.bfloat16).to(DEV)
+    outs = []
+    for fuse in (False, True, True):  # the first call attaches the quant states; fused from the second on
+        blk.fuse_front = fuse
+        h = hidden.clone().requires_grad_()
+        out, _ = blk(h)
+        out.backward(gout)
+        outs.append((out.detach(), h.grad))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[1][0], outs[2][0])
+    _grads_close(outs[1][1], outs[0][1], "d hidden, 4-bit")

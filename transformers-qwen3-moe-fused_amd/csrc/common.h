@@ -32,7 +32,13 @@ __device__ __forceinline__ T from_f32(float v) {
     return (T)v;  // bf16/f16: one round-to-nearest-even (v_cvt_pk_bf16_f32 on gfx950)
 }
 
-__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
+// 1 / (1 + 2^(-x log2 e)) on the hardware exp2 and reciprocal instructions (about an ulp of
+// error each, far below the bf16 rounding that follows).  The library's expf and an IEEE
+// division cost about ten times as many instructions, which made the SiLU as expensive as its
+// memory traffic.  Large |x|: 2^t overflows to +inf (sigmoid 0) or flushes to 0 (sigmoid 1).
+__device__ __forceinline__ float sigmoid_f32(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896341f));
+}
 
 // h = silu(e) * g with the rounding chain of the reference (qwen3_moe_fused/kernels/silu_mul.py:34-39):
 // silu in fp32, rounded to the storage type, then the product in the storage type.

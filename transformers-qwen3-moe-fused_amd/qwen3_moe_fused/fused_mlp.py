@@ -1,0 +1,96 @@
+"""Front half of the sparse MLP block as one differentiable op:
+
+    h = silu(xg @ w_gate[e]^T) * (xg @ w_up[e]^T),   xg = tokens[sort_idx // num_selected]
+
+i.e. qwen3_moe_fused/modular_qwen3_moe_fused.py:95-108 (replicate, sort, gate_proj, up_proj,
+SiLU-mul) in a single kernel launch; the reference names both fusions as possible (:101, :105).
+The forward keeps the two products only when a gradient will be asked for; the backward
+re-gathers the token rows instead of keeping a (rows, hidden) copy alive.
+"""
+from __future__ import annotations
+
+import torch
+
+from .grouped_gemm.backward_dw import grouped_gemm_backward_dw
+from .grouped_gemm.forward_transposed import grouped_gemm_forward_transposed
+from .grouped_gemm.fused import grouped_glu_forward, grouped_glu_forward_4bit
+from .kernels.routing import _combine, _gather
+from .kernels.silu_mul import silu_mul_backward
+from .quantize.nf4 import dequantize_nf4
+
+
+class _GluGathered(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, tokens, w_gate, w_up, m_sizes, sort_idx, inv_sort_idx, k):
+        need = any(ctx.needs_input_grad[:3])
+        out = grouped_glu_forward(tokens, w_gate, w_up, m_sizes, sort_idx, k, return_products=need)
+        if not need:
+            return out
+        h, e, g = out
+        ctx.save_for_backward(tokens, w_gate, w_up, m_sizes, sort_idx, inv_sort_idx, e, g)
+        ctx.k = k
+        return h
+
+    @staticmethod
+    def backward(ctx, dh):
+        tokens, w_gate, w_up, m_sizes, sort_idx, inv_sort_idx, e, g = ctx.saved_tensors
+        de, dg = silu_mul_backward(dh.contiguous(), e, g)
+        d_tokens = d_gate = d_up = None
+        if ctx.needs_input_grad[0]:
+            # rows of the two input gradients are summed in the GEMM epilogue (one rounding),
+            # then each token's k rows are summed
+            dx = grouped_gemm_forward_transposed(de, w_gate, m_sizes, tokens.dtype)
+            grouped_gemm_forward_transposed(dg, w_up, m_sizes, out=dx, accumulate=True)
+            d_tokens = _combine(dx, inv_sort_idx, None, tokens.shape[0], ctx.k)
+        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            xg = _gather(tokens, sort_idx, ctx.k, None)
+            if ctx.needs_input_grad[1]:
+                d_gate = grouped_gemm_backward_dw(xg, de, m_sizes, w_gate.dtype)
+            if ctx.needs_input_grad[2]:
+                d_up = grouped_gemm_backward_dw(xg, dg, m_sizes, w_up.dtype)
+        return d_tokens, d_gate, d_up, None, None, None, None
+
+
+def moe_fused_glu(tokens: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, m_sizes: torch.Tensor,
+                  sort_idx: torch.Tensor, inv_sort_idx: torch.Tensor, num_selected: int) -> torch.Tensor:
+    """``tokens`` (T, hidden); ``w_gate``, ``w_up`` (E, intermediate, hidden); ``sort_idx`` /
+    ``inv_sort_idx`` (T * num_selected,) int32 as ``get_expert_counts_and_idx`` returns them.
+    Result (T * num_selected, intermediate), rows grouped by expert.  Differentiable in
+    ``tokens``, ``w_gate`` and ``w_up``."""
+    return _GluGathered.apply(tokens, w_gate, w_up, m_sizes, sort_idx, inv_sort_idx, num_selected)
+
+
+class _GluGathered4bit(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, tokens, gate_packed, gate_state, up_packed, up_state, m_sizes, sort_idx, inv_sort_idx, k):
+        need = ctx.needs_input_grad[0]
+        out = grouped_glu_forward_4bit(tokens, gate_packed, gate_state, up_packed, up_state, m_sizes, sort_idx, k,
+                                       return_products=need)
+        if not need:
+            return out
+        h, e, g = out
+        ctx.save_for_backward(gate_packed, up_packed, m_sizes, inv_sort_idx, e, g)
+        ctx.states = (gate_state, up_state)
+        ctx.k, ctx.n_tokens = k, tokens.shape[0]
+        return h
+
+    @staticmethod
+    def backward(ctx, dh):
+        gate_packed, up_packed, m_sizes, inv_sort_idx, e, g = ctx.saved_tensors
+        de, dg = silu_mul_backward(dh.contiguous(), e, g)
+        # frozen weights: only the tokens get a gradient; no fused kernel covers the transposed
+        # product on packed weights, so each matrix is dequantised for it (quantize/layer.py:17-22)
+        dx = grouped_gemm_forward_transposed(de, dequantize_nf4(gate_packed, ctx.states[0], de.dtype), m_sizes, de.dtype)
+        grouped_gemm_forward_transposed(dg, dequantize_nf4(up_packed, ctx.states[1], dg.dtype), m_sizes, out=dx,
+                                        accumulate=True)
+        d_tokens = _combine(dx, inv_sort_idx, None, ctx.n_tokens, ctx.k)
+        return d_tokens, None, None, None, None, None, None, None, None
+
+
+def moe_fused_glu_4bit(tokens: torch.Tensor, gate_weight: torch.Tensor, up_weight: torch.Tensor,
+                       m_sizes: torch.Tensor, sort_idx: torch.Tensor, inv_sort_idx: torch.Tensor,
+                       num_selected: int) -> torch.Tensor:
+    """``moe_fused_glu`` on packed NF4 weights carrying a ``quant_state`` (frozen)."""
+    assert not gate_weight.requires_grad and not up_weight.requires_grad
+    return _GluGathered4bit.apply(tokens, gate_weight.data, gate_weight.quant_state, up_weight.data,
+                                  up_weight.quant_state, m_sizes, sort_idx, inv_sort_idx, num_selected)

@@ -76,14 +76,39 @@ class Qwen3MoeFusedSparseMoeBlock(nn.Module):
         self.up_proj = MoeFusedLinear(self.hidden_size, self.moe_intermediate_size, self.num_experts)
         self.down_proj = MoeFusedLinear(self.moe_intermediate_size, self.hidden_size, self.num_experts)
 
+    # gather + gate_proj + up_proj + SiLU-mul as one kernel when both projections are plain (or
+    # plain 4-bit) expert matrices in bf16; set to False to call the two modules one by one
+    fuse_front = True
+
+    def _fused_front(self, tokens, m_sizes, sort_idx, inv_sort_idx) -> Optional[torch.Tensor]:
+        from .fused_mlp import moe_fused_glu, moe_fused_glu_4bit
+        from .quantize.layer import MoeFusedLinear4bit
+
+        gate, up = self.gate_proj, self.up_proj
+        if tokens.dtype != torch.bfloat16 or type(gate) is not type(up):
+            return None
+        if type(gate) is MoeFusedLinear:
+            if gate.weight.dtype != torch.bfloat16 or up.weight.dtype != torch.bfloat16:
+                return None
+            return moe_fused_glu(tokens, gate.weight, up.weight, m_sizes, sort_idx, inv_sort_idx, self.num_selected)
+        if type(gate) is MoeFusedLinear4bit:
+            for proj in (gate, up):
+                if getattr(proj.weight, "quant_state", None) is None or proj.compute_dtype not in (None, torch.bfloat16):
+                    return None
+            return moe_fused_glu_4bit(tokens, gate.weight, up.weight, m_sizes, sort_idx, inv_sort_idx,
+                                      self.num_selected)
+        return None
+
     def forward(self, hidden_states: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         batch, seq, hidden = hidden_states.shape
         tokens = hidden_states.reshape(batch * seq, hidden).contiguous()
         router_logits, routing_weights, m_sizes, sort_idx, inv_sort_idx = route_tokens(self, tokens)
 
-        # every token once per selected expert, rows grouped by expert
-        x = gather_rows(tokens, sort_idx, self.num_selected, inv_sort_idx)
-        h = silu_mul(self.gate_proj(x, m_sizes), self.up_proj(x, m_sizes))
+        h = self._fused_front(tokens, m_sizes, sort_idx, inv_sort_idx) if self.fuse_front else None
+        if h is None:
+            # every token once per selected expert, rows grouped by expert
+            x = gather_rows(tokens, sort_idx, self.num_selected, inv_sort_idx)
+            h = silu_mul(self.gate_proj(x, m_sizes), self.up_proj(x, m_sizes))
         y = self.down_proj(h, m_sizes)
         out = combine_rows(y, inv_sort_idx, routing_weights, sort_idx)
         return out.view(batch, seq, hidden), router_logits
