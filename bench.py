@@ -245,9 +245,49 @@ def main() -> int:
         with torch.no_grad():
             for tokens in (16, 256, 16384):
                 h5 = torch.randn((1, tokens, HIDDEN), device=dev, dtype=torch.bfloat16)
-                us = _event_us(lambda i: blk(h5), 20 if tokens > 1000 else 50, 3, stream)
-                block[f"tokens_{tokens}"] = {"us": round(us, 1), "tokens_per_s": round(tokens / us * 1e6)}
+                n_it = 20 if tokens > 1000 else 50
+                blk.fuse_front = False                        # gather, gate_proj, up_proj, SiLU-mul one by one
+                us_sep = _event_us(lambda i: blk(h5), n_it, 3, stream)
+                blk.fuse_front = True                         # the default: the four as one kernel
+                us = _event_us(lambda i: blk(h5), n_it, 3, stream)
+                block[f"tokens_{tokens}"] = {"us": round(us, 1), "tokens_per_s": round(tokens / us * 1e6),
+                                             "module_by_module_us": round(us_sep, 1)}
         extra["nf4_sparse_block_fwd_config5"] = block
+        del blk
+        # the same block with bf16 experts at the headline configuration's 4096 tokens, and its front half
+        # (gather + gate_proj + up_proj + SiLU-mul) alone
+        from qwen3_moe_fused.grouped_gemm.fused import grouped_glu_forward
+        from qwen3_moe_fused.kernels.routing import _gather
+        blk = Qwen3MoeFusedSparseMoeBlock(cfg5).to(torch.bfloat16)
+        with torch.no_grad():
+            blk.gate.weight.copy_(torch.randn(blk.gate.weight.shape) * 0.02)
+            blk.gate_proj.weight.copy_(ws[0])
+            blk.up_proj.weight.copy_(ws[1])
+            blk.down_proj.weight.copy_(ws[2].view(E, HIDDEN, INTER))
+        blk = blk.to(dev)
+        toks = [torch.randn((1, TOKENS, HIDDEN), device=dev, dtype=torch.bfloat16) for _ in range(NB)]
+        bf16_block = {}
+        with torch.no_grad():
+            blk.fuse_front = False
+            us_sep = _event_us(lambda i: blk(toks[i % NB]), 50, 30, stream)
+            blk.fuse_front = True
+            us = _event_us(lambda i: blk(toks[i % NB]), 50, 30, stream)
+            bf16_block["block_fwd"] = {"us": round(us, 1), "tokens_per_s": round(TOKENS / us * 1e6),
+                                       "module_by_module_us": round(us_sep, 1)}
+            _, sort_idx2, _ = get_expert_counts_and_idx(selv, E)
+            wg_, wu_ = blk.gate_proj.weight, blk.up_proj.weight
+
+            def front_separate(i):
+                xg = _gather(toks[i % NB][0], sort_idx2, TOPK, None)
+                return silu_mul_forward(grouped_gemm_forward(xg, wg_, m_sizes), grouped_gemm_forward(xg, wu_, m_sizes))
+
+            us_sep = _event_us(front_separate, 50, 5, stream)
+            us = _event_us(lambda i: grouped_glu_forward(toks[i % NB][0], wg_, wu_, m_sizes, sort_idx2, TOPK), 50, 5,
+                           stream)
+            bf16_block["front_half"] = {"fused_us": round(us, 1), "four_kernels_us": round(us_sep, 1),
+                                        "fused_tflops": round(2 * flop / us / 1e6, 1)}
+        extra["bf16_sparse_block_fwd_config2"] = bf16_block
+        del blk, toks
         out["extra"] = extra
 
     if not args.no_cpu_baseline:
