@@ -550,7 +550,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         constexpr int NT_ = NW * 64;
         static_assert(!NF4 || BN * 2 <= NT_, "one thread per half row of the weight stage");
         float *lut = (float *)(smem + S * STAGE_BYTES);
-        const bool nf4_on = tid < BN * 2;
+        // whole waves decode (a wave is 32 stage rows): a wave-uniform condition, no lane mask
+        static_assert((BN * 2) % 64 == 0, "decoding threads are whole waves");
+        const bool nf4_on = wave < BN * 2 / 64;
         const int nf4_row = tid >> 1, nf4_half = tid & 1;
         // GLU: the thread's stage row belongs to the gate or to the up matrix, each with its own
         // packed bytes, absmax, block size and code table
@@ -576,20 +578,22 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 for (int u = 0; u < 4; ++u) r.am[u] = nf4_am[(el + 8 * u) >> nf4_shift];
             }
         };
+        // one packed dword (8 weights, one 16-byte chunk of the stage) of the thread's 32
+        auto nf4_decode_part = [&](int kt, const Nf4Regs &r, int u) {
+            unsigned char *sb = smem + (kt % S) * STAGE_BYTES + SA::kBytes + nf4_row * SB::kRowBytes;
+            const float am = nf4_shift >= 5 ? r.am[0] : r.am[u];
+            bf16x8 v;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t nib = (r.w[u] >> (8 * (j >> 1) + ((j & 1) ? 0 : 4))) & 15u;
+                v[j] = (bf16_t)(nf4_lut[nib] * am);
+            }
+            *(bf16x8 *)(sb + SB::swz(nf4_row, nf4_half * 4 + u) * 16) = v;
+        };
         auto nf4_decode = [&](int kt, const Nf4Regs &r) {
             if (!nf4_on) return;
-            unsigned char *sb = smem + (kt % S) * STAGE_BYTES + SA::kBytes + nf4_row * SB::kRowBytes;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const float am = nf4_shift >= 5 ? r.am[0] : r.am[u];
-                bf16x8 v;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const uint32_t nib = (r.w[u] >> (8 * (j >> 1) + ((j & 1) ? 0 : 4))) & 15u;
-                    v[j] = (bf16_t)(nf4_lut[nib] * am);
-                }
-                *(bf16x8 *)(sb + SB::swz(nf4_row, nf4_half * 4 + u) * 16) = v;
-            }
+            for (int u = 0; u < 4; ++u) nf4_decode_part(kt, r, u);
         };
         auto k_loop_nf4 = [&](auto ta_tag) {
             constexpr int TA = decltype(ta_tag)::value;
@@ -608,8 +612,15 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 __builtin_amdgcn_s_barrier();
                 if (kt + 1 < KT) issue(kt + 1);
                 if (kt + 2 < KT) nf4_load(kt + 2, r_even);
-                if (kt + 1 < KT) nf4_decode(kt + 1, r_odd);
                 const unsigned char *sa = smem + (kt % S) * STAGE_BYTES, *sb = sa + SA::kBytes;
+                // The decode of the next step's weights (vector ALU) is spread over the four
+                // sub-steps, so that it runs under this step's matrix instructions instead of
+                // ahead of them: the two waves of a SIMD move in lock step from barrier to
+                // barrier and would otherwise both decode first and both multiply after.
+                // (Forcing a finer interleave with scheduling barriers, or one straight-line
+                // variant of the step per case, made the register allocator spill.)
+                static_assert(KS == 4, "one packed dword per sub-step");
+                const bool dec = nf4_on && kt + 1 < KT;
                 bf16x8 fa[2][TA], fb[2][TN];
 #pragma unroll
                 for (int bj = 0; bj < TN; ++bj) fb[0][bj] = fo_b.load(sb, bj, 0);
@@ -623,6 +634,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 #pragma unroll
                         for (int t = 0; t < TA; ++t) fa[(ks + 1) & 1][t] = fo_a.load(sa, t, ks + 1);
                     }
+                    if (dec) nf4_decode_part(kt + 1, r_odd, ks);
 #pragma unroll
                     for (int t = 0; t < TA; ++t)
 #pragma unroll
