@@ -83,6 +83,18 @@ int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, cons
                      int blocksize, const void *m_sizes, int m_sizes_dtype, void *y, int64_t R,
                      int N, int K, int E, int in_dtype, int out_dtype, void *stream);
 
+/* Input-gradient product with NF4 weights: dx[m, n] = sum_k w[e(m), k, n] * dy[m, k] with
+ * w (E,K,N) packed as in mfl_gemm_fwd_nf4 (the forward weight (E, out=K, in=N) as stored);
+ * out = alpha * acc (+ out if accumulate).  The reference dequantises the whole matrix for this
+ * product (qwen3_moe_fused/kernels/fast_lora.py:57-63,127-131; quantize/layer.py:17-22 under
+ * autograd).  Returns MFL_ERR_UNSUPPORTED, with nothing enqueued, unless the element type is
+ * bf16, K % 64 == 0, N % 32 == 0, blocksize >= 8, E <= 512 and the pointers are 16-byte
+ * aligned; the caller then dequantises (mfl_nf4_dequant) and calls mfl_gemm_dx. */
+int mfl_gemm_dx_nf4(const void *dy, const uint8_t *wq, const float *code16, const float *absmax,
+                    int blocksize, const void *m_sizes, int m_sizes_dtype, void *dx, int64_t R,
+                    int N, int K, int E, int in_dtype, int out_dtype, float alpha, int accumulate,
+                    void *stream);
+
 /* ---- forward products fused with their neighbours in the sparse MLP block ---------
  * The reference names these fusions as future work (modular_qwen3_moe_fused.py:100-101,105).
  * Each call returns MFL_ERR_UNSUPPORTED, with nothing enqueued, for a request the pipelined

@@ -140,6 +140,20 @@ int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, cons
                          (hipStream_t)stream);
 }
 
+int mfl_gemm_dx_nf4(const void *dy, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                    const void *m_sizes, int m_sizes_dtype, void *dx, int64_t R, int N, int K, int E, int in_dtype,
+                    int out_dtype, float alpha, int accumulate, void *stream) {
+    if (R < 0 || N <= 0 || K <= 0 || E <= 0 || R > 0x7fffffff) return MFL_ERR_SHAPE;
+    if (blocksize < 2 || (blocksize & (blocksize - 1)) != 0) return MFL_ERR_SHAPE;
+    if (N % 2 != 0 || ((int64_t)E * N * K) % blocksize != 0) return MFL_ERR_SHAPE;
+    if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || !itype_ok(m_sizes_dtype)) return MFL_ERR_DTYPE;
+    if (!wq || !code16 || !absmax || !m_sizes || (R > 0 && (!dy || !dx))) return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    return gemm_nf4_pipe_dx(dy, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, dx, R, N, K, E,
+                            out_dtype, alpha, accumulate, (hipStream_t)stream);
+}
+
 /* ---- forward products fused with their neighbours in the sparse MLP block ---- */
 
 namespace {

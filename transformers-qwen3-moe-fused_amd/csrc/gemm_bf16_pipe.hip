@@ -160,9 +160,9 @@ using IC = std::integral_constant<int, V>;
 // partial reduction step (K not a multiple of BK).
 __device__ uint4_t g_zero_chunk = {0u, 0u, 0u, 0u};
 
-// NF4 weights (forward only): b points at the packed bytes; byte i holds element 2i in its high
-// nibble and 2i+1 in its low one; value = code16[nibble] * absmax[element >> bs_shift], rounded
-// once to bf16.
+// NF4 weights (forward and input-gradient products): b points at the packed bytes; byte i holds
+// element 2i in its high nibble and 2i+1 in its low one; value = code16[nibble] *
+// absmax[element >> bs_shift], rounded once to bf16.
 struct Nf4Params {
     const float *code16;
     const float *absmax;
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                                                                   TO *__restrict__ c, int64_t R, int N, int K, int E,
                                                                   float alpha, int accumulate, Nf4Params nf4,
                                                                   FwdFusion fu) {
-    static_assert(!NF4 || (MODE == MODE_FWD && S == 2 && BK == 64), "NF4 weights: forward product, two stages");
+    static_assert(!NF4 || (MODE != MODE_DW && S == 2 && BK == 64), "NF4 weights: row-grouped products, two stages");
     static_assert(!GLU || (MODE == MODE_FWD && WGN % 2 == 0 && sizeof(TO) == 2 && BK == 64),
                   "GLU: forward product, bf16 output, the waves along N split in a gate half and an up half");
     constexpr int BM = MB * 32, BN = NB * 32;
@@ -365,7 +365,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             r_begin = 0, r_end = K;
             lda = K, ldc = N;
             a_tile = (const unsigned char *)(a + (int64_t)i0 * lda);
-            nf4_base = ((int64_t)expert * N + j0) * K;  // first element of the tile's weight rows
+            // first weight element of the tile: rows j0.. of the (N, K) matrix in FWD, columns j0..
+            // of the (K, N) matrix in DX
+            nf4_base = B_RC ? ((int64_t)expert * N + j0) * K : (int64_t)expert * N * K + j0;
             if (B_RC) {
                 ldb = K;
                 b_tile = (const unsigned char *)(b + (int64_t)expert * N * K + (int64_t)j0 * ldb);
@@ -543,8 +545,11 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             }
         };
         // ---- NF4 weights: packed words travel through registers two steps ahead and are decoded
-        // into the other stage while the current one is multiplied.  A thread owns half a row of
-        // the weight stage: 32 weights = 16 packed bytes (one load) = four 16-byte LDS chunks.
+        // into the other stage while the current one is multiplied.  A thread owns 32 consecutive
+        // weights of one row of the weight stage: 16 packed bytes (one load) = four 16-byte LDS
+        // chunks.  FWD: a stage row is an output column, 64 weights along the reduction, two
+        // threads.  DX: a stage row is a reduction index, BN weights along the output columns,
+        // BN / 32 threads.
         // The 16 fp32 codes sit in LDS: whatever the nibbles, a wave's lookups fall in 16 different
         // banks (a 256-entry table of code pairs, one lookup per byte, was 2x slower: bank conflicts).
         constexpr int NT_ = NW * 64;
@@ -553,7 +558,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         // whole waves decode (a wave is 32 stage rows): a wave-uniform condition, no lane mask
         static_assert((BN * 2) % 64 == 0, "decoding threads are whole waves");
         const bool nf4_on = wave < BN * 2 / 64;
-        const int nf4_row = tid >> 1, nf4_half = tid & 1;
+        constexpr int NF4_SEGS = B_RC ? 2 : BN / 32;  // threads per stage row
+        const int nf4_row = tid / NF4_SEGS, nf4_half = tid % NF4_SEGS;
         // GLU: the thread's stage row belongs to the gate or to the up matrix, each with its own
         // packed bytes, absmax, block size and code table
         const bool nf4_up = GLU && glu_up(nf4_row);
@@ -567,9 +573,16 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         };
         auto nf4_load = [&](int kt, Nf4Regs &r) {
             if (!nf4_on) return;
-            int row = GLU ? glu_col(nf4_row) : nf4_row;
-            if (row >= j_lim) row = j_lim - 1;
-            const int64_t el = nf4_base + (int64_t)row * K + kt * BK + nf4_half * 32;
+            int64_t el;
+            if (B_RC) {
+                int row = GLU ? glu_col(nf4_row) : nf4_row;
+                if (row >= j_lim) row = j_lim - 1;
+                el = nf4_base + (int64_t)row * K + kt * BK + nf4_half * 32;
+            } else {
+                int col = nf4_half * 32;  // the host checked N % 32 == 0: a segment is inside or outside as a whole
+                if (col >= j_lim) col = j_lim - 32;
+                el = nf4_base + (int64_t)(kt * BK + nf4_row) * N + col;
+            }
             r.w = *(const uint4_t *)(nf4_w + (el >> 1));
             if (nf4_shift >= 5) {
                 r.am[0] = nf4_am[el >> nf4_shift];
@@ -861,6 +874,9 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
         } else {
             return MFL_ERR_UNSUPPORTED;
         }
+    } else if (nf4 != nullptr && mode == MODE_DX) {
+        if constexpr ((MODES & 2) && S == 2 && BK == 64 && NB * 64 <= NT) MFL_PIPE(MODE_DX, true, false)
+        else return MFL_ERR_UNSUPPORTED;
     } else if (nf4 != nullptr) {
         if constexpr ((MODES & 1) && S == 2 && BK == 64 && NB * 64 <= NT) MFL_PIPE(MODE_FWD, true, false)
         else return MFL_ERR_UNSUPPORTED;
@@ -1012,6 +1028,22 @@ int gemm_nf4_pipe(const void *x, const uint8_t *wq, const float *code16, const f
     const Nf4Params nf4 = {code16, absmax, shift};
     return dispatch_pipe(MODE_FWD, x, wq, m_sizes, ms_i64, y, R, N, K, E, out_dtype, 1.0f, 0, &nf4,
                          fusion ? &fu : nullptr, stream);
+}
+
+int gemm_nf4_pipe_dx(const void *dy, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                     const void *m_sizes, int ms_i64, void *dx, int64_t R, int N, int K, int E, int out_dtype,
+                     float alpha, int accumulate, hipStream_t stream) {
+    if (g_pipe_config < 0 || E > kMaxTableExperts) return MFL_ERR_UNSUPPORTED;
+    int shift = 0;
+    while ((1 << shift) < blocksize) ++shift;
+    // a thread decodes 32 consecutive output columns of one reduction row: whole segments only
+    if (K % 64 != 0 || N % 32 != 0 || N < 32 || blocksize < 8) return MFL_ERR_UNSUPPORTED;
+    if (!aligned(dy, 16) || !aligned(wq, 16) || !aligned(dx, 16)) return MFL_ERR_UNSUPPORTED;
+    if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
+    if (R <= 0) return MFL_OK;
+    const Nf4Params nf4 = {code16, absmax, shift};
+    return dispatch_pipe(MODE_DX, dy, wq, m_sizes, ms_i64, dx, R, N, K, E, out_dtype, alpha, accumulate, &nf4, nullptr,
+                         stream);
 }
 
 }  // namespace mfl

@@ -16,7 +16,7 @@ from .grouped_gemm.forward_transposed import grouped_gemm_forward_transposed
 from .grouped_gemm.fused import grouped_glu_forward, grouped_glu_forward_4bit
 from .kernels.routing import _combine, _gather
 from .kernels.silu_mul import silu_mul_backward
-from .quantize.nf4 import dequantize_nf4
+from .grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit
 
 
 class _GluGathered(torch.autograd.Function):
@@ -78,11 +78,9 @@ class _GluGathered4bit(torch.autograd.Function):
     def backward(ctx, dh):
         gate_packed, up_packed, m_sizes, inv_sort_idx, e, g = ctx.saved_tensors
         de, dg = silu_mul_backward(dh.contiguous(), e, g)
-        # frozen weights: only the tokens get a gradient; no fused kernel covers the transposed
-        # product on packed weights, so each matrix is dequantised for it (quantize/layer.py:17-22)
-        dx = grouped_gemm_forward_transposed(de, dequantize_nf4(gate_packed, ctx.states[0], de.dtype), m_sizes, de.dtype)
-        grouped_gemm_forward_transposed(dg, dequantize_nf4(up_packed, ctx.states[1], dg.dtype), m_sizes, out=dx,
-                                        accumulate=True)
+        # frozen weights: only the tokens get a gradient
+        dx = grouped_gemm_forward_transposed_4bit(de, gate_packed, ctx.states[0], m_sizes, de.dtype)
+        grouped_gemm_forward_transposed_4bit(dg, up_packed, ctx.states[1], m_sizes, out=dx, accumulate=True)
         d_tokens = _combine(dx, inv_sort_idx, None, ctx.n_tokens, ctx.k)
         return d_tokens, None, None, None, None, None, None, None, None
 

@@ -49,3 +49,40 @@ def grouped_gemm_forward_4bit(x: torch.Tensor, w_quant: torch.Tensor, w_quant_st
                                      _lib.dtype_code(x.dtype), _lib.dtype_code(y.dtype), _lib.stream())
     _lib.check(rc, "mfl_gemm_fwd_nf4")
     return y
+
+
+def grouped_gemm_forward_transposed_4bit(dy: torch.Tensor, w_quant: torch.Tensor, w_quant_state,
+                                         m_sizes: torch.Tensor, dtype: Optional[torch.dtype] = None, *,
+                                         out: Optional[torch.Tensor] = None, alpha: float = 1.0,
+                                         accumulate: bool = False) -> torch.Tensor:
+    """``grouped_gemm_forward_transposed(dy, W, m_sizes)`` with ``W`` = the NF4 weight of shape
+    (E, out, in) = ``w_quant_state.shape``: dx (rows, in) = dy (rows, out) @ W[e].  The weight is
+    decoded inside the kernel; for shapes the fused kernel does not take (status UNSUPPORTED) it
+    is dequantised first, as the reference always does (kernels/fast_lora.py:57-62,127-131)."""
+    from ..quantize.nf4 import dequantize_nf4
+    from .forward_transposed import grouped_gemm_forward_transposed
+
+    assert w_quant_state.quant_type == "nf4"
+    blocksize = int(w_quant_state.blocksize)
+    code = w_quant_state.code
+    absmax = resolve_absmax(w_quant_state)
+    assert dy.is_cuda and dy.ndim == 2 and dy.is_contiguous() and m_sizes.is_contiguous()
+    assert is_int_tensor(w_quant) and is_int_tensor(m_sizes) and w_quant.is_contiguous()
+    experts, k, n = w_quant_state.shape
+    rows = dy.shape[0]
+    assert dy.shape[1] == k and m_sizes.numel() == experts
+    if out is None:
+        assert not accumulate, "accumulate needs an existing output"
+        out = torch.empty((rows, n), device=dy.device, dtype=dy.dtype if dtype is None else dtype)
+    else:
+        assert out.shape == (rows, n) and out.is_contiguous() and out.device == dy.device
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_gemm_dx_nf4(_lib.ptr(dy), _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), blocksize,
+                                    _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(out), rows, n, k, experts,
+                                    _lib.dtype_code(dy.dtype), _lib.dtype_code(out.dtype), float(alpha),
+                                    int(bool(accumulate)), _lib.stream())
+    if rc == -6:  # MFL_ERR_UNSUPPORTED
+        w = dequantize_nf4(w_quant, w_quant_state, dy.dtype)
+        return grouped_gemm_forward_transposed(dy, w, m_sizes, dtype, out=out, alpha=alpha, accumulate=accumulate)
+    _lib.check(rc, "mfl_gemm_dx_nf4")
+    return out

@@ -11,8 +11,8 @@ Out = (Wp + S Bp Ap) In:
     dAp = S t^T In        dBp = S dOut^T u        dIn = dOut Wp + S t Ap
 Every LoRA gradient is therefore a rank-r grouped GEMM; the full (E, out, in) weight gradient
 that the reference forms and then contracts (fast_lora.py:139-149) is never built.  Base weights
-may be NF4 (``*qs`` not None): the forward products decode them inside the GEMM, the input
-gradients dequantise.
+may be NF4 (``*qs`` not None): the forward and the input-gradient products decode them inside
+the GEMM (the reference dequantises, fast_lora.py:57-62 "TODO: Fuse dequant and linear").
 """
 from __future__ import annotations
 
@@ -21,6 +21,7 @@ import torch
 from ..grouped_gemm.backward_dw import grouped_gemm_backward_dw as _dw
 from ..grouped_gemm.forward import grouped_gemm_forward as _fwd
 from ..grouped_gemm.forward_4bit import grouped_gemm_forward_4bit as _fwd4
+from ..grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit as _dx4
 from ..grouped_gemm.forward_transposed import grouped_gemm_forward_transposed as _dx
 from ..quantize.nf4 import dequantize_nf4
 from .silu_mul import silu_mul_backward_inplace, silu_mul_forward
@@ -47,8 +48,10 @@ def _proj_fwd(x, wq, wqs, a, b, s, m_sizes):
 
 def _proj_bwd_input(dout, t, wq, wqs, a, s, m_sizes, out=None):
     """dIn (+)= dOut W + s * t A."""
-    w = _dense(wq, wqs, dout.dtype)
-    out = _dx(dout, w, m_sizes, out=out, accumulate=out is not None)
+    if wqs is not None and dout.dtype == torch.bfloat16:
+        out = _dx4(dout, wq, wqs, m_sizes, out=out, accumulate=out is not None)
+    else:
+        out = _dx(dout, _dense(wq, wqs, dout.dtype), m_sizes, out=out, accumulate=out is not None)
     return _dx(t, a, m_sizes, out=out, alpha=s, accumulate=True)
 
 

@@ -2,7 +2,7 @@
 
 ``moe_fused_linear_4bit`` runs the forward product straight off the packed weights (NF4 decode
 fused into the grouped GEMM) instead of materialising the (E, N, K) weight as the reference does
-(quantize/layer.py:17-22); only the input gradient, which no fused kernel covers yet, dequantises.
+(quantize/layer.py:17-22), and so does the input gradient.
 ``MoeFusedLinear4bit`` keeps the module contract: frozen packed ``weight`` carrying a
 ``quant_state``, compute-dtype handling (:54-74, :83-96) and quant-state entries in the state
 dict (:76-81).
@@ -16,8 +16,7 @@ import torch
 from torch import nn
 
 from ..grouped_gemm.forward import grouped_gemm_forward
-from ..grouped_gemm.forward_4bit import grouped_gemm_forward_4bit
-from ..grouped_gemm.forward_transposed import grouped_gemm_forward_transposed
+from ..grouped_gemm.forward_4bit import grouped_gemm_forward_4bit, grouped_gemm_forward_transposed_4bit
 from ..modular_qwen3_moe_fused import MoeFusedLinear
 from .nf4 import Nf4QuantState, dequantize_nf4, quantize_nf4
 
@@ -36,8 +35,7 @@ class _GroupedGemm4bit(torch.autograd.Function):
         packed, m_sizes = ctx.saved_tensors
         dx = None
         if ctx.needs_input_grad[0]:
-            w = dequantize_nf4(packed, ctx.quant_state, dy.dtype)
-            dx = grouped_gemm_forward_transposed(dy.contiguous(), w, m_sizes, dy.dtype)
+            dx = grouped_gemm_forward_transposed_4bit(dy.contiguous(), packed, ctx.quant_state, m_sizes, dy.dtype)
         return dx, None, None, None
 
 
