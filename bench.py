@@ -194,6 +194,15 @@ def main() -> int:
                                        "fused_packed_gbs": round(packed_bytes / us_f / 1e3, 1),
                                        "fused_tflops": round(2.0 * tokens * TOPK * INTER * HIDDEN / us_f / 1e6, 1)}
         extra["nf4_gate_proj"] = nf4
+        # the input-gradient product on the same packed weights (seen as (E, K=768, N=2048)) at 4096 tokens
+        from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit
+        dyg = torch.randn((ROWS, INTER), device=dev, dtype=torch.bfloat16)
+        us_f = _event_us(lambda i: grouped_gemm_forward_transposed_4bit(dyg, packed, qstate, m_sizes), 50, 10, stream)
+        us_u = _event_us(lambda i: grouped_gemm_forward_transposed(dyg, dequantize_nf4(packed, qstate, torch.bfloat16),
+                                                                  m_sizes), 50, 10, stream)
+        extra["nf4_gate_proj_dx"] = {"fused_us": round(us_f, 1), "dequant_then_gemm_us": round(us_u, 1),
+                                     "fused_tflops": round(flop / us_f / 1e6, 1)}
+        del dyg
         del packed, qstate, x5
         # config 4: rank-16 LoRA on gate_proj, 8192 tokens, Zipf(1.2)-skewed top-8 routing (65536 rows):
         # the frozen base product and the five thin products of one forward + backward
