@@ -419,6 +419,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         const int64_t step_a = A_RC ? (int64_t)BK * 2 : (int64_t)BK * lda * 2;
         const int64_t step_b = B_RC ? (int64_t)BK * 2 : (int64_t)BK * ldb * 2;
 
+        constexpr bool SKIP_A = A_RC && S == 2;
+        constexpr int SA_ROWS_PER_COPY = 64 / SA::kChunksPerRow;
         auto issue = [&](int kt) {
             unsigned char *st = smem + (kt % S) * STAGE_BYTES;
             const unsigned char *pa = a_tile + kt * step_a;
@@ -433,9 +435,14 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             const bool tail = (kt + 1) * BK > red;
             if (!tail) {
 #pragma unroll
-                for (int q = 0; q < LA; ++q)
+                for (int q = 0; q < LA; ++q) {
+                    // a copy fills whole stage rows; rows past the tile's last one feed nothing that
+                    // is stored (with two stages every wait is for all copies, so leaving some out
+                    // does not disturb the counting)
+                    if (SKIP_A && (wave * LA + q) * SA_ROWS_PER_COPY >= i_lim) continue;
                     __builtin_amdgcn_global_load_lds((global_void_ptr)(pa + lane_off[q]),
                                                      (lds_void_ptr)(st + (wave * LA + q) * 1024), 16, 0, 0);
+                }
 #pragma unroll
                 for (int q = 0; q < LB; ++q)
                     __builtin_amdgcn_global_load_lds((global_void_ptr)(b_src(q) + lane_off[LA + q]),
