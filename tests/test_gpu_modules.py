@@ -313,3 +313,40 @@ def test_fused_front_of_block_with_4bit_projections():
         outs.append((out.detach(), h.grad))
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[1][0], outs[2][0])
     _grads_close(outs[1][1], outs[0][1], "d hidden, 4-bit")
+
+
+def test_fused_model_matches_installed_transformers_model():
+    """The method of the reference's test_model.py (tiny fp32 model, same weights in both
+    layouts, same hidden states), against the transformers release that is installed."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import Qwen3MoeConfig, Qwen3MoeModel
+
+    from qwen3_moe_fused.modular_qwen3_moe_fused import Qwen3MoeFusedModel
+
+    torch.manual_seed(42)
+    inter = 3
+    config = Qwen3MoeConfig(vocab_size=500, hidden_size=16, intermediate_size=5, num_hidden_layers=2,
+                            num_attention_heads=8, num_key_value_heads=4, max_window_layers=2,
+                            moe_intermediate_size=inter, num_experts=11, norm_topk_prob=True,   # test_model.py:29-40
+                            experts_implementation="eager")   # torch's grouped mm refuses rows of 3 elements
+    model = Qwen3MoeModel(config).to(DEV, torch.float32).eval()
+    fused = Qwen3MoeFusedModel(config).to(DEV, torch.float32).eval()
+    sd = {}
+    for key, value in model.state_dict().items():
+        if key.endswith("mlp.experts.gate_up_proj"):      # (E, 2 * inter, hidden): gate rows first
+            stem = key[: -len("experts.gate_up_proj")]
+            sd[stem + "gate_proj.weight"] = value[:, :inter].contiguous()
+            sd[stem + "up_proj.weight"] = value[:, inter:].contiguous()
+        elif key.endswith("mlp.experts.down_proj"):
+            sd[key[: -len("experts.down_proj")] + "down_proj.weight"] = value
+        elif ".mlp.experts." in key:                      # per-expert layout of older releases
+            pytest.skip("installed transformers keeps one matrix per expert; covered by tests/test_convert.py")
+        else:
+            sd[key] = value
+    missing, unexpected = fused.load_state_dict(sd, strict=False)
+    assert not unexpected and not [k for k in missing if "rotary" not in k], (missing, unexpected)
+    ids = torch.randint(0, 500, (7, 13), generator=gen(1)).to(DEV)
+    with torch.no_grad():
+        h_ref = model(input_ids=ids).last_hidden_state
+        h = fused(input_ids=ids).last_hidden_state
+    torch.testing.assert_close(h, h_ref, rtol=1e-4, atol=1e-4)

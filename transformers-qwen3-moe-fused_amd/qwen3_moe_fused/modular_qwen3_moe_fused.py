@@ -117,15 +117,28 @@ class Qwen3MoeFusedSparseMoeBlock(nn.Module):
 def _hf_subclasses():
     """Model-level wiring (decoder layer / model / causal LM with the fused block swapped in),
     built on demand so that importing this module does not import transformers."""
+    import inspect
+
     from transformers.models.qwen3_moe.modeling_qwen3_moe import (Qwen3MoeDecoderLayer, Qwen3MoeForCausalLM,
-                                                                  Qwen3MoeMLP, Qwen3MoeModel)
+                                                                  Qwen3MoeMLP, Qwen3MoeModel, Qwen3MoeSparseMoeBlock)
+
+    # The reference was written against a transformers revision whose sparse block returns
+    # (hidden_states, router_logits) (modular_qwen3_moe_fused.py:1,118); later releases return the
+    # hidden states alone and the decoder layer adds them to the residual as they come.
+    block_cls = Qwen3MoeFusedSparseMoeBlock
+    if inspect.signature(Qwen3MoeSparseMoeBlock.forward).return_annotation is torch.Tensor:
+        class _TensorBlock(Qwen3MoeFusedSparseMoeBlock):
+            def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+                return super().forward(hidden_states)[0]
+
+        block_cls = _TensorBlock
 
     class Qwen3MoeFusedDecoderLayer(Qwen3MoeDecoderLayer):
         def __init__(self, config, layer_idx: int) -> None:
             super().__init__(config, layer_idx)
             sparse = (layer_idx not in config.mlp_only_layers and config.num_experts > 0
                       and (layer_idx + 1) % config.decoder_sparse_step == 0)
-            self.mlp = (Qwen3MoeFusedSparseMoeBlock(config) if sparse
+            self.mlp = (block_cls(config) if sparse
                         else Qwen3MoeMLP(config, intermediate_size=config.intermediate_size))
 
     class Qwen3MoeFusedModel(Qwen3MoeModel):
