@@ -14,11 +14,18 @@ struct Vec {
     T v[N];
 };
 
+// (the loads fill their destination in place: returning the vector by value made the compiler
+// take it apart into elements and pack it again)
 template <typename T>
-__device__ __forceinline__ Vec<T> ld_vec(const T *p) {
-    Vec<T> r;
+__device__ __forceinline__ void ld_vec(Vec<T> &r, const T *p) {
     *(uint4_t *)r.v = *(const uint4_t *)p;
-    return r;
+}
+// 16-byte load of data that is read once (non-temporal: does not displace what the caches hold).
+// It pays where rows are picked at random (combine: 50 -> 27 us); the contiguous sweeps of the
+// SiLU kernels were 10 % slower with it.
+template <typename T>
+__device__ __forceinline__ void ld_vec_stream(Vec<T> &r, const T *p) {
+    *(uint4_t *)r.v = __builtin_nontemporal_load((const uint4_t *)p);
 }
 template <typename T>
 __device__ __forceinline__ void st_vec(T *p, const Vec<T> &r) {
@@ -47,7 +54,9 @@ __global__ __launch_bounds__(256) void silu_fwd_kernel(const T *e, const T *g, T
     if (vec_ok) {
         const int64_t nv = n / V;
         for (int64_t q = i; q < nv; q += stride) {
-            Vec<T> ve = ld_vec(e + q * V), vg = ld_vec(g + q * V), vh;
+            Vec<T> ve, vg, vh;
+            ld_vec(ve, e + q * V);
+            ld_vec(vg, g + q * V);
 #pragma unroll
             for (int u = 0; u < V; ++u) vh.v[u] = silu_fwd_one(ve.v[u], vg.v[u]);
             st_vec(h + q * V, vh);
@@ -67,7 +76,10 @@ __global__ __launch_bounds__(256) void silu_bwd_kernel(const T *dh, const T *e, 
     if (vec_ok) {
         const int64_t nv = n / V;
         for (int64_t q = i; q < nv; q += stride) {
-            Vec<T> vdh = ld_vec(dh + q * V), ve = ld_vec(e + q * V), vg = ld_vec(g + q * V), vh, vde, vdg;
+            Vec<T> vdh, ve, vg, vh, vde, vdg;
+            ld_vec(vdh, dh + q * V);
+            ld_vec(ve, e + q * V);
+            ld_vec(vg, g + q * V);
 #pragma unroll
             for (int u = 0; u < V; ++u) silu_bwd_one(vdh.v[u], ve.v[u], vg.v[u], vh.v[u], vde.v[u], vdg.v[u]);
             if (h) st_vec(h + q * V, vh);
@@ -114,7 +126,7 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const T *src, const in
             Vec<T> v[U];
 #pragma unroll
             for (int q = 0; q < U; ++q)
-                if (c0 + q * 64 * V < H) v[q] = ld_vec(s + c0 + q * 64 * V);
+                if (c0 + q * 64 * V < H) ld_vec(v[q], s + c0 + q * 64 * V);
 #pragma unroll
             for (int q = 0; q < U; ++q) {
                 if (c0 + q * 64 * V >= H) continue;
@@ -141,33 +153,48 @@ __global__ __launch_bounds__(256) void combine_rows_kernel(const T *src, const i
     const int32_t *p = pos + t * k;
     T *d = dst + t * H;
     if (vec_ok) {
-        for (int c = lane * V; c < H; c += 64 * V) {
-            float acc[V];
+        // A lane owns CC chunks of V columns, 64 * V apart, so that the wave reads whole rows (a
+        // row is one contiguous run in memory): U rows at a time, all chunks of a row together,
+        // before they are added (in order: the sum is the same as one row after the other).
+        // Every row is read exactly once: streaming loads, which leave the caches to the writes.
+        // (Measured at 4096 tokens x 8 rows of 2048: a 1 KiB piece of each of 8 rows per pass
+        // with ordinary loads, 55 us; this, 27 us.)
+        constexpr int CC = 4, U = 4;
+        for (int c0 = lane * V; c0 < H; c0 += CC * 64 * V) {
+            float acc[CC][V];
 #pragma unroll
-            for (int u = 0; u < V; ++u) acc[u] = 0.f;
-            // the selected rows are read eight at a time before they are added (in order: the sum
-            // is the same as one row after the other)
-            constexpr int U = 8;
+            for (int cc = 0; cc < CC; ++cc)
+#pragma unroll
+                for (int u = 0; u < V; ++u) acc[cc][u] = 0.f;
             for (int j0 = 0; j0 < k; j0 += U) {
-                Vec<T> v[U];
+                Vec<T> v[U][CC];
                 float w[U];
 #pragma unroll
                 for (int q = 0; q < U; ++q) {
                     if (j0 + q >= k) continue;
                     w[q] = weights ? to_f32(weights[t * k + j0 + q]) : 1.0f;
-                    v[q] = ld_vec(src + (int64_t)p[j0 + q] * H + c);
+                    const T *row = src + (int64_t)p[j0 + q] * H + c0;
+#pragma unroll
+                    for (int cc = 0; cc < CC; ++cc)
+                        if (c0 + cc * 64 * V < H) ld_vec_stream(v[q][cc], row + cc * 64 * V);
                 }
 #pragma unroll
                 for (int q = 0; q < U; ++q) {
                     if (j0 + q >= k) continue;
 #pragma unroll
-                    for (int u = 0; u < V; ++u) acc[u] = fmaf(to_f32(v[q].v[u]), w[q], acc[u]);
+                    for (int cc = 0; cc < CC; ++cc)
+#pragma unroll
+                        for (int u = 0; u < V; ++u) acc[cc][u] = fmaf(to_f32(v[q][cc].v[u]), w[q], acc[cc][u]);
                 }
             }
-            Vec<T> o;
 #pragma unroll
-            for (int u = 0; u < V; ++u) o.v[u] = from_f32<T>(acc[u]);
-            st_vec(d + c, o);
+            for (int cc = 0; cc < CC; ++cc) {
+                if (c0 + cc * 64 * V >= H) continue;
+                Vec<T> o;
+#pragma unroll
+                for (int u = 0; u < V; ++u) o.v[u] = from_f32<T>(acc[cc][u]);
+                st_vec(d + c0 + cc * 64 * V, o);
+            }
         }
     } else {
         for (int c = lane; c < H; c += 64) {
