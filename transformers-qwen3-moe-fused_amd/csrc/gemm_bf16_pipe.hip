@@ -419,6 +419,11 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         const int64_t step_a = A_RC ? (int64_t)BK * 2 : (int64_t)BK * lda * 2;
         const int64_t step_b = B_RC ? (int64_t)BK * 2 : (int64_t)BK * ldb * 2;
 
+        // Cache policy of the weight copies in the row-grouped products: a weight is read by exactly
+        // one workgroup, so it is fetched non-temporal (bit 1 of the instruction's cache-policy
+        // field) and leaves the L2 to the rows, which the workgroups of an expert share
+        // (fwd 146.6 -> 140.5 us, dX 161.4 -> 157.3 us; the same hint on the rows costs 5-10 %).
+        constexpr int B_POLICY = MODE == MODE_DW ? 0 : 2;
         constexpr bool SKIP_A = A_RC && S == 2;
         constexpr int SA_ROWS_PER_COPY = 64 / SA::kChunksPerRow;
         auto issue = [&](int kt) {
@@ -446,7 +451,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 #pragma unroll
                 for (int q = 0; q < LB; ++q)
                     __builtin_amdgcn_global_load_lds((global_void_ptr)(b_src(q) + lane_off[LA + q]),
-                                                     (lds_void_ptr)(st + SA::kBytes + (wave * LB + q) * 1024), 16, 0, 0);
+                                                     (lds_void_ptr)(st + SA::kBytes + (wave * LB + q) * 1024), 16, 0,
+                                                     B_POLICY);
                 return;
             }
 #pragma unroll
@@ -728,9 +734,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 #pragma unroll
                         for (int u = 0; u < 8; ++u) h8[u] = silu_fwd_one<bf16_t>(e8[u], g8[u]);
                         const int64_t o = (int64_t)row * ldc + col;
-                        *(bf16x8 *)((bf16_t *)c_base + o) = h8;
-                        if (fu.c_e) *(bf16x8 *)((bf16_t *)fu.c_e + o) = e8;
-                        if (fu.c_g) *(bf16x8 *)((bf16_t *)fu.c_g + o) = g8;
+                        __builtin_nontemporal_store(h8, (bf16x8 *)((bf16_t *)c_base + o));
+                        if (fu.c_e) __builtin_nontemporal_store(e8, (bf16x8 *)((bf16_t *)fu.c_e + o));
+                        if (fu.c_g) __builtin_nontemporal_store(g8, (bf16x8 *)((bf16_t *)fu.c_g + o));
                     }
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -767,8 +773,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                     const int col = j0 + wn * WTN + lcol;
                     if (row >= i_end || col >= j_end) continue;
                     // the output width is a multiple of 8: a chunk is inside or outside as a whole
-                    *(uint4_t *)((bf16_t *)c_base + (int64_t)row * ldc + col) =
-                        *(const uint4_t *)(ep + row_l * ROWB + lcol * 2);
+                    // written once, read by a later kernel: streaming store (dW 205 -> 199 us)
+                    __builtin_nontemporal_store(*(const uint4_t *)(ep + row_l * ROWB + lcol * 2),
+                                                (uint4_t *)((bf16_t *)c_base + (int64_t)row * ldc + col));
                 }
             }
         } else if (sizeof(TO) == 2) {
