@@ -261,6 +261,20 @@ def main() -> int:
                 us = _event_us(lambda i: blk(h5), n_it, 3, stream)
                 block[f"tokens_{tokens}"] = {"us": round(us, 1), "tokens_per_s": round(tokens / us * 1e6),
                                              "module_by_module_us": round(us_sep, 1)}
+                if tokens <= 256:
+                    # decode-sized calls are bound by the seven launches: the same forward captured once in a
+                    # HIP graph and replayed (the library only enqueues kernels, so capture needs nothing special)
+                    side = torch.cuda.Stream()
+                    side.wait_stream(torch.cuda.current_stream())
+                    with torch.cuda.stream(side):
+                        blk(h5)
+                    torch.cuda.current_stream().wait_stream(side)
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        blk(h5)
+                    us_g = _event_us(lambda i: graph.replay(), n_it, 3, stream)
+                    block[f"tokens_{tokens}"]["hip_graph_replay_us"] = round(us_g, 1)
+                    del graph
         extra["nf4_sparse_block_fwd_config5"] = block
         del blk
         # the same block with bf16 experts at the headline configuration's 4096 tokens, and its front half
