@@ -24,7 +24,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of the benchmarked kernel, from the FETCH_SIZE / WRITE_SIZE passes summarised in
 # profiles/gemm_fwd_gate_proj_config2_hbm_traffic.txt (537.1 MB read + 50.3 MB written)
-MEASURED_TRAFFIC_BYTES = 587.5e6
+MEASURED_TRAFFIC_BYTES = 591.0e6
 
 E, HIDDEN, INTER, TOKENS, TOPK = 128, 2048, 768, 4096, 8
 ROWS = TOKENS * TOPK
