@@ -152,7 +152,7 @@ def main() -> int:
         dys = [torch.randn((ROWS, HIDDEN), device=dev, dtype=torch.bfloat16) for _ in range(NB)]   # grad of down_proj out
         hs = [torch.randn((ROWS, INTER), device=dev, dtype=torch.bfloat16) for _ in range(NB)]     # down_proj input
         wd = [w.view(E, HIDDEN, INTER) for w in ws]                                                # (128, 2048, 768)
-        it, wm = 50, 5
+        it, wm = 50, 100      # 100 warm-up launches: a burst of launches starts in a power-management transient
         us = _event_us(lambda i: grouped_gemm_forward_transposed(dys[i % NB], wd[i % NB], m_sizes), it, wm, stream)
         extra["dx_down_proj"] = {"us": round(us, 1), "tflops": round(flop / us / 1e6, 1),
                                  "mfma_frac": round(flop / us / 1e6 / PEAK_BF16_TFLOPS, 4),
@@ -183,10 +183,10 @@ def main() -> int:
             _, _, s5 = softmax_topk_raw(lgt, TOPK, True, torch.bfloat16)
             ms5, _, _ = get_expert_counts_and_idx(s5.view(-1), E)
             x5 = torch.randn((tokens * TOPK, HIDDEN), device=dev, dtype=torch.bfloat16)
-            n_it = 20 if tokens > 1000 else 50
-            us_f = _event_us(lambda i: grouped_gemm_forward_4bit(x5, packed, qstate, ms5), n_it, 3, stream)
+            n_it, n_wm = (20, 30) if tokens > 1000 else (50, 100)
+            us_f = _event_us(lambda i: grouped_gemm_forward_4bit(x5, packed, qstate, ms5), n_it, n_wm, stream)
             us_u = _event_us(lambda i: grouped_gemm_forward(x5, dequantize_nf4(packed, qstate, torch.bfloat16), ms5),
-                             n_it, 3, stream)
+                             n_it, n_wm, stream)
             active = int((ms5 > 0).sum().item())                       # host read outside any timed loop
             packed_bytes = active * INTER * HIDDEN * (0.5 + 4.0 / 64)
             nf4[f"tokens_{tokens}"] = {"fused_us": round(us_f, 1), "dequant_then_gemm_us": round(us_u, 1),
@@ -197,9 +197,9 @@ def main() -> int:
         # the input-gradient product on the same packed weights (seen as (E, K=768, N=2048)) at 4096 tokens
         from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit
         dyg = torch.randn((ROWS, INTER), device=dev, dtype=torch.bfloat16)
-        us_f = _event_us(lambda i: grouped_gemm_forward_transposed_4bit(dyg, packed, qstate, m_sizes), 50, 10, stream)
+        us_f = _event_us(lambda i: grouped_gemm_forward_transposed_4bit(dyg, packed, qstate, m_sizes), 50, 100, stream)
         us_u = _event_us(lambda i: grouped_gemm_forward_transposed(dyg, dequantize_nf4(packed, qstate, torch.bfloat16),
-                                                                  m_sizes), 50, 10, stream)
+                                                                  m_sizes), 50, 50, stream)
         extra["nf4_gate_proj_dx"] = {"fused_us": round(us_f, 1), "dequant_then_gemm_us": round(us_u, 1),
                                      "fused_tflops": round(flop / us_f / 1e6, 1)}
         del dyg
@@ -228,7 +228,7 @@ def main() -> int:
                 ("lora_dy_b", lambda i: grouped_gemm_forward_transposed(dy4, lb, ms4), R4 * INTER * 2),
                 ("lora_da", lambda i: grouped_gemm_backward_dw(x4, t4, ms4, torch.bfloat16), R4 * HIDDEN * 2),
                 ("lora_db", lambda i: grouped_gemm_backward_dw(u4, dy4, ms4, torch.bfloat16), R4 * INTER * 2)):
-            us = _event_us(fn, 20, 3, stream)
+            us = _event_us(fn, 50, 100, stream)
             lora[name] = {"us": round(us, 1)}
             if stream_bytes is None:
                 lora[name]["tflops"] = round(flop4 / us / 1e6, 1)
@@ -309,6 +309,19 @@ def main() -> int:
                            stream)
             bf16_block["front_half"] = {"fused_us": round(us, 1), "four_kernels_us": round(us_sep, 1),
                                         "fused_tflops": round(2 * flop / us / 1e6, 1)}
+        # one training step of the block: forward + backward to the hidden states and all four weight matrices
+        blk.zero_grad(set_to_none=True)
+        gouts = [torch.randn((1, TOKENS, HIDDEN), device=dev, dtype=torch.bfloat16) for _ in range(NB)]
+
+        def train_step(i):
+            h = toks[i % NB].detach().requires_grad_()
+            out, _ = blk(h)
+            out.backward(gouts[i % NB])
+            blk.zero_grad(set_to_none=True)
+
+        us = _event_us(train_step, 20, 10, stream)
+        bf16_block["block_fwd_bwd"] = {"us": round(us, 1), "tokens_per_s": round(TOKENS / us * 1e6),
+                                       "tflops": round(9 * flop / us / 1e6, 1)}   # 3 products x (fwd + dX + dW)
         extra["bf16_sparse_block_fwd_config2"] = bf16_block
         del blk, toks
         out["extra"] = extra
