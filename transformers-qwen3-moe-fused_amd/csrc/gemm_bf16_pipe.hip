@@ -10,8 +10,9 @@
 //   RC stage: row i holds BK elements (BK*2 bytes); 16-byte chunk c of row i is stored at
 //             chunk c ^ ((i / rows_per_256B) % chunks_per_row): the 16 rows one half-wave reads
 //             for an MFMA fragment then fall in 16 different bank groups.
-//   RS stage: row r holds BI elements; chunk c of row r is stored at c ^ ((r & 3) << 1): the
-//             four rows a transposing read (ds_read_b64_tr_b16) touches fall in different banks.
+//   RS stage: row r holds BI elements; chunk c of row r is stored at c ^ ((r & 3) << s), s = 1 or
+//             2 by row length: the four rows a transposing read (ds_read_b64_tr_b16) touches
+//             fall in different banks.
 //
 // Tiles.  A tile is MB x NB blocks of 32 x 32.  The WGM x WGN waves of a workgroup split the
 // columns in contiguous runs and take the 32-row blocks round robin (wave row w owns blocks
@@ -55,6 +56,12 @@ struct Stage {
     static constexpr int kWaveLoads = kBytes / 1024;       // 1 KiB per wave-wide copy
     static constexpr int kChunksPerRow = kRowBytes / 16;
     static constexpr int kRowsPer256 = kRowBytes >= 256 ? 1 : 256 / kRowBytes;
+    // RS rows: a transposing read touches 4 consecutive rows, and the two 16-lane groups that the
+    // LDS serves together read 32 bytes each of every row, 32 bytes apart.  Rows whose length is
+    // a multiple of 256 bytes start in the same bank: they are spread 64 bytes apart (4 rows x 64
+    // bytes = all 64 banks).  Other row lengths (384 bytes) already differ by 128 bytes from row to
+    // row, and a 32-byte spread keeps the XOR inside the row.
+    static constexpr int kRsShift = kChunksPerRow % 16 == 0 ? 2 : 1;
     static_assert(kBytes % 1024 == 0 && kChunksPerRow % 8 == 0, "stage must be whole copies, rows whole 128 B");
 
     // stage row and physical chunk that lane `lane` of wave-load `load` fills (a copy covers 64
@@ -65,7 +72,7 @@ struct Stage {
     // physical 16-byte chunk of logical chunk c in row `row`
     __device__ static __forceinline__ int swz(int row, int c) {
         if (RC) return c ^ ((row / kRowsPer256) % kChunksPerRow);
-        return c ^ ((row & 3) << 1);
+        return c ^ ((row & 3) << kRsShift);
     }
 };
 
