@@ -145,3 +145,27 @@ def test_gather_combine_autograd_fp32():
     torch.testing.assert_close(out, out2, rtol=1e-5, atol=1e-5)
     torch.testing.assert_close(hidden.grad, h2.grad, rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(logits.grad, l2.grad, rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("T,k,H,dtype", [(300, 8, 2048, torch.bfloat16), (50, 3, 40, torch.bfloat16),
+                                         (50, 5, 36, torch.bfloat16), (33, 2, 4104, torch.bfloat16),
+                                         (64, 8, 64, torch.float32)])
+def test_rows_dot_against_numpy(T, k, H, dtype):
+    """dots[t, j] = <a[t], b[pos[t*k+j]]> (gradient of the combine with respect to the routing
+    weights): vector path, scalar path (row length not a multiple of 16 bytes), rows longer than
+    one pass of the wave, k not a multiple of the rows in flight."""
+    from qwen3_moe_fused import _lib
+
+    g = gen(T + H)
+    a = randn((T, H), g, 1.0, dtype)
+    b = randn((T * k, H), g, 1.0, dtype)
+    pos = torch.randperm(T * k, generator=g).to(torch.int32)
+    dots = torch.empty((T, k), dtype=dtype, device=DEV)
+    ad, bd, pd = a.to(DEV), b.to(DEV), pos.to(DEV)
+    rc = _lib.lib().mfl_rows_dot(_lib.ptr(ad), _lib.ptr(bd), _lib.ptr(pd), _lib.ptr(dots), T, k, H,
+                                 _lib.dtype_code(dtype), _lib.stream())
+    _lib.check(rc, "mfl_rows_dot")
+    ref = np.einsum("th,tjh->tj", to_np32(a).astype(np.float64),
+                    to_np32(b)[pos.numpy().astype(np.int64)].reshape(T, k, H).astype(np.float64))
+    tol = 1e-2 if dtype == torch.bfloat16 else 1e-5
+    check_close(dots, ref, tol, tol, "rows_dot")

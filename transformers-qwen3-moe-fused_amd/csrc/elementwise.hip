@@ -208,20 +208,62 @@ __global__ __launch_bounds__(256) void combine_rows_kernel(const T *src, const i
     }
 }
 
-// One wave per (token, selection) pair.
+// One wave per token: dots[t, j] = <a[t, :], b[pos[t*k+j], :]>.  Like the combine kernel it reads
+// whole rows of b, U at a time with streaming loads (each is read exactly once); the token's own
+// row of a comes from the cache after the first group.
 template <typename T>
 __global__ __launch_bounds__(256) void rows_dot_kernel(const T *a, const T *b, const int32_t *pos, T *dots,
-                                                       int64_t n_pairs, int k, int H) {
+                                                       int64_t Tn, int k, int H, int vec_ok) {
+    constexpr int V = Vec<T>::N;
     const int lane = threadIdx.x & 63;
-    const int64_t pair = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (pair >= n_pairs) return;
-    const T *pa = a + (pair / k) * H;
-    const T *pb = b + (int64_t)pos[pair] * H;
-    float acc = 0.f;
-    for (int c = lane; c < H; c += 64) acc = fmaf(to_f32(pa[c]), to_f32(pb[c]), acc);
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= Tn) return;
+    const T *pa = a + t * H;
+    const int32_t *p = pos + t * k;
+    constexpr int CC = 4, U = 4;
+    for (int j0 = 0; j0 < k; j0 += U) {
+        float acc[U];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-    if (lane == 0) dots[pair] = from_f32<T>(acc);
+        for (int q = 0; q < U; ++q) acc[q] = 0.f;
+        if (vec_ok) {
+            for (int c0 = lane * V; c0 < H; c0 += CC * 64 * V) {
+                Vec<T> va[CC], vb[U][CC];
+#pragma unroll
+                for (int q = 0; q < U; ++q) {
+                    if (j0 + q >= k) continue;
+                    const T *row = b + (int64_t)p[j0 + q] * H + c0;
+#pragma unroll
+                    for (int cc = 0; cc < CC; ++cc)
+                        if (c0 + cc * 64 * V < H) ld_vec_stream(vb[q][cc], row + cc * 64 * V);
+                }
+#pragma unroll
+                for (int cc = 0; cc < CC; ++cc)
+                    if (c0 + cc * 64 * V < H) ld_vec(va[cc], pa + c0 + cc * 64 * V);
+#pragma unroll
+                for (int q = 0; q < U; ++q) {
+                    if (j0 + q >= k) continue;
+#pragma unroll
+                    for (int cc = 0; cc < CC; ++cc) {
+                        if (c0 + cc * 64 * V >= H) continue;
+#pragma unroll
+                        for (int u = 0; u < V; ++u)
+                            acc[q] = fmaf(to_f32(va[cc].v[u]), to_f32(vb[q][cc].v[u]), acc[q]);
+                    }
+                }
+            }
+        } else {
+            for (int q = 0; q < U && j0 + q < k; ++q) {
+                const T *pb = b + (int64_t)p[j0 + q] * H;
+                for (int c = lane; c < H; c += 64) acc[q] = fmaf(to_f32(pa[c]), to_f32(pb[c]), acc[q]);
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < U; ++q) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) acc[q] += __shfl_xor(acc[q], off);
+            if (lane == 0 && j0 + q < k) dots[t * k + j0 + q] = from_f32<T>(acc[q]);
+        }
+    }
 }
 
 // ---------------------------------------------------------------- NF4
@@ -366,11 +408,12 @@ int combine_rows(const void *src, const int32_t *pos, const void *weights, void 
 
 int rows_dot(const void *a, const void *b, const int32_t *pos, void *dots, int64_t T_, int k, int H, int dtype,
              hipStream_t stream) {
-    const int64_t pairs = T_ * k;
-    if (pairs == 0) return MFL_OK;
-    const unsigned grid = (unsigned)((pairs + 3) / 4);
+    if (T_ * k == 0) return MFL_OK;
+    const size_t es = dtype_size(dtype);
+    const int vec_ok = aligned(a, 16) && aligned(b, 16) && ((size_t)H * es) % 16 == 0;
+    const unsigned grid = (unsigned)((T_ + 3) / 4);
     MFL_DISPATCH_FLOAT(dtype, T, (rows_dot_kernel<T><<<grid, 256, 0, stream>>>((const T *)a, (const T *)b, pos,
-                                                                               (T *)dots, pairs, k, H)));
+                                                                               (T *)dots, T_, k, H, vec_ok)));
     return launch_status();
 }
 
