@@ -142,3 +142,53 @@ def test_unsupported_requests_fall_back_to_the_separate_kernels():
     e = oracle.linear_fwd(to_np32(x)[rows], to_np32(wg), np.sort(sel, kind="stable"))
     g = oracle.linear_fwd(to_np32(x)[rows], to_np32(wu), np.sort(sel, kind="stable"))
     check_close(h, oracle.silu_mul_fwd_f32(e, g), 1e-4, 1e-4, "fp32 glu")
+
+
+def _random_fused_case(seed):
+    """Arbitrary per-expert row counts (empty experts, tile-edge sizes, one hot expert) and an
+    arbitrary row index (any source row may appear any number of times)."""
+    rng = np.random.default_rng(1000 + seed)
+    E = int(rng.choice([1, 2, 5, 9, 24]))
+    N = int(rng.choice([8, 40, 96, 104, 192, 200, 328]))
+    K = int(rng.choice([8, 24, 64, 72, 128, 264]))
+    kind = seed % 4
+    if kind == 0:
+        m = rng.integers(0, 12, size=E)
+    elif kind == 1:
+        m = rng.integers(0, 400, size=E)
+    elif kind == 2:
+        m = rng.integers(0, 20, size=E)
+        m[int(rng.integers(0, E))] += int(rng.integers(500, 1500))
+    else:
+        m = rng.choice([0, 1, 31, 32, 33, 319, 320, 321, 640, 641], size=E)
+    if m.sum() == 0:
+        m[0] = 3
+    R = int(m.sum())
+    div = int(rng.choice([1, 2, 8]))
+    T = max(1, R // div + int(rng.integers(0, 5)))
+    row_idx = rng.integers(0, T * div, size=R).astype(np.int32)
+    return E, N, K, torch.from_numpy(m.astype(np.int32)), T, div, torch.from_numpy(row_idx)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_shapes_gathered_and_glu(seed):
+    E, N, K, ms, T, div, row_idx = _random_fused_case(seed)
+    R = int(ms.sum())
+    what = f"seed {seed}: E={E} N={N} K={K} T={T} div={div} m_sizes={ms.tolist()}"
+    x = randn((T, K), gen(seed), 1.0, torch.bfloat16)
+    wg = randn((E, N, K), gen(seed + 1), 0.1, torch.bfloat16)
+    wu = randn((E, N, K), gen(seed + 2), 0.1, torch.bfloat16)
+    rows = (row_idx.numpy() // div).astype(np.int64)
+    xg = x[rows].contiguous()
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    y = grouped_gemm_forward_gathered(x.to(DEV), row_idx.to(DEV), div, wg.to(DEV), ms.to(DEV))
+    check_close(y, oracle.linear_fwd(to_np32(xg), to_np32(wg), sel), what=what + " gathered")
+    assert torch.equal(y, grouped_gemm_forward(xg.to(DEV), wg.to(DEV), ms.to(DEV))), what
+    h, e, g = grouped_glu_forward(x.to(DEV), wg.to(DEV), wu.to(DEV), ms.to(DEV), row_idx.to(DEV), div,
+                                  return_products=True)
+    assert torch.equal(e, y), what
+    g2 = grouped_gemm_forward(xg.to(DEV), wu.to(DEV), ms.to(DEV))
+    assert torch.equal(g, g2), what
+    assert torch.equal(h, silu_mul_forward(y, g2)), what
+    h_ref, _, _ = _oracle_glu(to_np32(xg), to_np32(wg), to_np32(wu), sel)
+    check_close(h, h_ref, 2e-2, 2e-2, what=what + " glu")
