@@ -95,6 +95,17 @@ int mfl_gemm_dx_nf4(const void *dy, const uint8_t *wq, const float *code16, cons
                     int N, int K, int E, int in_dtype, int out_dtype, float alpha, int accumulate,
                     void *stream);
 
+/* Input gradient with two terms in one kernel: dx = dy1 w1 + dy2 w2 (each term as in
+ * mfl_gemm_dx; one reduction over both, one rounding, one pass over dx).  It is the input
+ * gradient of the gated unit, de w_gate + dg w_up, which the reference forms as two products
+ * and an addition (autograd of modular_qwen3_moe_fused.py:106-108;
+ * kernels/fast_lora.py:151-152 with LoRA).  Returns MFL_ERR_UNSUPPORTED, with nothing
+ * enqueued, unless the element type is bf16, K % 64 == 0, N % 8 == 0, E <= 512 and the
+ * pointers are 16-byte aligned; the caller then calls mfl_gemm_dx twice (accumulate = 1). */
+int mfl_gemm_dx_dual(const void *dy1, const void *w1, const void *dy2, const void *w2,
+                     const void *m_sizes, int m_sizes_dtype, void *dx, int64_t R, int N, int K,
+                     int E, int in_dtype, int out_dtype, void *stream);
+
 /* ---- forward products fused with their neighbours in the sparse MLP block ---------
  * The reference names these fusions as future work (modular_qwen3_moe_fused.py:100-101,105).
  * Each call returns MFL_ERR_UNSUPPORTED, with nothing enqueued, for a request the pipelined

@@ -192,3 +192,29 @@ def test_random_shapes_gathered_and_glu(seed):
     assert torch.equal(h, silu_mul_forward(y, g2)), what
     h_ref, _, _ = _oracle_glu(to_np32(xg), to_np32(wg), to_np32(wu), sel)
     check_close(h, h_ref, 2e-2, 2e-2, what=what + " glu")
+
+
+from qwen3_moe_fused.grouped_gemm.forward_transposed import grouped_gemm_forward_transposed  # noqa: E402
+from qwen3_moe_fused.grouped_gemm.fused import grouped_gemm_forward_transposed_dual  # noqa: E402
+
+
+# dx (R, N) = dy1 (R, K) @ w1[e] + dy2 (R, K) @ w2[e], w (E, K, N)
+@pytest.mark.parametrize("R,N,K,E", [(2048, 2048, 768, 8), (700, 200, 64, 5), (300, 72, 128, 3), (33, 8, 192, 40),
+                                     (5000, 392, 64, 2), (64, 24, 72, 4)])   # the last: K % 64 != 0, two plain products
+def test_two_term_input_gradient(R, N, K, E):
+    g = gen(R + N)
+    dy1, dy2 = randn((R, K), g, 1.0, torch.bfloat16), randn((R, K), g, 1.0, torch.bfloat16)
+    w1, w2 = randn((E, K, N), g, 0.05, torch.bfloat16), randn((E, K, N), g, 0.05, torch.bfloat16)
+    ms = m_sizes_uniform(R, E, g)
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    dx = grouped_gemm_forward_transposed_dual(dy1.to(DEV), w1.to(DEV), dy2.to(DEV), w2.to(DEV), ms.to(DEV))
+    ref = (oracle.linear_bwd_input(to_np32(dy1), to_np32(w1), sel).astype(np.float64)
+           + oracle.linear_bwd_input(to_np32(dy2), to_np32(w2), sel))
+    check_close(dx, ref, what="two-term dx vs oracle")
+    # closed form: one product over the concatenated reduction
+    dx_cat = grouped_gemm_forward_transposed(torch.cat([dy1, dy2], 1).contiguous().to(DEV),
+                                             torch.cat([w1, w2], 1).contiguous().to(DEV), ms.to(DEV))
+    if K % 64 == 0:
+        assert torch.equal(dx, dx_cat), "the same reduction in the same order"
+    else:
+        check_close(dx, to_np32(dx_cat), what="two-term dx vs concatenated product")

@@ -154,6 +154,19 @@ int mfl_gemm_dx_nf4(const void *dy, const uint8_t *wq, const float *code16, cons
                             out_dtype, alpha, accumulate, (hipStream_t)stream);
 }
 
+int mfl_gemm_dx_dual(const void *dy1, const void *w1, const void *dy2, const void *w2, const void *m_sizes,
+                     int m_sizes_dtype, void *dx, int64_t R, int N, int K, int E, int in_dtype, int out_dtype,
+                     void *stream) {
+    int rc = check_gemm(dy1, w1, m_sizes, m_sizes_dtype, dx, R, N, K, E, in_dtype, out_dtype);
+    if (rc) return rc;
+    if (R > 0 && (!dy2 || !w2)) return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    const GemmFusion fu = {nullptr, 1, 0, w2, nullptr, nullptr, 0, nullptr, nullptr, dy2};
+    return gemm_bf16_pipe(MODE_DX, dy1, w1, m_sizes, m_sizes_dtype == MFL_I64, dx, R, N, K, E, out_dtype, 1.0f, 0,
+                          (hipStream_t)stream, &fu);
+}
+
 /* ---- forward products fused with their neighbours in the sparse MLP block ---- */
 
 namespace {

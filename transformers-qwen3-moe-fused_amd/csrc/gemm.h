@@ -28,6 +28,8 @@ struct GemmFusion {
     const float *code16_2, *absmax_2;
     int blocksize_2;
     void *e_out, *g_out;
+    // input gradient with two terms (DX only): dx = dy w + x2 w2, x2 and w2 shaped like dy and w
+    const void *x2;
 };
 
 // Pipelined bf16 MFMA kernels (direct global->LDS copies, multi-stage) for aligned shapes.

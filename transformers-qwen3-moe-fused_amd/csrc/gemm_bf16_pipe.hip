@@ -179,6 +179,7 @@ struct Nf4Params {
 // Fusions of the forward product with its neighbours in the sparse MLP block.
 //   Gather: row i of A is row row_idx[i] / idx_div of `a` (the replicate-and-sort of the tokens
 //   never materialises).
+//   Two-term DX: see a2 below (the input gradient of the gated unit, de w_gate + dg w_up).
 //   GLU: two weight matrices b (gate) and b2 (up) of the same shape; the output is
 //   silu(A b^T) * (A b2^T), rounded like the separate kernels round (each product to bf16, silu
 //   in fp32 to bf16, product to bf16); the two products are stored too where c_e / c_g are given.
@@ -188,6 +189,9 @@ struct FwdFusion {
     const void *b2;
     Nf4Params nf4_2;
     void *c_e, *c_g;
+    // Two-term input gradient (DX only): the reduction runs over (a, b) and then over (a2, b2),
+    // same shapes, one accumulator, one epilogue: dx = a b + a2 b2.
+    const void *a2;
 };
 
 template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODE, bool NF4, bool GLU, typename TO>
@@ -330,6 +334,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         const unsigned char *a_tile;
         const unsigned char *b_tile;
         const unsigned char *b2_tile = nullptr;
+        const unsigned char *a2_tile = nullptr;  // two-term DX: second pair of operands
         int lda, ldb;
         int64_t ldc, nf4_base = 0;
         TO *c_base;
@@ -382,11 +387,16 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             } else {
                 ldb = N;
                 b_tile = (const unsigned char *)(b + (int64_t)expert * N * K + j0);
+                if (fu.a2 != nullptr) {
+                    a2_tile = (const unsigned char *)((const bf16_t *)fu.a2 + (int64_t)i0 * lda);
+                    b2_tile = (const unsigned char *)((const bf16_t *)fu.b2 + (int64_t)expert * N * K + j0);
+                }
             }
             c_base = c;
         }
         const int red = r_end - r_begin;
-        const int KT = ceil_div(red, BK);
+        const int KT1 = ceil_div(red, BK);                                      // steps of one term
+        const int KT = MODE == MODE_DX && fu.a2 != nullptr ? 2 * KT1 : KT1;  // the host checked K % BK == 0
         const int i_lim = i_end - i0 < BM ? i_end - i0 : BM;  // valid rows (or columns) of A from the tile origin
         const int j_lim = j_end - j0 < BNH ? j_end - j0 : BNH;
 
@@ -435,16 +445,24 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         constexpr int SA_ROWS_PER_COPY = 64 / SA::kChunksPerRow;
         auto issue = [&](int kt) {
             unsigned char *st = smem + (kt % S) * STAGE_BYTES;
-            const unsigned char *pa = a_tile + kt * step_a;
-            const unsigned char *pb = b_tile + kt * step_b;
-            const unsigned char *pb2 = GLU ? b2_tile + kt * step_b : pb;
+            // step of the term that is being reduced (two-term DX: the second term follows the first)
+            int ks = kt;
+            const unsigned char *a_term = a_tile, *b_term = b_tile;
+            if (MODE == MODE_DX && kt >= KT1) {
+                ks = kt - KT1;
+                a_term = a2_tile;
+                b_term = b2_tile;
+            }
+            const unsigned char *pa = a_term + ks * step_a;
+            const unsigned char *pb = b_term + ks * step_b;
+            const unsigned char *pb2 = GLU ? b2_tile + ks * step_b : pb;
             // weight matrix of the wave's q-th copy (wave-uniform)
             auto b_src = [&](int q) { return GLU && glu_up((wave * LB + q) * (64 / SB::kChunksPerRow)) ? pb2 : pb; };
             // The last step may be partial.  Reduction-strided operand: lanes whose row lies past
             // the end re-read the last valid row (in DW those rows of A are zeroed in LDS before
             // use; in DX they meet zeros of A).  Reduction-contiguous operand: chunks past the
             // end of the row are copied from a chunk of zeros.
-            const bool tail = (kt + 1) * BK > red;
+            const bool tail = (ks + 1) * BK > red;
             if (!tail) {
 #pragma unroll
                 for (int q = 0; q < LA; ++q) {
@@ -468,9 +486,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 const unsigned char *p = pa + lane_off[q];
                 if (A_RC) {
                     const int c = SA::swz(SA::row_of(load, lane), SA::phys_of(load, lane));
-                    if (kt * BK + c * 8 >= red) p = (const unsigned char *)&g_zero_chunk;
+                    if (ks * BK + c * 8 >= red) p = (const unsigned char *)&g_zero_chunk;
                 } else {
-                    const int row = SA::row_of(load, lane) + kt * BK;
+                    const int row = SA::row_of(load, lane) + ks * BK;
                     if (row >= red) p -= (int64_t)(row - (red - 1)) * lda * 2;
                 }
                 __builtin_amdgcn_global_load_lds((global_void_ptr)p, (lds_void_ptr)(st + load * 1024), 16, 0, 0);
@@ -481,9 +499,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 const unsigned char *p = b_src(q) + lane_off[LA + q];
                 if (B_RC) {
                     const int c = SB::swz(SB::row_of(load, lane), SB::phys_of(load, lane));
-                    if (kt * BK + c * 8 >= red) p = (const unsigned char *)&g_zero_chunk;
+                    if (ks * BK + c * 8 >= red) p = (const unsigned char *)&g_zero_chunk;
                 } else {
-                    const int row = SB::row_of(load, lane) + kt * BK;
+                    const int row = SB::row_of(load, lane) + ks * BK;
                     if (row >= red) p -= (int64_t)(row - (red - 1)) * ldb * 2;
                 }
                 __builtin_amdgcn_global_load_lds((global_void_ptr)p, (lds_void_ptr)(st + SA::kBytes + load * 1024), 16,
@@ -865,10 +883,11 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
     TO *pc = (TO *)c;
     const int grid = device_info().cu_count / kXcd * kXcd;  // one persistent workgroup per CU
     const Nf4Params none = {nullptr, nullptr, 0};
-    const FwdFusion no_fusion = {nullptr, 1, nullptr, none, nullptr, nullptr};
+    const FwdFusion no_fusion = {nullptr, 1, nullptr, none, nullptr, nullptr, nullptr};
     const FwdFusion fu = fusion ? *fusion : no_fusion;
-    const bool glu = fu.b2 != nullptr;
+    const bool glu = fu.b2 != nullptr && fu.a2 == nullptr;
     if ((glu || fu.row_idx) && mode != MODE_FWD) return MFL_ERR_UNSUPPORTED;
+    if (fu.a2 != nullptr && (mode != MODE_DX || nf4 != nullptr || fu.b2 == nullptr)) return MFL_ERR_UNSUPPORTED;
 #define MFL_PIPE(MODE, NF4, GLU)                                                                                \
     {                                                                                                           \
         auto kern = gemm_pipe_kernel<MB, NB, BK, S, WGM, WGN, MODE, NF4, GLU, TO>;                              \
@@ -938,7 +957,7 @@ int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, i
     // Rank-r LoRA products (one side of the output at most 64 wide) are bound by streaming the
     // wide operand: small stages, many of them, so that a CU keeps 100 KiB and more in flight.
     // Products with the GLU epilogue (bit 3): the configurations whose waves along N split in two halves.
-    const bool glu = fusion != nullptr && fusion->b2 != nullptr;
+    const bool glu = fusion != nullptr && fusion->b2 != nullptr && fusion->a2 == nullptr;
     int cfg = g_pipe_config;
     if (glu && (cfg == 0 || nf4 != nullptr)) {
         cfg = R >= (int64_t)512 * E ? 8 : (R <= (int64_t)32 * E && nf4 == nullptr) ? 15 : 3;
@@ -980,7 +999,7 @@ namespace {
 // Checks the fusion request of a forward product and translates it for the kernel.
 // Returns MFL_ERR_UNSUPPORTED for what the pipelined kernels do not take.
 int make_fusion(const GemmFusion *f, int K, bool nf4, FwdFusion *out) {
-    *out = FwdFusion{nullptr, 1, nullptr, Nf4Params{nullptr, nullptr, 0}, nullptr, nullptr};
+    *out = FwdFusion{nullptr, 1, nullptr, Nf4Params{nullptr, nullptr, 0}, nullptr, nullptr, nullptr};
     if (f == nullptr) return MFL_OK;
     if (f->row_idx != nullptr) {
         // the kernel addresses the source rows with 32-bit byte offsets
@@ -988,6 +1007,15 @@ int make_fusion(const GemmFusion *f, int K, bool nf4, FwdFusion *out) {
             return MFL_ERR_UNSUPPORTED;
         out->row_idx = f->row_idx;
         out->idx_div = f->idx_div;
+    }
+    if (f->x2 != nullptr) {
+        // two-term input gradient: whole reduction steps only, bf16 weights
+        if (nf4 || f->w2 == nullptr || K % 64 != 0 || !aligned(f->x2, 16) || !aligned(f->w2, 16) ||
+            f->row_idx != nullptr)
+            return MFL_ERR_UNSUPPORTED;
+        out->a2 = f->x2;
+        out->b2 = f->w2;
+        return MFL_OK;
     }
     if (f->w2 != nullptr) {
         out->b2 = f->w2;
@@ -1016,8 +1044,9 @@ int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, 
     if (mode == MODE_DW && (N % 8 != 0 || K % 8 != 0 || N < 8 || K < 8)) return MFL_ERR_UNSUPPORTED;
     FwdFusion fu;
     if (fusion != nullptr) {
-        if (mode != MODE_FWD) return MFL_ERR_UNSUPPORTED;
-        if (fusion->w2 != nullptr && (out_dtype != MFL_BF16 || accumulate || alpha != 1.0f)) return MFL_ERR_UNSUPPORTED;
+        if (mode != (fusion->x2 != nullptr ? MODE_DX : MODE_FWD)) return MFL_ERR_UNSUPPORTED;
+        if (fusion->x2 == nullptr && fusion->w2 != nullptr && (out_dtype != MFL_BF16 || accumulate || alpha != 1.0f))
+            return MFL_ERR_UNSUPPORTED;
         const int rc = make_fusion(fusion, K, false, &fu);
         if (rc) return rc;
     }

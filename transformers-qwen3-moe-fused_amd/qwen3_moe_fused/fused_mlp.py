@@ -12,8 +12,8 @@ from __future__ import annotations
 import torch
 
 from .grouped_gemm.backward_dw import grouped_gemm_backward_dw
-from .grouped_gemm.forward_transposed import grouped_gemm_forward_transposed
-from .grouped_gemm.fused import grouped_glu_forward, grouped_glu_forward_4bit
+from .grouped_gemm.fused import (grouped_gemm_forward_transposed_dual, grouped_glu_forward,
+                                 grouped_glu_forward_4bit)
 from .kernels.routing import _combine, _gather
 from .kernels.silu_mul import silu_mul_backward
 from .grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit
@@ -37,10 +37,9 @@ class _GluGathered(torch.autograd.Function):
         de, dg = silu_mul_backward(dh.contiguous(), e, g)
         d_tokens = d_gate = d_up = None
         if ctx.needs_input_grad[0]:
-            # rows of the two input gradients are summed in the GEMM epilogue (one rounding),
-            # then each token's k rows are summed
-            dx = grouped_gemm_forward_transposed(de, w_gate, m_sizes, tokens.dtype)
-            grouped_gemm_forward_transposed(dg, w_up, m_sizes, out=dx, accumulate=True)
+            # both terms of the input gradient in one reduction (one rounding), then each token's
+            # k rows are summed
+            dx = grouped_gemm_forward_transposed_dual(de, w_gate, dg, w_up, m_sizes, tokens.dtype)
             d_tokens = _combine(dx, inv_sort_idx, None, tokens.shape[0], ctx.k)
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
             xg = _gather(tokens, sort_idx, ctx.k, None)

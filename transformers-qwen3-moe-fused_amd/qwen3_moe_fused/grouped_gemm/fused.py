@@ -157,3 +157,27 @@ def grouped_glu_forward_4bit(x: torch.Tensor, gate_quant: torch.Tensor, gate_sta
     else:
         _lib.check(rc, "mfl_glu_fwd_nf4")
     return (h, e, g) if return_products else h
+
+
+def grouped_gemm_forward_transposed_dual(dy1: torch.Tensor, w1: torch.Tensor, dy2: torch.Tensor, w2: torch.Tensor,
+                                         m_sizes: torch.Tensor, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``grouped_gemm_forward_transposed(dy1, w1, m_sizes) + grouped_gemm_forward_transposed(dy2, w2,
+    m_sizes)`` in one kernel (one reduction over both terms, one rounding): the input gradient of
+    the gated unit, ``de @ w_gate + dg @ w_up``."""
+    from .forward_transposed import grouped_gemm_forward_transposed
+
+    check_operands(m_sizes, dy1, w1, dy2, w2)
+    assert dy1.ndim == 2 and w1.ndim == 3 and dy2.shape == dy1.shape and w2.shape == w1.shape
+    rows, k = dy1.shape
+    experts, k_w, n = w1.shape
+    assert k_w == k and m_sizes.numel() == experts
+    dx = torch.empty((rows, n), device=dy1.device, dtype=dy1.dtype if dtype is None else dtype)
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_gemm_dx_dual(_lib.ptr(dy1), _lib.ptr(w1), _lib.ptr(dy2), _lib.ptr(w2), _lib.ptr(ms),
+                                     _lib.itype_code(ms.dtype), _lib.ptr(dx), rows, n, k, experts,
+                                     _lib.dtype_code(dy1.dtype), _lib.dtype_code(dx.dtype), _lib.stream())
+    if rc == UNSUPPORTED:
+        grouped_gemm_forward_transposed(dy1, w1, m_sizes, dtype, out=dx)
+        return grouped_gemm_forward_transposed(dy2, w2, m_sizes, dtype, out=dx, accumulate=True)
+    _lib.check(rc, "mfl_gemm_dx_dual")
+    return dx

@@ -23,6 +23,7 @@ from ..grouped_gemm.forward import grouped_gemm_forward as _fwd
 from ..grouped_gemm.forward_4bit import grouped_gemm_forward_4bit as _fwd4
 from ..grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit as _dx4
 from ..grouped_gemm.forward_transposed import grouped_gemm_forward_transposed as _dx
+from ..grouped_gemm.fused import grouped_gemm_forward_transposed_dual as _dx_dual
 from ..quantize.nf4 import dequantize_nf4
 from .silu_mul import silu_mul_backward_inplace, silu_mul_forward
 
@@ -96,8 +97,14 @@ class FastLora(torch.autograd.Function):
 
         dx = None
         if ctx.needs_input_grad[0]:
-            dx = _proj_bwd_input(de, tg, Gq, Gqs, Ag, Sg, m_sizes)
-            dx = _proj_bwd_input(dg, tu, Uq, Uqs, Au, Su, m_sizes, out=dx)
+            if Gqs is None and Uqs is None and dt == torch.bfloat16 and Gq.dtype == dt and Uq.dtype == dt:
+                # both base terms in one reduction, then the two rank-r terms on top
+                dx = _dx_dual(de, Gq, dg, Uq, m_sizes)
+                _dx(tg, Ag, m_sizes, out=dx, alpha=Sg, accumulate=True)
+                _dx(tu, Au, m_sizes, out=dx, alpha=Su, accumulate=True)
+            else:
+                dx = _proj_bwd_input(de, tg, Gq, Gqs, Ag, Sg, m_sizes)
+                dx = _proj_bwd_input(dg, tu, Uq, Uqs, Au, Su, m_sizes, out=dx)
 
         return (dx, None, None, dAg, dBg, None, None, None, dAu, dBu, None, None, None, dAw, dBw, None, None)
 
