@@ -177,6 +177,17 @@ int mfl_route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int 
                            int renorm, float *weights_f32, void *weights_cast, int cast_dtype,
                            int64_t *idx, void *stream);
 
+/* mfl_route_softmax_topk followed by mfl_expert_sort of its T * k selections, as ONE launch
+ * for decode-sized batches (the three launches of the separate calls cost more than their
+ * work there).  Same outputs, bit for bit: weights_f32 / weights_cast / idx as in
+ * mfl_route_softmax_topk; counts (E,), sort_idx and inv_sort_idx (T*k,) as in mfl_expert_sort
+ * (both index arrays required).  Returns MFL_ERR_UNSUPPORTED, with nothing enqueued, when
+ * T > 128, T * k > 8192, E > 512 or T == 0; the caller then makes the two separate calls.
+ * Replaces qwen3_moe_fused/modular_qwen3_moe_fused.py:87-93 + kernels/indexing.py:48-65. */
+int mfl_route_sort_small(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm,
+                         float *weights_f32, void *weights_cast, int cast_dtype, int64_t *idx,
+                         int32_t *counts, int32_t *sort_idx, int32_t *inv_sort_idx, void *stream);
+
 /* Stable counting sort of expert ids sel (R,) in [0, E):
  *   counts[e]        = #{j : sel[j] == e}
  *   sort_idx[i]      = j of the i-th row in the stable ascending order

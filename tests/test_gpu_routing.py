@@ -169,3 +169,21 @@ def test_rows_dot_against_numpy(T, k, H, dtype):
                     to_np32(b)[pos.numpy().astype(np.int64)].reshape(T, k, H).astype(np.float64))
     tol = 1e-2 if dtype == torch.bfloat16 else 1e-5
     check_close(dots, ref, tol, tol, "rows_dot")
+
+
+@pytest.mark.parametrize("T,E,k,dtype", [(16, 128, 8, torch.float32), (1, 128, 8, torch.bfloat16), (128, 128, 8, torch.bfloat16),
+                                         (7, 11, 3, torch.float32), (100, 512, 6, torch.float32), (33, 60, 1, torch.float32),
+                                         (129, 128, 8, torch.float32)])          # the last: past the limit, separate calls
+def test_route_and_sort_in_one_launch_equals_the_separate_calls(T, E, k, dtype):
+    from qwen3_moe_fused.kernels.routing import route_and_sort
+
+    logits = randn((T, E), gen(T + E), 2.0, dtype).to(DEV)
+    w, sel, m_sizes, sort_idx, inv = route_and_sort(logits, k, True, torch.bfloat16, E)
+    _, w_ref, sel_ref = softmax_topk_raw(logits, k, True, torch.bfloat16)
+    c_ref, s_ref, i_ref = get_expert_counts_and_idx(sel_ref.view(-1), E)
+    assert torch.equal(sel, sel_ref) and torch.equal(w, w_ref)
+    assert torch.equal(m_sizes, c_ref) and torch.equal(sort_idx, s_ref) and torch.equal(inv, i_ref)
+    # and against the oracle
+    c_o, s_o, i_o = oracle.expert_counts_and_idx(sel.view(-1).cpu().numpy(), E)
+    assert np.array_equal(m_sizes.cpu().numpy(), c_o) and np.array_equal(sort_idx.cpu().numpy(), s_o)
+    assert np.array_equal(inv.cpu().numpy(), i_o)

@@ -285,6 +285,17 @@ int mfl_route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int 
                               weights_cast ? cast_dtype : MFL_F32, idx, (hipStream_t)stream);
 }
 
+int mfl_route_sort_small(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, float *weights_f32,
+                         void *weights_cast, int cast_dtype, int64_t *idx, int32_t *counts, int32_t *sort_idx,
+                         int32_t *inv_sort_idx, void *stream) {
+    if (T < 0 || E <= 0 || k <= 0 || k > E || k > 64) return MFL_ERR_SHAPE;
+    if (!dtype_ok(logits_dtype) || (weights_cast && !dtype_ok(cast_dtype))) return MFL_ERR_DTYPE;
+    if (!counts || (T > 0 && (!logits || !idx))) return MFL_ERR_NULL;
+    return route_sort_small(logits, logits_dtype, T, E, k, renorm, weights_f32, weights_cast,
+                            weights_cast ? cast_dtype : MFL_F32, idx, counts, sort_idx, inv_sort_idx,
+                            (hipStream_t)stream);
+}
+
 size_t mfl_expert_sort_workspace(int64_t R, int E) { return expert_sort_workspace(R, E); }
 
 int mfl_expert_sort(const void *sel, int sel_dtype, int64_t R, int E, int32_t *counts, int32_t *sort_idx,

@@ -22,6 +22,9 @@ int nf4_quant(const void *w, int w_dtype, int64_t n, int blocksize, const float 
 
 int route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, float *w_f32,
                        void *w_cast, int cast_dtype, int64_t *idx, hipStream_t stream);
+int route_sort_small(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, float *w_f32,
+                     void *w_cast, int cast_dtype, int64_t *idx, int32_t *counts, int32_t *sort_idx,
+                     int32_t *inv_sort_idx, hipStream_t stream);
 size_t expert_sort_workspace(int64_t R, int E);
 int expert_sort(const void *sel, int is_i64, int64_t R, int E, int32_t *counts, int32_t *sort_idx,
                 int32_t *inv_sort_idx, void *workspace, size_t ws_bytes, hipStream_t stream);

@@ -14,12 +14,9 @@ namespace {
 
 // One wave per token.  Lane l holds experts l, l+64, l+128, ... (VPL of them).
 template <typename TI, typename TC, int VPL>
-__global__ __launch_bounds__(256) void softmax_topk_kernel(const TI *__restrict__ logits, int64_t T, int E, int k,
-                                                           int renorm, float *__restrict__ w_f32,
-                                                           TC *__restrict__ w_cast, int64_t *__restrict__ idx) {
-    const int lane = threadIdx.x & 63;
-    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (t >= T) return;
+__device__ __forceinline__ void topk_one_token(const TI *__restrict__ logits, int64_t t, int E, int k, int renorm,
+                                               float *__restrict__ w_f32, TC *__restrict__ w_cast,
+                                               int64_t *__restrict__ idx, int lane) {
     const TI *row = logits + t * E;
 
     float p[VPL];
@@ -85,6 +82,16 @@ __global__ __launch_bounds__(256) void softmax_topk_kernel(const TI *__restrict_
         if (w_cast) w_cast[t * k + lane] = from_f32<TC>(w);
         idx[t * k + lane] = my_i;
     }
+}
+
+template <typename TI, typename TC, int VPL>
+__global__ __launch_bounds__(256) void softmax_topk_kernel(const TI *__restrict__ logits, int64_t T, int E, int k,
+                                                           int renorm, float *__restrict__ w_f32,
+                                                           TC *__restrict__ w_cast, int64_t *__restrict__ idx) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;
+    topk_one_token<TI, TC, VPL>(logits, t, E, k, renorm, w_f32, w_cast, idx, lane);
 }
 
 template <typename TI, typename TC>
@@ -203,12 +210,12 @@ __device__ __forceinline__ void segment_of(int w, int n_waves, int64_t R, int64_
     if (e > R) e = R;
 }
 
-// Whole sort in one workgroup (n_waves <= 16): the (wave, expert) table lives in LDS.
-__global__ __launch_bounds__(1024) void sort_single_kernel(const void *__restrict__ sel, int is_i64, int64_t R,
-                                                           int E, int key_bits, int32_t *__restrict__ counts,
-                                                           int32_t *__restrict__ sort_idx,
-                                                           int32_t *__restrict__ inv_sort_idx) {
-    extern __shared__ int lds[];  // [n_waves][E] table, then [E] totals
+// Whole sort in one workgroup (n_waves <= 16): the (wave, expert) table lives in LDS
+// (lds: [n_waves][E] table, then [E] totals).
+__device__ __forceinline__ void sort_single_body(const void *__restrict__ sel, int is_i64, int64_t R, int E,
+                                                 int key_bits, int32_t *__restrict__ counts,
+                                                 int32_t *__restrict__ sort_idx, int32_t *__restrict__ inv_sort_idx,
+                                                 int *lds) {
     const int n_waves = blockDim.x >> 6;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int *table = lds;
@@ -250,6 +257,33 @@ __global__ __launch_bounds__(1024) void sort_single_kernel(const void *__restric
     }
     __syncthreads();
     wave_scatter(sel, is_i64, E, sb, se, table + wave * E, totals, sort_idx, inv_sort_idx, lane);
+}
+
+__global__ __launch_bounds__(1024) void sort_single_kernel(const void *__restrict__ sel, int is_i64, int64_t R,
+                                                           int E, int key_bits, int32_t *__restrict__ counts,
+                                                           int32_t *__restrict__ sort_idx,
+                                                           int32_t *__restrict__ inv_sort_idx) {
+    extern __shared__ int lds[];
+    sort_single_body(sel, is_i64, R, E, key_bits, counts, sort_idx, inv_sort_idx, lds);
+}
+
+// Decode-sized batches: softmax + top-k of every token and the stable expert sort of the T * k
+// selections in ONE launch of one workgroup (three launches otherwise, each a few microseconds of
+// work): the waves take the tokens round robin, then sort what they wrote.
+template <typename TI, typename TC, int VPL>
+__global__ __launch_bounds__(1024) void route_sort_small_kernel(const TI *__restrict__ logits, int64_t T, int E,
+                                                                int k, int renorm, float *__restrict__ w_f32,
+                                                                TC *__restrict__ w_cast, int64_t *__restrict__ idx,
+                                                                int key_bits, int32_t *__restrict__ counts,
+                                                                int32_t *__restrict__ sort_idx,
+                                                                int32_t *__restrict__ inv_sort_idx) {
+    extern __shared__ int lds[];
+    const int lane = threadIdx.x & 63, n_waves = blockDim.x >> 6;
+    for (int64_t t = threadIdx.x >> 6; t < T; t += n_waves)
+        topk_one_token<TI, TC, VPL>(logits, t, E, k, renorm, w_f32, w_cast, idx, lane);
+    __threadfence();  // the selections are read back from memory by other waves of the workgroup
+    __syncthreads();
+    sort_single_body(idx, 1, T * k, E, key_bits, counts, sort_idx, inv_sort_idx, lds);
 }
 
 // Multi-workgroup path: count -> scan -> scatter, table in global workspace.
@@ -494,6 +528,47 @@ int route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int E, i
     int rc = MFL_ERR_DTYPE;
     MFL_DISPATCH_FLOAT(logits_dtype, TI, MFL_DISPATCH_FLOAT(cast_dtype, TC, rc = (launch_topk<TI, TC>(
         logits, T, E, k, renorm, w_f32, w_cast, idx, stream))));
+    return rc;
+}
+
+namespace {
+
+template <typename TI, typename TC>
+int launch_route_sort_small(const void *logits, int64_t T, int E, int k, int renorm, float *w_f32, void *w_cast,
+                            int64_t *idx, int32_t *counts, int32_t *sort_idx, int32_t *inv_sort_idx,
+                            hipStream_t stream) {
+    int key_bits = 0;
+    while ((1 << key_bits) < E) ++key_bits;
+    const int n_waves = 16;
+    const size_t lds = (size_t)(n_waves + 1) * E * 4;
+    const int vpl = ceil_div(E, 64);
+#define MFL_RS(V)                                                                                              \
+    route_sort_small_kernel<TI, TC, V><<<1, n_waves * 64, lds, stream>>>(                                      \
+        (const TI *)logits, T, E, k, renorm, w_f32, (TC *)w_cast, idx, key_bits, counts, sort_idx, inv_sort_idx)
+    if (vpl <= 1)
+        MFL_RS(1);
+    else if (vpl <= 2)
+        MFL_RS(2);
+    else if (vpl <= 4)
+        MFL_RS(4);
+    else
+        MFL_RS(8);
+#undef MFL_RS
+    return launch_status();
+}
+
+}  // namespace
+
+int route_sort_small(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, float *w_f32,
+                     void *w_cast, int cast_dtype, int64_t *idx, int32_t *counts, int32_t *sort_idx,
+                     int32_t *inv_sort_idx, hipStream_t stream) {
+    // one workgroup does everything: worth it only while the tokens are few
+    if (T > 128 || T * k > 8192 || E > 512 || inv_sort_idx == nullptr || sort_idx == nullptr)
+        return MFL_ERR_UNSUPPORTED;
+    if (T == 0) return MFL_ERR_UNSUPPORTED;  // the separate entry points define the empty case
+    int rc = MFL_OK;
+    MFL_DISPATCH_FLOAT(logits_dtype, TI, MFL_DISPATCH_FLOAT(cast_dtype, TC, rc = (launch_route_sort_small<TI, TC>(
+        logits, T, E, k, renorm, w_f32, w_cast, idx, counts, sort_idx, inv_sort_idx, stream))));
     return rc;
 }
 

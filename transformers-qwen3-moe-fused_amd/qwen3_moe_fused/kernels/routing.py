@@ -47,15 +47,67 @@ class _SoftmaxTopk(torch.autograd.Function):
     def backward(ctx, dw, _didx):
         # Not on the hot path (a (T, E) problem; the frozen-router LoRA recipes never reach it).
         logits, idx, w32 = ctx.saved_tensors
-        dw = dw.float()
-        p = torch.softmax(logits.float(), dim=-1)
-        if ctx.renorm:
-            # w = p_sel / s  ->  dp_sel = (dw - sum(dw * w)) / s, with s = sum(p_sel)
-            s = p.gather(1, idx).sum(dim=-1, keepdim=True)
-            dw = (dw - (dw * w32).sum(dim=-1, keepdim=True)) / s
-        dp = torch.zeros_like(p).scatter_(1, idx, dw)
-        dlogits = p * (dp - (dp * p).sum(dim=-1, keepdim=True))
-        return dlogits.to(logits.dtype), None, None, None
+        return _softmax_topk_backward(logits, idx, w32, ctx.renorm, dw), None, None, None
+
+
+def _softmax_topk_backward(logits, idx, w32, renorm, dw):
+    dw = dw.float()
+    p = torch.softmax(logits.float(), dim=-1)
+    if renorm:
+        # w = p_sel / s  ->  dp_sel = (dw - sum(dw * w)) / s, with s = sum(p_sel)
+        s = p.gather(1, idx).sum(dim=-1, keepdim=True)
+        dw = (dw - (dw * w32).sum(dim=-1, keepdim=True)) / s
+    dp = torch.zeros_like(p).scatter_(1, idx, dw)
+    dlogits = p * (dp - (dp * p).sum(dim=-1, keepdim=True))
+    return dlogits.to(logits.dtype)
+
+
+class _RouteAndSort(torch.autograd.Function):
+    """softmax + top-k and the stable expert sort of its selections.  Decode-sized batches take
+    one launch (``mfl_route_sort_small``); otherwise the two separate calls run.  Returns
+    (routing weights (T,k), expert ids (T,k) int64, m_sizes (E,), sort_idx, inv_sort_idx)."""
+
+    @staticmethod
+    def forward(ctx, logits, k, renorm, out_dtype, num_experts):
+        assert logits.is_cuda and logits.ndim == 2 and logits.is_contiguous()
+        T, E = logits.shape
+        assert E == num_experts
+        out_dtype = logits.dtype if out_dtype is None else out_dtype
+        rc = -6
+        if 0 < T <= 128:
+            w32 = torch.empty((T, k), device=logits.device, dtype=torch.float32)
+            wc = torch.empty((T, k), device=logits.device, dtype=out_dtype)
+            idx = torch.empty((T, k), device=logits.device, dtype=torch.int64)
+            buf = torch.empty(E + 2 * T * k, device=logits.device, dtype=torch.int32)
+            m_sizes, sort_idx, inv = buf[:E], buf[E:E + T * k], buf[E + T * k:]
+            rc = _lib.lib().mfl_route_sort_small(_lib.ptr(logits), _lib.dtype_code(logits.dtype), T, E, k,
+                                                 int(bool(renorm)), _lib.ptr(w32), _lib.ptr(wc),
+                                                 _lib.dtype_code(out_dtype), _lib.ptr(idx), _lib.ptr(m_sizes),
+                                                 _lib.ptr(sort_idx), _lib.ptr(inv), _lib.stream())
+            if rc != -6:  # MFL_ERR_UNSUPPORTED: fall through to the separate calls
+                _lib.check(rc, "mfl_route_sort_small")
+        if rc == -6:
+            from .indexing import get_expert_counts_and_idx
+
+            w32, wc, idx = softmax_topk_raw(logits, k, renorm, out_dtype)
+            m_sizes, sort_idx, inv = get_expert_counts_and_idx(idx.view(-1), E)
+        ctx.save_for_backward(logits, idx, w32)
+        ctx.renorm = renorm
+        ctx.mark_non_differentiable(idx, m_sizes, sort_idx, inv)
+        return wc, idx, m_sizes, sort_idx, inv
+
+    @staticmethod
+    def backward(ctx, dw, *_unused):
+        logits, idx, w32 = ctx.saved_tensors
+        return _softmax_topk_backward(logits, idx, w32, ctx.renorm, dw), None, None, None, None
+
+
+def route_and_sort(logits: torch.Tensor, k: int, renorm: bool, out_dtype: Optional[torch.dtype],
+                   num_experts: int):
+    """(routing_weights (T,k) in ``out_dtype``, selected_experts (T,k) int64, m_sizes, sort_idx,
+    inv_sort_idx): ``softmax_topk`` followed by ``get_expert_counts_and_idx`` on its selections
+    (modular_qwen3_moe_fused.py:87-93,102)."""
+    return _RouteAndSort.apply(logits, k, renorm, out_dtype, num_experts)
 
 
 def softmax_topk(logits: torch.Tensor, k: int, renorm: bool,

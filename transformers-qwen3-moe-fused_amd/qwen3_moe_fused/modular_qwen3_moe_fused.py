@@ -15,8 +15,7 @@ import torch
 from torch import nn
 
 from .functional import moe_fused_linear
-from .kernels.indexing import get_expert_counts_and_idx
-from .kernels.routing import combine_rows, gather_rows, softmax_topk
+from .kernels.routing import combine_rows, gather_rows, route_and_sort
 from .kernels.silu_mul import silu_mul
 
 
@@ -53,9 +52,8 @@ def route_tokens(block, hidden_2d: torch.Tensor):
     """Router half of the block, shared with the fast-LoRA forward: returns
     (router_logits, routing_weights (T,k), m_sizes, sort_idx, inv_sort_idx)."""
     router_logits = block.gate(hidden_2d)
-    routing_weights, selected = softmax_topk(router_logits.contiguous(), block.num_selected, block.norm_topk_prob,
-                                             hidden_2d.dtype)
-    m_sizes, sort_idx, inv_sort_idx = get_expert_counts_and_idx(selected.view(-1), block.num_experts)
+    routing_weights, _selected, m_sizes, sort_idx, inv_sort_idx = route_and_sort(
+        router_logits.contiguous(), block.num_selected, block.norm_topk_prob, hidden_2d.dtype, block.num_experts)
     return router_logits, routing_weights, m_sizes, sort_idx, inv_sort_idx
 
 
