@@ -25,8 +25,18 @@
 //
 // Shapes this kernel takes (the caller falls back to gemm_bf16_mfma.hip otherwise):
 //   N % 8 == 0, K % 8 == 0 (NF4 weights: K % BK == 0).
-// Rows or columns past a tile's valid range are loaded from a clamped (valid) address and never
-// stored; in DW the rows of the last, partial reduction step are zeroed in LDS before use.
+// Rows or columns past a tile's valid range are loaded from a clamped (valid) address (or, with
+// two stages, not copied at all) and never stored; in DW the rows of the last, partial reduction
+// step are zeroed in LDS before use.
+//
+// Variants of the same kernel:
+//   NF4 weights (FWD, DX): the packed weights travel through registers and are decoded into the
+//     weight part of the stage, one step ahead of the multiply.
+//   FWD with gathered rows: the copy of row i reads row row_idx[i] / idx_div of the source.
+//   FWD with two weight matrices (gate, up) and a silu(gate) * up epilogue.
+//   DX with two terms: the reduction runs over a second pair of operands after the first.
+// Memory hints: weights of the row-grouped products are copied non-temporal (each is read by one
+// workgroup), the output leaves with streaming stores.
 #include <type_traits>
 
 #include "common.h"
