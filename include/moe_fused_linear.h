@@ -12,8 +12,9 @@
  *     it: no synchronisation, no allocation, no host read of device data;
  *   - return value: 0 = OK, negative = argument error (MFL_ERR_*), positive =
  *     hipError_t of a failed launch;
- *   - the library keeps no mutable global state (device properties are cached
- *     read-only); calls are re-entrant.
+ *   - the library keeps no mutable global state (device properties and per-kernel launch
+ *     attributes are cached read-only at the first call, for the device that is current
+ *     then: one device per process); calls are re-entrant.
  */
 #ifndef MOE_FUSED_LINEAR_H
 #define MOE_FUSED_LINEAR_H
