@@ -26,8 +26,8 @@
 // Shapes this kernel takes (the caller falls back to gemm_bf16_mfma.hip otherwise):
 //   N % 8 == 0, K % 8 == 0 (NF4 weights: K % BK == 0).
 // Rows or columns past a tile's valid range are loaded from a clamped (valid) address (or, with
-// two stages, not copied at all) and never stored; in DW the rows of the last, partial reduction
-// step are zeroed in LDS before use.
+// two stages, not copied at all) and never stored; in DW the rows of A in the last, partial
+// reduction step are copied from a chunk of zeros.
 //
 // Variants of the same kernel:
 //   NF4 weights (FWD, DX): the packed weights travel through registers and are decoded into the
@@ -472,8 +472,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             // weight matrix of the wave's q-th copy (wave-uniform)
             auto b_src = [&](int q) { return GLU && glu_up((wave * LB + q) * (64 / SB::kChunksPerRow)) ? pb2 : pb; };
             // The last step may be partial.  Reduction-strided operand: lanes whose row lies past
-            // the end re-read the last valid row (in DW those rows of A are zeroed in LDS before
-            // use; in DX they meet zeros of A).  Reduction-contiguous operand: chunks past the
+            // the end re-read the last valid row (in DW those rows of A are copied from a chunk of
+            // zeros instead; in DX they meet zeros of A).  Reduction-contiguous operand: chunks past the
             // end of the row are copied from a chunk of zeros.
             const bool tail = (ks + 1) * BK > red;
             if (!tail) {
@@ -501,8 +501,15 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                     const int c = SA::swz(SA::row_of(load, lane), SA::phys_of(load, lane));
                     if (ks * BK + c * 8 >= red) p = (const unsigned char *)&g_zero_chunk;
                 } else {
+                    // rows past the end: zeros in DW (the rows of B that meet them are re-reads of
+                    // the last valid row: finite data), the last valid row again in DX
                     const int row = SA::row_of(load, lane) + ks * BK;
-                    if (row >= red) p -= (int64_t)(row - (red - 1)) * lda * 2;
+                    if (row >= red) {
+                        if (MODE == MODE_DW)
+                            p = (const unsigned char *)&g_zero_chunk;
+                        else
+                            p -= (int64_t)(row - (red - 1)) * lda * 2;
+                    }
                 }
                 __builtin_amdgcn_global_load_lds((global_void_ptr)p, (lds_void_ptr)(st + load * 1024), 16, 0, 0);
             }
@@ -562,15 +569,6 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 if (kt + S - 1 < KT) issue(kt + S - 1);
 
                 unsigned char *st = smem + (kt % S) * STAGE_BYTES;
-                if (MODE == MODE_DW && (kt + 1) * BK > red) {
-                    // zero the rows of A past the end of the expert (B's are multiplied by them)
-                    const int first = red - kt * BK;
-                    for (int q = tid; q < (BK - first) * SA::kChunksPerRow; q += NW * 64)
-                        *(uint4_t *)(st + first * SA::kRowBytes + q * 16) = uint4_t{0u, 0u, 0u, 0u};
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                    __builtin_amdgcn_s_barrier();
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-                }
                 const unsigned char *sa = st, *sb = st + SA::kBytes;
                 // fragments of sub-step ks+1 are fetched while sub-step ks is multiplied
                 bf16x8 fa[2][TA], fb[2][TN];
