@@ -45,6 +45,76 @@ def _event_us(fn, iters, warm, stream):
     return start.elapsed_time(stop) * 1e3 / iters
 
 
+def _kernel_tour(n, dev):
+    """N launches of each hot kernel at the shapes of configurations 2, 3 and 5, in a fixed order, with a line
+    per kernel that states its algorithmic bytes and flops per launch.  Nothing is timed: counter passes
+    (rocprofv3 --pmc) and kernel traces are taken over this."""
+    import torch
+
+    from qwen3_moe_fused.grouped_gemm.backward_dw import grouped_gemm_backward_dw
+    from qwen3_moe_fused.grouped_gemm.forward import grouped_gemm_forward
+    from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_4bit
+    from qwen3_moe_fused.grouped_gemm.forward_transposed import grouped_gemm_forward_transposed
+    from qwen3_moe_fused.grouped_gemm.fused import grouped_glu_forward
+    from qwen3_moe_fused.kernels.indexing import get_expert_counts_and_idx
+    from qwen3_moe_fused.kernels.routing import combine_rows, gather_rows, softmax_topk_raw
+    from qwen3_moe_fused.kernels.silu_mul import silu_mul_backward, silu_mul_forward
+    from qwen3_moe_fused.quantize.nf4 import dequantize_nf4, quantize_nf4
+
+    g = torch.Generator(device=dev).manual_seed(0)
+    bf = torch.bfloat16
+
+    def rnd(*shape, scale=1.0):
+        return (torch.randn(shape, device=dev, generator=g) * scale).to(bf)
+
+    logits = torch.randn((TOKENS, E), device=dev, generator=g)
+    _, rw, sel = softmax_topk_raw(logits, TOPK, True, bf)
+    m_sizes, sort_idx, inv_sort_idx = get_expert_counts_and_idx(sel.view(-1), E)
+    hidden = rnd(TOKENS, HIDDEN)
+    x = rnd(ROWS, HIDDEN)
+    w_gate, w_up = rnd(E, INTER, HIDDEN, scale=0.02), rnd(E, INTER, HIDDEN, scale=0.02)
+    w_down = rnd(E, HIDDEN, INTER, scale=0.02)
+    h, h2, dh = rnd(ROWS, INTER), rnd(ROWS, INTER), rnd(ROWS, INTER)
+    dy = rnd(ROWS, HIDDEN)
+    packed, qstate = quantize_nf4(w_gate, 64)
+    gemm_b = 2.0 * (ROWS * HIDDEN + E * INTER * HIDDEN + ROWS * INTER)
+    gemm_f = 2.0 * ROWS * INTER * HIDDEN
+    nf4_b = E * INTER * HIDDEN * (0.5 + 4.0 / 64)
+    legs = [
+        ("gemm_fwd gate_proj 4096 tokens", gemm_b, gemm_f, lambda: grouped_gemm_forward(x, w_gate, m_sizes)),
+        ("gemm_dx down_proj 4096 tokens", gemm_b, gemm_f, lambda: grouped_gemm_forward_transposed(dy, w_down, m_sizes)),
+        ("gemm_dw down_proj 4096 tokens", gemm_b, gemm_f, lambda: grouped_gemm_backward_dw(h, dy, m_sizes, bf)),
+        ("glu_fwd (gather + gate + up + SiLU-mul) 4096 tokens",
+         2.0 * (TOKENS * HIDDEN + 2 * E * INTER * HIDDEN + ROWS * INTER), 2 * gemm_f,
+         lambda: grouped_glu_forward(hidden, w_gate, w_up, m_sizes, sort_idx, TOPK)),
+        ("silu_mul_fwd 32768 rows", 3.0 * ROWS * INTER * 2, 0.0, lambda: silu_mul_forward(h, h2)),
+        ("silu_mul_bwd 32768 rows", 5.0 * ROWS * INTER * 2, 0.0, lambda: silu_mul_backward(dh, h, h2)),
+        ("gather_rows 4096 tokens", 2.0 * (TOKENS + ROWS) * HIDDEN, 0.0,
+         lambda: gather_rows(hidden, sort_idx, TOPK, inv_sort_idx)),
+        ("combine_rows 4096 tokens", 2.0 * (TOKENS + ROWS) * HIDDEN, 0.0,
+         lambda: combine_rows(dy, inv_sort_idx, rw, sort_idx)),
+        ("softmax_topk 4096 tokens", TOKENS * E * 4.0 + TOKENS * TOPK * (4 + 2 + 8), 0.0,
+         lambda: softmax_topk_raw(logits, TOPK, True, bf)),
+        ("expert_sort 32768 rows", ROWS * 8.0 + 2 * ROWS * 4 + E * 4, 0.0,
+         lambda: get_expert_counts_and_idx(sel.view(-1), E)),
+        ("nf4_dequant gate_proj", nf4_b + 2.0 * E * INTER * HIDDEN, 0.0, lambda: dequantize_nf4(packed, qstate, bf)),
+    ]
+    for tokens in (16, 256, 16384):
+        lgt = torch.randn((tokens, E), device=dev, generator=g)
+        _, _, s5 = softmax_topk_raw(lgt, TOPK, True, bf)
+        ms5, _, _ = get_expert_counts_and_idx(s5.view(-1), E)
+        x5 = rnd(tokens * TOPK, HIDDEN)
+        active = int((ms5 > 0).sum().item())
+        legs.append((f"gemm_fwd_nf4 gate_proj {tokens} tokens ({active} experts hit)",
+                     active * nf4_b / E + 2.0 * tokens * TOPK * (HIDDEN + INTER), 2.0 * tokens * TOPK * INTER * HIDDEN,
+                     lambda x5=x5, ms5=ms5: grouped_gemm_forward_4bit(x5, packed, qstate, ms5)))
+    for name, nbytes, flops, fn in legs:
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        print(f"{name}: {n} launches, algorithmic {nbytes / 1e6:.1f} MB, {flops / 1e9:.2f} GFLOP per launch", flush=True)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -55,6 +125,9 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run plain 512 MiB device copies instead (reference reading for the FETCH_SIZE / "
                          "WRITE_SIZE counters of a profiling pass)")
+    ap.add_argument("--kernel-tour", type=int, default=0, metavar="N",
+                    help="launch every hot kernel N times at the benchmark shapes, untimed, and exit "
+                         "(the program behind the per-kernel counter passes)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -87,6 +160,10 @@ def main() -> int:
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": {"bytes_read": src.numel() * 2, "bytes_written": src.numel() * 2,
                                                "launches": 5}}))
+        return 0
+
+    if args.kernel_tour > 0:
+        _kernel_tour(args.kernel_tour, dev)
         return 0
 
     # ---- synthetic inputs of config 2 (seeded on the CPU, then copied)
