@@ -59,6 +59,30 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | 0x70 | 0xF00 | ((N >> 4) << 14));
 }
 
+// One wave-wide copy of 16 bytes per lane from global memory to 1 KiB of consecutive LDS.
+// ASM: the instruction is written out by hand.  The compiler orders every transposing LDS read
+// (ds_read_b64_tr_b16) behind all copies it knows to be in flight, i.e. it waits for the stage it
+// has just requested before it reads the current one; a copy it does not see leaves the waiting
+// to the kernel's own s_waitcnt vmcnt.  M0 holds the LDS address of the wave's 1 KiB.
+template <int POLICY, bool ASM>
+__device__ __forceinline__ void copy_to_lds(const unsigned char *src, unsigned char *dst) {
+    if constexpr (ASM) {
+        const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_void_ptr)dst;
+        if constexpr (POLICY == 2)
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"
+                         :
+                         : "v"(src), "s"(lds_addr)
+                         : "memory");
+        else
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         :
+                         : "v"(src), "s"(lds_addr)
+                         : "memory");
+    } else {
+        __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)dst, 16, 0, POLICY);
+    }
+}
+
 template <int BI, int BK, bool RC>
 struct Stage {
     static constexpr int kRowBytes = RC ? BK * 2 : BI * 2;
@@ -338,16 +362,20 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
     }
     if (L_end > total) L_end = total;
 
-    for (int L = L_begin + blockIdx.x / kXcd; L < L_end; L += per_xcd) {
+    // ---- state of the tile that is being copied and multiplied (set by setup_tile)
+    int i0 = 0, i_end = 0, j0 = 0, j_end = 0, r_begin = 0, r_end = 0;
+    const unsigned char *a_tile = nullptr, *b_tile = nullptr;
+    const unsigned char *b2_tile = nullptr;
+    const unsigned char *a2_tile = nullptr;  // two-term DX: second pair of operands
+    int lda = 0, ldb = 0;
+    int64_t ldc = 0, nf4_base = 0;
+    TO *c_base = nullptr;
+    int red = 0, KT1 = 0, KT = 0, i_lim = 0, j_lim = 0, active = 0;
+    int64_t step_a = 0, step_b = 0;
+    uint32_t lane_off[LPW];
+    auto setup_tile = [&](int L) {
         // ---- tile coordinates
-        int i0, i_end, j0, j_end, r_begin, r_end;
-        const unsigned char *a_tile;
-        const unsigned char *b_tile;
-        const unsigned char *b2_tile = nullptr;
-        const unsigned char *a2_tile = nullptr;  // two-term DX: second pair of operands
-        int lda, ldb;
-        int64_t ldc, nf4_base = 0;
-        TO *c_base;
+        b2_tile = nullptr, a2_tile = nullptr, nf4_base = 0;
         if (MODE == MODE_DW) {
             const int e = L / per_expert, local = L % per_expert;
             i0 = (local / tiles_n) * BM, i_end = N;
@@ -404,15 +432,14 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             }
             c_base = c;
         }
-        const int red = r_end - r_begin;
-        const int KT1 = ceil_div(red, BK);                                      // steps of one term
-        const int KT = MODE == MODE_DX && fu.a2 != nullptr ? 2 * KT1 : KT1;  // the host checked K % BK == 0
-        const int i_lim = i_end - i0 < BM ? i_end - i0 : BM;  // valid rows (or columns) of A from the tile origin
-        const int j_lim = j_end - j0 < BNH ? j_end - j0 : BNH;
+        red = r_end - r_begin;
+        KT1 = ceil_div(red, BK);                                      // steps of one term
+        KT = MODE == MODE_DX && fu.a2 != nullptr ? 2 * KT1 : KT1;  // the host checked K % BK == 0
+        i_lim = i_end - i0 < BM ? i_end - i0 : BM;  // valid rows (or columns) of A from the tile origin
+        j_lim = j_end - j0 < BNH ? j_end - j0 : BNH;
 
         // per-lane 32-bit source offsets of this wave's copies (tile origin, reduction step 0);
         // the step advances a wave-uniform base pointer
-        uint32_t lane_off[LPW];
 #pragma unroll
         for (int q = 0; q < LA; ++q)
             lane_off[q] = (uint32_t)lane_src_offset<BM, BK, A_RC>(wave * LA + q, lane, lda, i_lim);
@@ -443,8 +470,17 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 lane_off[LA + q] = (uint32_t)lane_src_offset<BN, BK, B_RC>(wave * LB + q, lane, ldb, j_lim);
             }
         }
-        const int64_t step_a = A_RC ? (int64_t)BK * 2 : (int64_t)BK * lda * 2;
-        const int64_t step_b = B_RC ? (int64_t)BK * 2 : (int64_t)BK * ldb * 2;
+        step_a = A_RC ? (int64_t)BK * 2 : (int64_t)BK * lda * 2;
+        step_b = B_RC ? (int64_t)BK * 2 : (int64_t)BK * ldb * 2;
+        // row blocks of this wave that hold at least one valid row: blocks wm, wm+WGM, ... below
+        // ceil(i_lim / 32)
+        const int n_blocks = ceil_div(i_lim, 32);
+        active = n_blocks > wm ? ceil_div(n_blocks - wm, WGM) : 0;
+        if (active > TM) active = TM;
+    };
+
+    for (int L = L_begin + blockIdx.x / kXcd; L < L_end; L += per_xcd) {
+        setup_tile(L);
 
         // Cache policy of the weight copies in the row-grouped products: a weight is read by exactly
         // one workgroup, so it is fetched non-temporal (bit 1 of the instruction's cache-policy
@@ -455,6 +491,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         // panel (N / BM); fetching it non-temporal gains 2 % (195 -> 191.5 us); on x it costs 3 %.
         constexpr int A_POLICY = MODE == MODE_DW && NB > 2 ? 2 : 0;
         constexpr bool SKIP_A = A_RC && S == 2;
+        // products with a reduction-strided operand read it with transposing LDS reads
+        constexpr bool ASM_COPY = MODE != MODE_FWD;
         constexpr int SA_ROWS_PER_COPY = 64 / SA::kChunksPerRow;
         auto issue = [&](int kt) {
             unsigned char *st = smem + (kt % S) * STAGE_BYTES;
@@ -483,19 +521,21 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                     // is stored (with two stages every wait is for all copies, so leaving some out
                     // does not disturb the counting)
                     if (SKIP_A && (wave * LA + q) * SA_ROWS_PER_COPY >= i_lim) continue;
-                    __builtin_amdgcn_global_load_lds((global_void_ptr)(pa + lane_off[q]),
-                                                     (lds_void_ptr)(st + (wave * LA + q) * 1024), 16, 0, A_POLICY);
+                    copy_to_lds<A_POLICY, ASM_COPY>(pa + lane_off[q], st + (wave * LA + q) * 1024);
                 }
 #pragma unroll
                 for (int q = 0; q < LB; ++q)
-                    __builtin_amdgcn_global_load_lds((global_void_ptr)(b_src(q) + lane_off[LA + q]),
-                                                     (lds_void_ptr)(st + SA::kBytes + (wave * LB + q) * 1024), 16, 0,
-                                                     B_POLICY);
+                    copy_to_lds<B_POLICY, ASM_COPY>(b_src(q) + lane_off[LA + q], st + SA::kBytes + (wave * LB + q) * 1024);
                 return;
             }
+            // DW, two stages: the last step multiplies only the 16-row sub-steps that hold rows, and
+            // copies that lie wholly past them are left out (every wait is for all copies, so the
+            // counting is not disturbed)
+            const int tail_rows = MODE == MODE_DW && S == 2 ? ceil_div(red - ks * BK, 16) * 16 : BK;
 #pragma unroll
             for (int q = 0; q < LA; ++q) {
                 const int load = wave * LA + q;
+                if (MODE == MODE_DW && SA::row_of(load, 0) >= tail_rows) continue;
                 const unsigned char *p = pa + lane_off[q];
                 if (A_RC) {
                     const int c = SA::swz(SA::row_of(load, lane), SA::phys_of(load, lane));
@@ -511,11 +551,12 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                             p -= (int64_t)(row - (red - 1)) * lda * 2;
                     }
                 }
-                __builtin_amdgcn_global_load_lds((global_void_ptr)p, (lds_void_ptr)(st + load * 1024), 16, 0, 0);
+                copy_to_lds<0, ASM_COPY>(p, st + load * 1024);
             }
 #pragma unroll
             for (int q = 0; q < LB; ++q) {
                 const int load = wave * LB + q;
+                if (MODE == MODE_DW && SB::row_of(load, 0) >= tail_rows) continue;
                 const unsigned char *p = b_src(q) + lane_off[LA + q];
                 if (B_RC) {
                     const int c = SB::swz(SB::row_of(load, lane), SB::phys_of(load, lane));
@@ -524,8 +565,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                     const int row = SB::row_of(load, lane) + ks * BK;
                     if (row >= red) p -= (int64_t)(row - (red - 1)) * ldb * 2;
                 }
-                __builtin_amdgcn_global_load_lds((global_void_ptr)p, (lds_void_ptr)(st + SA::kBytes + load * 1024), 16,
-                                                 0, 0);
+                copy_to_lds<0, ASM_COPY>(p, st + SA::kBytes + load * 1024);
             }
         };
 
@@ -536,12 +576,6 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             for (int bj = 0; bj < TN; ++bj)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[t][bj][r] = 0.f;
-
-        // row blocks of this wave that hold at least one valid row: blocks wm, wm+WGM, ... below
-        // ceil(i_lim / 32)
-        const int n_blocks = ceil_div(i_lim, 32);
-        int active = n_blocks > wm ? ceil_div(n_blocks - wm, WGM) : 0;
-        if (active > TM) active = TM;
 
         // every store of the previous tile has left, every wave is done with the stages
         wait_vmcnt<0>();
@@ -557,6 +591,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         // row lane % 32 of the block, the columns 8g + 4*(lane / 32) + {0..3}, g = 0..3.
         auto k_loop = [&](auto ta_tag) {
             constexpr int TA = decltype(ta_tag)::value;
+            // The partial last step of DW multiplies only the 16-row sub-steps that hold rows.
+            const int ks_last = MODE == MODE_DW ? ceil_div(red - (KT - 1) * BK, 16) : KS;
             for (int kt = 0; kt < KT; ++kt) {
                 // step kt has landed for this wave's copies; the barrier extends that to all
                 // waves and tells us everybody finished reading step kt-1, whose stage is
@@ -570,6 +606,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 
                 unsigned char *st = smem + (kt % S) * STAGE_BYTES;
                 const unsigned char *sa = st, *sb = st + SA::kBytes;
+                const int ks_lim = MODE == MODE_DW && kt == KT - 1 ? ks_last : KS;
                 // fragments of sub-step ks+1 are fetched while sub-step ks is multiplied
                 bf16x8 fa[2][TA], fb[2][TN];
 #pragma unroll
@@ -578,6 +615,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 for (int t = 0; t < TA; ++t) fa[0][t] = fo_a.load(sa, t, 0);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
+                    if (MODE == MODE_DW && ks >= ks_lim) break;
                     if (ks + 1 < KS) {
 #pragma unroll
                         for (int bj = 0; bj < TN; ++bj) fb[(ks + 1) & 1][bj] = fo_b.load(sb, bj, ks + 1);
