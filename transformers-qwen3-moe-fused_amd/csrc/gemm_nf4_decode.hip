@@ -41,7 +41,11 @@ struct Nf4Matrix {
 // 16-byte load per step instead, the four touches of a line were four steps apart and the L1
 // had lost the line each time: 875 MB of requests to L2 per launch for 113 MB of weights and 8 MB
 // of rows at 256 tokens.
-template <bool GLU, bool SUPER, typename TO>
+// AM1 (quantisation blocks of at least 32 weights): the 32 weights of a lane and step share one
+// scale, fetched with one load instead of four.  Every lane reads its own line of the scales, so a
+// load instruction costs the L1 as many tag lookups as it has lanes, and those lookups, not bytes,
+// are what the kernel runs out of.
+template <bool GLU, bool SUPER, bool AM1, typename TO>
 __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restrict__ x,
                                                          const int32_t *__restrict__ row_idx, int idx_div,
                                                          Nf4Matrix w0, Nf4Matrix w1,
@@ -126,10 +130,12 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
         for (int cb = 0; cb < CB; ++cb) {
             const int64_t el = w_el + step_off(kt);
             if (!SUPER) s.w[cb] = *(const uint4_t *)(wq_of[cb] + (el >> 1));
-            // four scales per step whatever the block size (the same one four times when a block
-            // spans the step): a branch here would split the loop body
+            if (AM1) {
+                s.am[cb][0] = am_of[cb][el >> shift_of[cb]];
+            } else {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) s.am[cb][u] = am_of[cb][(el + 8 * u) >> shift_of[cb]];
+                for (int u = 0; u < 4; ++u) s.am[cb][u] = am_of[cb][(el + 8 * u) >> shift_of[cb]];
+            }
         }
         const uint4_t *px = (const uint4_t *)(x_row + step_off(kt));
 #pragma unroll
@@ -166,7 +172,7 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 const uint32_t w = SUPER ? sw.w[cb][d][ks] : s.w[cb][ks];
-                const float am = s.am[cb][ks];
+                const float am = AM1 ? s.am[cb][0] : s.am[cb][ks];
                 bf16x8 wf;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
@@ -304,9 +310,16 @@ int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const
     if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
     const bf16_t *px = (const bf16_t *)x;
     const bool wide = K % 256 == 0;  // 64 packed bytes per lane and super-step
-#define MFL_DECODE(GLU, SUPER, TO, Y, EO, GO)                                                                     \
-    nf4_decode_kernel<GLU, SUPER, TO><<<(unsigned)grid, 256, 0, stream>>>(px, row_idx, idx_div, w0, w1, m_sizes, \
-                                                                         ms_i64, Y, EO, GO, R, N, K, E, tiles_n)
+    const bool am1 = w0.bs_shift >= 5 && w1.bs_shift >= 5;  // one scale per lane and step
+#define MFL_DECODE(GLU, SUPER, TO, Y, EO, GO)                                                            \
+    do {                                                                                                 \
+        if (am1)                                                                                         \
+            nf4_decode_kernel<GLU, SUPER, true, TO><<<(unsigned)grid, 256, 0, stream>>>(                 \
+                px, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, tiles_n);          \
+        else                                                                                             \
+            nf4_decode_kernel<GLU, SUPER, false, TO><<<(unsigned)grid, 256, 0, stream>>>(                \
+                px, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, tiles_n);          \
+    } while (0)
     if (glu) {
         if (wide)
             MFL_DECODE(true, true, bf16_t, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out);
