@@ -35,7 +35,10 @@ def _quantised(E, N, K, blocksize, seed):
                                                (2048, 64, 128, 2, 16), (1500, 72, 192, 3, 8),
                                                # decode-sized batches (register-decode kernel), small blocks, a
                                                # column count that is not a multiple of 32
-                                               (60, 64, 128, 3, 16), (90, 72, 256, 5, 8), (200, 200, 192, 9, 32)])
+                                               (60, 64, 128, 3, 16), (90, 72, 256, 5, 8), (200, 200, 192, 9, 32),
+                                               # at most two rows per expert: the decode kernel loads the
+                                               # rows a lane per row, without its LDS stage
+                                               (10, 64, 128, 8, 16), (12, 72, 256, 6, 64)])
 def test_fused_nf4_forward(R, N, K, E, blocksize):
     packed, state, w_deq = _quantised(E, N, K, blocksize, R + N)
     g = gen(R)

@@ -9,7 +9,9 @@
 //     owns 32 consecutive weights of its column per 64-wide step: ONE 16-byte load per lane and
 //     step feeds 4 MFMAs.  The weights are decoded in registers (16-entry code table in LDS,
 //     code * absmax in fp32, one rounding to bf16) straight into the fragment layout.
-//   * the rows come the same way: lane l holds 32 consecutive elements of row l % 32 (64 bytes).
+//   * the rows are multiplied the same way: lane l holds 32 consecutive elements of row l % 32
+//     (64 bytes).  They are loaded eight lanes to a row and change hands in a 4 KiB LDS stage of
+//     the wave: a load of one row per lane costs the L1 one tag lookup per lane.
 //   * loads run DEPTH steps ahead in registers, and two or three workgroups share a CU: tens of
 //     KiB of packed weights in flight per CU.
 // The accumulator of a lane holds output row l % 32, columns 8g + 4*(l / 32) + {0..3}.
@@ -45,7 +47,7 @@ struct Nf4Matrix {
 // scale, fetched with one load instead of four.  Every lane reads its own line of the scales, so a
 // load instruction costs the L1 as many tag lookups as it has lanes, and those lookups, not bytes,
 // are what the kernel runs out of.
-template <bool GLU, bool SUPER, bool AM1, typename TO>
+template <bool GLU, bool SUPER, bool AM1, bool XSTAGE, typename TO>
 __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restrict__ x,
                                                          const int32_t *__restrict__ row_idx, int idx_div,
                                                          Nf4Matrix w0, Nf4Matrix w1,
@@ -55,6 +57,9 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
                                                          int tiles_n) {
     constexpr int CB = GLU ? 2 : 1;  // products per wave: block cb uses weight matrix cb
     __shared__ float lut[16 * CB];
+    // 4 KiB per wave: the rows of one step on their way from the layout they are loaded in (eight
+    // lanes per row) to the layout the MFMA takes them in (a lane per row and half)
+    __shared__ __attribute__((aligned(16))) unsigned char x_stage[XSTAGE ? 4 : 1][XSTAGE ? 4096 : 16];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
@@ -112,9 +117,26 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
     }
     // element offset of reduction step kt from the lane's first element
     auto step_off = [](int kt) { return SUPER ? (kt >> 2) * 256 + (kt & 3) * 32 : kt * 64; };
-    int64_t src_row = i0 + (n < rows ? n : rows - 1);
-    if (row_idx != nullptr) src_row = (uint32_t)row_idx[src_row] / (uint32_t)idx_div;
-    const bf16_t *x_row = x + src_row * K + h * (SUPER ? 128 : 32);
+    // XSTAGE (more than a row or two per expert; with fewer, the lanes of a load that reads one
+    // row per lane mostly hit the same lines anyway, and the detour costs 2 us at 16 tokens).
+    // Rows: load u of a step brings rows 8u .. 8u+7, eight lanes per row: four lanes per 64-byte
+    // piece (the piece of half 0 and the piece of half 1), so an instruction touches 8 or 16 lines
+    // instead of 64.  The lanes pass the chunks on through the wave's LDS stage (no barrier: LDS
+    // operations of one wave complete in order); chunk c of row r sits at c ^ ((r >> 1) & 7), which
+    // keeps the reads of 16 lanes in 16 different bank groups.
+    const bf16_t *x_src[4];
+    int x_wr[4], x_rd[4];
+    unsigned char *xl = x_stage[wave];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        // without the stage: lane l loads 64 bytes of row l % 32 itself, chunk u with load u
+        const int r = XSTAGE ? 8 * u + (lane >> 3) : n, p = XSTAGE ? (lane >> 2) & 1 : h, q = XSTAGE ? lane & 3 : u;
+        int64_t src_row = i0 + (r < rows ? r : rows - 1);
+        if (row_idx != nullptr) src_row = (uint32_t)row_idx[src_row] / (uint32_t)idx_div;
+        x_src[u] = x + src_row * K + p * (SUPER ? 128 : 32) + q * 8;
+        x_wr[u] = r * 128 + (((p * 4 + q) ^ ((r >> 1) & 7)) << 4);
+        x_rd[u] = n * 128 + (((h * 4 + u) ^ ((n >> 1) & 7)) << 4);
+    }
     const int KT = K / 64;
     const uint8_t *wq_of[2] = {w0.wq, w1.wq};
     const float *am_of[2] = {w0.absmax, w1.absmax};
@@ -137,9 +159,8 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
                 for (int u = 0; u < 4; ++u) s.am[cb][u] = am_of[cb][(el + 8 * u) >> shift_of[cb]];
             }
         }
-        const uint4_t *px = (const uint4_t *)(x_row + step_off(kt));
 #pragma unroll
-        for (int u = 0; u < 4; ++u) s.xs[u] = px[u];
+        for (int u = 0; u < 4; ++u) s.xs[u] = *(const uint4_t *)(x_src[u] + step_off(kt));
     };
 
     floatx16 acc[CB];
@@ -162,13 +183,17 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
     };
 
     auto multiply = [&](const Step &s, const SuperW &sw, int d) {
+        if (XSTAGE) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) *(uint4_t *)(xl + x_wr[u]) = s.xs[u];
+        }
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             union {
                 uint4_t u;
                 bf16x8 v;
             } xa;
-            xa.u = s.xs[ks];
+            xa.u = XSTAGE ? *(const uint4_t *)(xl + x_rd[ks]) : s.xs[ks];
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 const uint32_t w = SUPER ? sw.w[cb][d][ks] : s.w[cb][ks];
@@ -311,14 +336,20 @@ int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const
     const bf16_t *px = (const bf16_t *)x;
     const bool wide = K % 256 == 0;  // 64 packed bytes per lane and super-step
     const bool am1 = w0.bs_shift >= 5 && w1.bs_shift >= 5;  // one scale per lane and step
-#define MFL_DECODE(GLU, SUPER, TO, Y, EO, GO)                                                            \
-    do {                                                                                                 \
-        if (am1)                                                                                         \
-            nf4_decode_kernel<GLU, SUPER, true, TO><<<(unsigned)grid, 256, 0, stream>>>(                 \
-                px, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, tiles_n);          \
-        else                                                                                             \
-            nf4_decode_kernel<GLU, SUPER, false, TO><<<(unsigned)grid, 256, 0, stream>>>(                \
-                px, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, tiles_n);          \
+    const bool xstage = R > 2 * (int64_t)E;                   // rows change hands in LDS
+#define MFL_DECODE_K(GLU, SUPER, AM1, XS, TO, Y, EO, GO)                                        \
+    nf4_decode_kernel<GLU, SUPER, AM1, XS, TO><<<(unsigned)grid, 256, 0, stream>>>(                \
+        px, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, tiles_n)
+#define MFL_DECODE(GLU, SUPER, TO, Y, EO, GO)                                                   \
+    do {                                                                                        \
+        if (am1 && xstage)                                                                      \
+            MFL_DECODE_K(GLU, SUPER, true, true, TO, Y, EO, GO);                                \
+        else if (am1)                                                                           \
+            MFL_DECODE_K(GLU, SUPER, true, false, TO, Y, EO, GO);                               \
+        else if (xstage)                                                                        \
+            MFL_DECODE_K(GLU, SUPER, false, true, TO, Y, EO, GO);                               \
+        else                                                                                    \
+            MFL_DECODE_K(GLU, SUPER, false, false, TO, Y, EO, GO);                              \
     } while (0)
     if (glu) {
         if (wide)
@@ -337,6 +368,7 @@ int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const
             MFL_DECODE(false, false, float, (float *)y, nullptr, nullptr);
     }
 #undef MFL_DECODE
+#undef MFL_DECODE_K
     return launch_status();
 }
 
