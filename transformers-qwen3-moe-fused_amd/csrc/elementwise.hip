@@ -268,8 +268,11 @@ __global__ __launch_bounds__(256) void rows_dot_kernel(const T *a, const T *b, c
 
 // ---------------------------------------------------------------- NF4
 
-// Each thread decodes 8 packed bytes (16 elements).  blocksize is a power of two; when it is
-// >= 16 the 16 elements of a thread share one absmax.
+// Vector path (blocksize >= 8, aligned pointers): a lane decodes one packed dword (8 elements that
+// share one absmax) into one 16-byte chunk of bf16 (two of fp32), and the 64 lanes of a wave take 64
+// consecutive dwords, so a wave's loads and stores are whole contiguous runs (256 bytes in, 1 KiB
+// out per instruction); four such groups per iteration keep four loads in flight per lane.  The
+// output is written once and read by a later kernel: streaming stores.
 template <typename T>
 __global__ __launch_bounds__(256) void nf4_dequant_kernel(const uint8_t *__restrict__ wq,
                                                           const float *__restrict__ code16,
@@ -282,23 +285,41 @@ __global__ __launch_bounds__(256) void nf4_dequant_kernel(const uint8_t *__restr
     const int64_t nbytes = n / 2;
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (vec_ok) {
-        const int64_t nchunks = nbytes / 8;
-        for (int64_t q = i; q < nchunks; q += stride) {
-            const uint2_t packed = *(const uint2_t *)(wq + q * 8);
-            const float am = absmax[(q * 16) >> bs_shift];
-            T vals[16];
+        constexpr int U = 4;
+        const int64_t nchunks = nbytes / 4;  // packed dwords
+        const int lane = threadIdx.x & 63;
+        const int64_t wave = i >> 6, nwaves = stride >> 6;
+        for (int64_t base = wave * (64 * U); base < nchunks; base += nwaves * (64 * U)) {
+            uint32_t pk[U];
+            float am[U];
 #pragma unroll
-            for (int bt = 0; bt < 8; ++bt) {
-                const uint32_t word = bt < 4 ? packed.x : packed.y;
-                const uint32_t byte = (word >> (8 * (bt & 3))) & 0xffu;
-                vals[2 * bt] = from_f32<T>(code[byte >> 4] * am);
-                vals[2 * bt + 1] = from_f32<T>(code[byte & 15u] * am);
+            for (int u = 0; u < U; ++u) {
+                const int64_t c = base + u * 64 + lane;
+                if (c < nchunks) {
+                    pk[u] = __builtin_nontemporal_load((const uint32_t *)wq + c);
+                    am[u] = absmax[(c * 8) >> bs_shift];
+                }
             }
-            T *o = out + q * 16;
 #pragma unroll
-            for (int u = 0; u < 16 * (int)sizeof(T) / 16; ++u) ((uint4_t *)o)[u] = ((const uint4_t *)vals)[u];
+            for (int u = 0; u < U; ++u) {
+                const int64_t c = base + u * 64 + lane;
+                if (c >= nchunks) continue;
+                union {
+                    T e[8];
+                    uint4_t v[sizeof(T) / 2];
+                } vals;
+#pragma unroll
+                for (int bt = 0; bt < 4; ++bt) {
+                    const uint32_t byte = (pk[u] >> (8 * bt)) & 0xffu;
+                    vals.e[2 * bt] = from_f32<T>(code[byte >> 4] * am[u]);
+                    vals.e[2 * bt + 1] = from_f32<T>(code[byte & 15u] * am[u]);
+                }
+                uint4_t *o = (uint4_t *)(out + c * 8);
+#pragma unroll
+                for (int v = 0; v < (int)sizeof(T) / 2; ++v) __builtin_nontemporal_store(vals.v[v], o + v);
+            }
         }
-        i += nchunks * 8;
+        i += nchunks * 4;
     }
     for (int64_t q = i; q < nbytes; q += stride) {
         const uint32_t byte = wq[q];
@@ -422,8 +443,8 @@ int nf4_dequant(const uint8_t *wq, const float *code16, const float *absmax, int
     if (n == 0) return MFL_OK;
     const int shift = log2_exact(blocksize);
     if (shift < 1) return MFL_ERR_SHAPE;
-    const int vec_ok = aligned(wq, 8) && aligned(out, 16) && blocksize >= 16;
-    MFL_DISPATCH_FLOAT(out_dtype, T, (nf4_dequant_kernel<T><<<stream_grid(n / 16 + 1), 256, 0, stream>>>(
+    const int vec_ok = aligned(wq, 4) && aligned(out, 16) && blocksize >= 8;
+    MFL_DISPATCH_FLOAT(out_dtype, T, (nf4_dequant_kernel<T><<<stream_grid(n / 32 + 1), 256, 0, stream>>>(
                                          wq, code16, absmax, shift, (T *)out, n, vec_ok)));
     return launch_status();
 }

@@ -63,7 +63,9 @@ __device__ __forceinline__ void wait_vmcnt() {
 // ASM: the instruction is written out by hand.  The compiler orders every transposing LDS read
 // (ds_read_b64_tr_b16) behind all copies it knows to be in flight, i.e. it waits for the stage it
 // has just requested before it reads the current one; a copy it does not see leaves the waiting
-// to the kernel's own s_waitcnt vmcnt.  M0 holds the LDS address of the wave's 1 KiB.
+// to the kernel's own s_waitcnt vmcnt.  M0 holds the LDS address of the wave's 1 KiB; nothing else
+// in the kernels built with ASM uses M0 (no builtin copy, no message, no indexed move), so it is
+// set in the same statement as the copy and not saved.
 template <int POLICY, bool ASM>
 __device__ __forceinline__ void copy_to_lds(const unsigned char *src, unsigned char *dst) {
     if constexpr (ASM) {
