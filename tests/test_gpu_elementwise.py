@@ -86,6 +86,24 @@ def test_nf4_dequant_bit_exact(blocksize, dtype):
     assert n == out.numel()
 
 
+@pytest.mark.parametrize("shape,blocksize", [((5, 36, 20), 8), ((7, 40, 24), 32), ((3, 50, 14), 4), ((1, 2, 2), 2),
+                                             ((2, 1000, 264), 64)])
+def test_nf4_dequant_ragged_sizes(shape, blocksize):
+    # sizes that end inside a wave's group of packed dwords, and blocks too small for the vector path
+    w = randn(shape, gen(blocksize + shape[1]), 0.02)
+    q_ref, absmax_ref = oracle.nf4_quant(w.numpy(), blocksize)
+    for dtype in (torch.bfloat16, torch.float32):
+        state = Nf4QuantState(absmax=torch.from_numpy(absmax_ref).to(DEV), shape=shape, code=nf4_code(DEV),
+                              blocksize=blocksize, dtype=dtype)
+        out = dequantize_nf4(torch.from_numpy(q_ref).view(-1, 1).to(DEV), state)
+        assert out.shape == shape and out.dtype == dtype
+        if dtype == torch.bfloat16:
+            ref_bits = oracle.nf4_dequant(q_ref, absmax_ref, blocksize, bf16=True)
+            assert np.array_equal(_bits(out).reshape(-1), ref_bits)
+        else:
+            assert np.array_equal(out.cpu().numpy().reshape(-1), oracle.nf4_dequant(q_ref, absmax_ref, blocksize))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_nf4_quant_matches_oracle_and_round_trips(dtype):
     w = randn((4, 64, 128), gen(77), 0.02, dtype)
