@@ -271,6 +271,11 @@ def main() -> int:
                                        "fused_packed_gbs": round(packed_bytes / us_f / 1e3, 1),
                                        "fused_tflops": round(2.0 * tokens * TOPK * INTER * HIDDEN / us_f / 1e6, 1)}
         extra["nf4_gate_proj"] = nf4
+        # the dequant kernel alone: packed bytes + scales in, bf16 out (a fresh output tensor per call)
+        us = _event_us(lambda i: dequantize_nf4(packed, qstate, torch.bfloat16), 50, 100, stream)
+        b = E * INTER * HIDDEN * (0.5 + 4.0 / 64 + 2.0)
+        extra["nf4_dequant_gate_proj"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 1),
+                                          "hbm_frac": round(b / us / 1e3 / PEAK_HBM_GBS, 4)}
         # the input-gradient product on the same packed weights (seen as (E, K=768, N=2048)) at 4096 tokens
         from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit
         dyg = torch.randn((ROWS, INTER), device=dev, dtype=torch.bfloat16)
