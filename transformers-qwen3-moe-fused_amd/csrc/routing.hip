@@ -12,6 +12,27 @@ namespace {
 
 // ---------------------------------------------------------------- softmax + top-k
 
+// Maximum over the 64 lanes of a wave, the same value in every lane: data-parallel-primitive moves
+// inside the vector ALU (two quad permutes, two rotations inside each row of 16 lanes, two row
+// broadcasts), then a read of lane 63.  A butterfly of six cross-lane shuffles goes through the
+// LDS crossbar six times instead.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_max_step(float x) {
+    const int xi = __builtin_bit_cast(int, x);
+    // lanes that the move does not write keep x: max(x, x) = x
+    const int yi = __builtin_amdgcn_update_dpp(xi, xi, CTRL, ROW_MASK, 0xf, false);
+    return fmaxf(x, __builtin_bit_cast(float, yi));
+}
+__device__ __forceinline__ float wave_max_f32(float x) {
+    x = dpp_max_step<0xb1, 0xf>(x);   // quad_perm [1,0,3,2]
+    x = dpp_max_step<0x4e, 0xf>(x);   // quad_perm [2,3,0,1]
+    x = dpp_max_step<0x124, 0xf>(x);  // row_ror 4
+    x = dpp_max_step<0x128, 0xf>(x);  // row_ror 8: every lane holds the maximum of its row
+    x = dpp_max_step<0x142, 0xa>(x);  // row_bcast 15: rows 1 and 3 take in rows 0 and 2
+    x = dpp_max_step<0x143, 0xc>(x);  // row_bcast 31: rows 2 and 3 take in rows 0..1
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+}
+
 // One wave per token.  Lane l holds experts l, l+64, l+128, ... (VPL of them).
 template <typename TI, typename TC, int VPL>
 __device__ __forceinline__ void topk_one_token(const TI *__restrict__ logits, int64_t t, int E, int k, int renorm,
@@ -27,8 +48,7 @@ __device__ __forceinline__ void topk_one_token(const TI *__restrict__ logits, in
         p[v] = e < E ? to_f32(row[e]) : -INFINITY;
         mx = fmaxf(mx, p[v]);
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    mx = wave_max_f32(mx);
     float sum = 0.f;
 #pragma unroll
     for (int v = 0; v < VPL; ++v) {
@@ -57,15 +77,21 @@ __device__ __forceinline__ void topk_one_token(const TI *__restrict__ logits, in
                 bi = lane + 64 * v;
             }
         }
+        // the wave's best: the maximum, then its owner; several lanes with the same value (rare)
+        // settle for the lowest expert id the slow way
+        const float m = wave_max_f32(bp);
+        const uint64_t owners = __ballot(bp == m);
+        if (__popcll(owners) == 1) {
+            bi = __builtin_amdgcn_readlane(bi, __ffsll((unsigned long long)owners) - 1);
+        } else {
+            if (bp != m) bi = 0x7fffffff;
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float op = __shfl_xor(bp, off);
-            const int oi = __shfl_xor(bi, off);
-            if (op > bp || (op == bp && oi < bi)) {
-                bp = op;
-                bi = oi;
+            for (int off = 32; off > 0; off >>= 1) {
+                const int oi = __shfl_xor(bi, off);
+                if (oi < bi) bi = oi;
             }
         }
+        bp = m;
         // the owner retires the winner
 #pragma unroll
         for (int v = 0; v < VPL; ++v)

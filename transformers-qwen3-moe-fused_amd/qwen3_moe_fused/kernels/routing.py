@@ -62,9 +62,9 @@ def _softmax_topk_backward(logits, idx, w32, renorm, dw):
     return dlogits.to(logits.dtype)
 
 
-# Up to this many tokens, top-k and the expert sort run as one launch of one workgroup (its time
-# grows by about 0.4 us per token: 21 us at 16 tokens, 32 us at 64, 56 us at 128, against 36 us for
-# the three separate launches at any of these sizes).
+# Up to this many tokens, top-k and the expert sort run as one launch of one workgroup (with the
+# wrapper: 21 us at 16 and at 64 tokens, 35 us at 128, against 36 us for the three separate launches
+# at any of these sizes, of which about 22 us are kernel time).
 SMALL_ROUTE_MAX_TOKENS = 64
 
 
