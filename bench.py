@@ -45,6 +45,14 @@ def _event_us(fn, iters, warm, stream):
     return start.elapsed_time(stop) * 1e3 / iters
 
 
+def _event_us_median(fn, iters, warm, stream, blocks=5):
+    """Median over `blocks` timed runs of `iters` calls each: calls that are bound by the host (a few
+    microseconds of GPU work per launch) now and then hit a one-off stall of tens of milliseconds in a
+    long loop, which a single mean would spread over every call."""
+    runs = sorted(_event_us(fn, iters, warm if b == 0 else 0, stream) for b in range(blocks))
+    return runs[len(runs) // 2]
+
+
 def _kernel_tour(n, dev):
     """N launches of each hot kernel at the shapes of configurations 2, 3 and 5, in a fixed order, with a line
     per kernel that states its algorithmic bytes and flops per launch.  Nothing is timed: counter passes
@@ -260,7 +268,7 @@ def main() -> int:
             _, _, s5 = softmax_topk_raw(lgt, TOPK, True, torch.bfloat16)
             ms5, _, _ = get_expert_counts_and_idx(s5.view(-1), E)
             x5 = torch.randn((tokens * TOPK, HIDDEN), device=dev, dtype=torch.bfloat16)
-            n_it, n_wm = (20, 30) if tokens > 1000 else (50, 100)
+            n_it, n_wm = (20, 30) if tokens > 1000 else (100, 300)
             us_f = _event_us(lambda i: grouped_gemm_forward_4bit(x5, packed, qstate, ms5), n_it, n_wm, stream)
             us_u = _event_us(lambda i: grouped_gemm_forward(x5, dequantize_nf4(packed, qstate, torch.bfloat16), ms5),
                              n_it, n_wm, stream)
@@ -336,11 +344,13 @@ def main() -> int:
         with torch.no_grad():
             for tokens in (16, 256, 16384):
                 h5 = torch.randn((1, tokens, HIDDEN), device=dev, dtype=torch.bfloat16)
-                n_it = 20 if tokens > 1000 else 50
+                # short calls need a long warm-up to leave the power-management transient of a launch burst
+                n_it, n_wm = (20, 30) if tokens > 1000 else (40, 200)
+                timer = _event_us if tokens > 1000 else _event_us_median
                 blk.fuse_front = False                        # gather, gate_proj, up_proj, SiLU-mul one by one
-                us_sep = _event_us(lambda i: blk(h5), n_it, 3, stream)
+                us_sep = timer(lambda i: blk(h5), n_it, n_wm, stream)
                 blk.fuse_front = True                         # the default: the four as one kernel
-                us = _event_us(lambda i: blk(h5), n_it, 3, stream)
+                us = timer(lambda i: blk(h5), n_it, n_wm, stream)
                 block[f"tokens_{tokens}"] = {"us": round(us, 1), "tokens_per_s": round(tokens / us * 1e6),
                                              "module_by_module_us": round(us_sep, 1)}
                 if tokens <= 256:
@@ -354,7 +364,7 @@ def main() -> int:
                     graph = torch.cuda.CUDAGraph()
                     with torch.cuda.graph(graph):
                         blk(h5)
-                    us_g = _event_us(lambda i: graph.replay(), n_it, 3, stream)
+                    us_g = _event_us_median(lambda i: graph.replay(), n_it, n_wm, stream)
                     block[f"tokens_{tokens}"]["hip_graph_replay_us"] = round(us_g, 1)
                     del graph
         extra["nf4_sparse_block_fwd_config5"] = block
