@@ -56,6 +56,26 @@ __device__ __forceinline__ int load_msize(const void *m_sizes, int is_i64, int e
 
 __host__ __device__ constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Inclusive prefix sum over the 64 lanes of a wave (all lanes active) on data-parallel-primitive
+// moves: a Kogge-Stone scan inside each row of 16 lanes (shifts by 1, 2, 4, 8; lanes without a
+// source add 0), then the last lane of rows 0 and 2 is added to rows 1 and 3, and lane 31 to rows
+// 2 and 3.  Six vector-ALU instructions instead of six trips through the LDS crossbar.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_add_step(int x) {
+    return x + __builtin_amdgcn_update_dpp(0, x, CTRL, ROW_MASK, 0xf, true);
+}
+__device__ __forceinline__ int wave_inclusive_scan(int x) {
+    x = dpp_add_step<0x111, 0xf>(x);  // row_shr 1
+    x = dpp_add_step<0x112, 0xf>(x);  // row_shr 2
+    x = dpp_add_step<0x114, 0xf>(x);  // row_shr 4
+    x = dpp_add_step<0x118, 0xf>(x);  // row_shr 8
+    x = dpp_add_step<0x142, 0xa>(x);  // row_bcast 15 into rows 1 and 3
+    x = dpp_add_step<0x143, 0xc>(x);  // row_bcast 31 into rows 2 and 3
+    return x;
+}
+// value of lane 63, in every lane
+__device__ __forceinline__ int wave_last(int x) { return __builtin_amdgcn_readlane(x, 63); }
+
 inline size_t dtype_size(int dt) { return dt == MFL_F32 ? 4 : 2; }
 inline bool dtype_ok(int dt) { return dt == MFL_BF16 || dt == MFL_F32 || dt == MFL_F16; }
 inline bool itype_ok(int it) { return it == MFL_I32 || it == MFL_I64; }

@@ -297,24 +297,15 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             const int m = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
             const int t = e >= E ? 0 : MODE == MODE_DW ? per_expert : m_tiles_of<BM>(m) * tiles_n;
             const int w = t * tile_work(m);
-            int minc = m, tinc = t, winc = w;
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const int om = __shfl_up(minc, off), ot = __shfl_up(tinc, off), ow = __shfl_up(winc, off);
-                if (lane >= off) {
-                    minc += om;
-                    tinc += ot;
-                    winc += ow;
-                }
-            }
+            const int minc = wave_inclusive_scan(m), tinc = wave_inclusive_scan(t), winc = wave_inclusive_scan(w);
             if (wave == 0 && e <= E) {  // entry E comes from the lane behind the last expert, or from below
                 tab_rows[e] = row_carry + minc - m;
                 tab_tiles[e] = tile_carry + tinc - t;
                 tab_work[e] = work_carry + winc - w;
             }
-            row_carry += __shfl(minc, 63);
-            tile_carry += __shfl(tinc, 63);
-            work_carry += __shfl(winc, 63);
+            row_carry += wave_last(minc);
+            tile_carry += wave_last(tinc);
+            work_carry += wave_last(winc);
         }
         if (wave == 0 && lane == 0 && E % 64 == 0) {
             tab_rows[E] = row_carry;

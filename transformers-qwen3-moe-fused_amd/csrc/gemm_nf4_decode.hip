@@ -75,15 +75,7 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
             const int e = e0 + lane;
             const int m = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
             const int t = ceil_div(m, 32);
-            int minc = m, tinc = t;
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const int om = __shfl_up(minc, off), ot = __shfl_up(tinc, off);
-                if (lane >= off) {
-                    minc += om;
-                    tinc += ot;
-                }
-            }
+            const int minc = wave_inclusive_scan(m), tinc = wave_inclusive_scan(t);
             const int tb = tile_carry + tinc - t;
             const uint64_t hits = __ballot(rt >= tb && rt < tb + t);
             if (hits) {
@@ -94,8 +86,8 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
                 t_begin = __shfl(tb, src);
                 break;
             }
-            row_carry += __shfl(minc, 63);
-            tile_carry += __shfl(tinc, 63);
+            row_carry += wave_last(minc);
+            tile_carry += wave_last(tinc);
         }
     }
     __syncthreads();  // the code table is in LDS (every wave of the workgroup takes the same path below)
