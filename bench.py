@@ -338,7 +338,7 @@ def main() -> int:
             blk.gate.weight.copy_(torch.randn(blk.gate.weight.shape) * 0.02)
             for name, (fin, fout), wsrc in (("gate_proj", (HIDDEN, INTER), ws[0]), ("up_proj", (HIDDEN, INTER), ws[1]),
                                             ("down_proj", (INTER, HIDDEN), ws[2].view(E, HIDDEN, INTER))):
-                setattr(blk, name, MoeFusedLinear4bit(fin, fout, E, weight=wsrc, quant_type="nf4", blocksize=64))
+                setattr(blk, name, MoeFusedLinear4bit(fin, fout, E, weight=wsrc, quant_type="nf4", compress_statistics=False, blocksize=64))
         blk = blk.to(dev)
         block = {}
         with torch.no_grad():

@@ -28,6 +28,9 @@ extern "C" {
 
 #define MFL_ABI_VERSION 1
 
+/* the library is built with hidden visibility: these entry points are all it exports */
+#define MFL_API __attribute__((visibility("default")))
+
 /* element types */
 #define MFL_BF16 0
 #define MFL_F32 1
@@ -45,9 +48,9 @@ extern "C" {
 #define MFL_ERR_WORKSPACE (-5)   /* workspace missing or too small                  */
 #define MFL_ERR_UNSUPPORTED (-6) /* valid request this build has no kernel for      */
 
-int mfl_abi_version(void);
+MFL_API int mfl_abi_version(void);
 /* Static, NUL-terminated description of a return code of this library. */
-const char *mfl_strerror(int code);
+MFL_API const char *mfl_strerror(int code);
 
 /* ---- grouped GEMM ---------------------------------------------------------------
  * Rows of x are grouped by expert, ascending; m_sizes[e] rows belong to expert e and
@@ -57,21 +60,21 @@ const char *mfl_strerror(int code);
 
 /* y[m, n] = sum_k w[e(m), n, k] * x[m, k];  x (R,K), w (E,N,K), y (R,N).
  * Replaces grouped_gemm_forward, qwen3_moe_fused/grouped_gemm/forward.py:116-160. */
-int mfl_gemm_fwd(const void *x, const void *w, const void *m_sizes, int m_sizes_dtype, void *y,
+MFL_API int mfl_gemm_fwd(const void *x, const void *w, const void *m_sizes, int m_sizes_dtype, void *y,
                  int64_t R, int N, int K, int E, int in_dtype, int out_dtype, float alpha,
                  int accumulate, void *stream);
 
 /* dx[m, n] = sum_k w[e(m), k, n] * dy[m, k];  dy (R,K), w (E,K,N), dx (R,N).
  * Replaces grouped_gemm_forward_transposed,
  * qwen3_moe_fused/grouped_gemm/forward_transposed.py:107-151. */
-int mfl_gemm_dx(const void *dy, const void *w, const void *m_sizes, int m_sizes_dtype, void *dx,
+MFL_API int mfl_gemm_dx(const void *dy, const void *w, const void *m_sizes, int m_sizes_dtype, void *dx,
                 int64_t R, int N, int K, int E, int in_dtype, int out_dtype, float alpha,
                 int accumulate, void *stream);
 
 /* dw[e, n, k] = sum_{m in e} dy[m, n] * x[m, k];  x (R,K), dy (R,N), dw (E,N,K).
  * Every element of dw is written; experts without rows get exact zeros.
  * Replaces grouped_gemm_backward_dw, qwen3_moe_fused/grouped_gemm/backward_dw.py:92-134. */
-int mfl_gemm_dw(const void *x, const void *dy, const void *m_sizes, int m_sizes_dtype, void *dw,
+MFL_API int mfl_gemm_dw(const void *x, const void *dy, const void *m_sizes, int m_sizes_dtype, void *dw,
                 int64_t R, int N, int K, int E, int in_dtype, int out_dtype, float alpha,
                 int accumulate, void *stream);
 
@@ -80,7 +83,7 @@ int mfl_gemm_dw(const void *x, const void *dy, const void *m_sizes, int m_sizes_
  * in_dtype; byte i of wq holds element 2i in its high nibble, 2i+1 in its low nibble.
  * code16 (16 floats) and absmax (E*N*K/blocksize floats) are device pointers.
  * Replaces grouped_gemm_forward_4bit, qwen3_moe_fused/grouped_gemm/forward_4bit.py:135-208. */
-int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, const float *absmax,
+MFL_API int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, const float *absmax,
                      int blocksize, const void *m_sizes, int m_sizes_dtype, void *y, int64_t R,
                      int N, int K, int E, int in_dtype, int out_dtype, void *stream);
 
@@ -91,7 +94,7 @@ int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, cons
  * autograd).  Returns MFL_ERR_UNSUPPORTED, with nothing enqueued, unless the element type is
  * bf16, K % 64 == 0, N % 32 == 0, blocksize >= 8, E <= 512 and the pointers are 16-byte
  * aligned; the caller then dequantises (mfl_nf4_dequant) and calls mfl_gemm_dx. */
-int mfl_gemm_dx_nf4(const void *dy, const uint8_t *wq, const float *code16, const float *absmax,
+MFL_API int mfl_gemm_dx_nf4(const void *dy, const uint8_t *wq, const float *code16, const float *absmax,
                     int blocksize, const void *m_sizes, int m_sizes_dtype, void *dx, int64_t R,
                     int N, int K, int E, int in_dtype, int out_dtype, float alpha, int accumulate,
                     void *stream);
@@ -103,7 +106,7 @@ int mfl_gemm_dx_nf4(const void *dy, const uint8_t *wq, const float *code16, cons
  * kernels/fast_lora.py:151-152 with LoRA).  Returns MFL_ERR_UNSUPPORTED, with nothing
  * enqueued, unless the element type is bf16, K % 64 == 0, N % 8 == 0, E <= 512 and the
  * pointers are 16-byte aligned; the caller then calls mfl_gemm_dx twice (accumulate = 1). */
-int mfl_gemm_dx_dual(const void *dy1, const void *w1, const void *dy2, const void *w2,
+MFL_API int mfl_gemm_dx_dual(const void *dy1, const void *w1, const void *dy2, const void *w2,
                      const void *m_sizes, int m_sizes_dtype, void *dx, int64_t R, int N, int K,
                      int E, int in_dtype, int out_dtype, void *stream);
 
@@ -118,12 +121,12 @@ int mfl_gemm_dx_dual(const void *dy1, const void *w1, const void *dy2, const voi
  * the rows are gathered while they are copied into the kernel's staging memory, x is never
  * written.  x_src (src_rows, K); row_idx (R,) int32 with values in [0, src_rows * idx_div).
  * Replaces modular_qwen3_moe_fused.py:95-103 followed by forward.py:116-160. */
-int mfl_gemm_fwd_gather(const void *x_src, int64_t src_rows, const int32_t *row_idx, int idx_div,
+MFL_API int mfl_gemm_fwd_gather(const void *x_src, int64_t src_rows, const int32_t *row_idx, int idx_div,
                         const void *w, const void *m_sizes, int m_sizes_dtype, void *y, int64_t R,
                         int N, int K, int E, int in_dtype, int out_dtype, void *stream);
 
 /* The same with NF4 weights (see mfl_gemm_fwd_nf4). */
-int mfl_gemm_fwd_nf4_gather(const void *x_src, int64_t src_rows, const int32_t *row_idx,
+MFL_API int mfl_gemm_fwd_nf4_gather(const void *x_src, int64_t src_rows, const int32_t *row_idx,
                             int idx_div, const uint8_t *wq, const float *code16,
                             const float *absmax, int blocksize, const void *m_sizes,
                             int m_sizes_dtype, void *y, int64_t R, int N, int K, int E,
@@ -136,13 +139,13 @@ int mfl_gemm_fwd_nf4_gather(const void *x_src, int64_t src_rows, const int32_t *
  * (a training step needs them for the backward pass).  row_idx may be NULL: x is then (R,K)
  * and src_rows, idx_div are ignored; otherwise rows are gathered as in mfl_gemm_fwd_gather.
  * Replaces modular_qwen3_moe_fused.py:105-108 (gate_proj, up_proj, silu_mul). */
-int mfl_glu_fwd(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div,
+MFL_API int mfl_glu_fwd(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div,
                 const void *w_gate, const void *w_up, const void *m_sizes, int m_sizes_dtype,
                 void *h, void *e_out, void *g_out, int64_t R, int N, int K, int E, int dtype,
                 void *stream);
 
 /* The same with NF4 weights, each matrix with its own quantisation state. */
-int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div,
+MFL_API int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div,
                     const uint8_t *wq_gate, const float *code16_gate, const float *absmax_gate,
                     int blocksize_gate, const uint8_t *wq_up, const float *code16_up,
                     const float *absmax_up, int blocksize_up, const void *m_sizes,
@@ -154,18 +157,18 @@ int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int
 /* out[i] = code16[nibble(i)] * absmax[i / blocksize], i < n (n even).  Stands in for the
  * bitsandbytes dequantize_4bit calls at qwen3_moe_fused/quantize/layer.py:21 and
  * qwen3_moe_fused/kernels/fast_lora.py:62. */
-int mfl_nf4_dequant(const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+MFL_API int mfl_nf4_dequant(const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
                     void *out, int64_t n, int out_dtype, void *stream);
 
 /* out[i] = code256[v[i]] * absmax2[i / blocksize2] + offset  (nested absmax),
  * qwen3_moe_fused/grouped_gemm/forward_4bit.py:149-152. */
-int mfl_dequant_blockwise_u8(const uint8_t *v, const float *code256, const float *absmax2,
+MFL_API int mfl_dequant_blockwise_u8(const uint8_t *v, const float *code256, const float *absmax2,
                              int blocksize2, float offset, float *out, int64_t n, void *stream);
 
 /* Blockwise NF4 quantiser: absmax[b] = max|block b|, nibble = nearest code16 entry to
  * x / absmax (ties -> lower entry).  w has n elements of w_dtype, n % blocksize == 0.
  * Stands in for bitsandbytes quantize_4bit as used at test_moe_fused_linear.py:40. */
-int mfl_nf4_quant(const void *w, int w_dtype, int64_t n, int blocksize, const float *code16,
+MFL_API int mfl_nf4_quant(const void *w, int w_dtype, int64_t n, int blocksize, const float *code16,
                   uint8_t *wq, float *absmax, void *stream);
 
 /* ---- routing ---------------------------------------------------------------------- */
@@ -174,7 +177,7 @@ int mfl_nf4_quant(const void *w, int w_dtype, int64_t n, int blocksize, const fl
  * first; if renorm, weights /= sum(weights).  weights_f32 (T,k) and/or weights_cast (T,k) of
  * cast_dtype may be NULL; idx (T,k) int64 is required.
  * Replaces qwen3_moe_fused/modular_qwen3_moe_fused.py:87-93 (= fast_lora.py:52-58). */
-int mfl_route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int E, int k,
+MFL_API int mfl_route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int E, int k,
                            int renorm, float *weights_f32, void *weights_cast, int cast_dtype,
                            int64_t *idx, void *stream);
 
@@ -185,7 +188,7 @@ int mfl_route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int 
  * (both index arrays required).  Returns MFL_ERR_UNSUPPORTED, with nothing enqueued, when
  * T > 128, T * k > 8192, E > 512 or T == 0; the caller then makes the two separate calls.
  * Replaces qwen3_moe_fused/modular_qwen3_moe_fused.py:87-93 + kernels/indexing.py:48-65. */
-int mfl_route_sort_small(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm,
+MFL_API int mfl_route_sort_small(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm,
                          float *weights_f32, void *weights_cast, int cast_dtype, int64_t *idx,
                          int32_t *counts, int32_t *sort_idx, int32_t *inv_sort_idx, void *stream);
 
@@ -198,38 +201,38 @@ int mfl_route_sort_small(const void *logits, int logits_dtype, int64_t T, int E,
  * workspace: mfl_expert_sort_workspace(R, E) bytes of device memory, contents ignored.
  * Replaces get_expert_counts_and_idx / get_expert_counts,
  * qwen3_moe_fused/kernels/indexing.py:18-23,48-65. */
-size_t mfl_expert_sort_workspace(int64_t R, int E);
-int mfl_expert_sort(const void *sel, int sel_dtype, int64_t R, int E, int32_t *counts,
+MFL_API size_t mfl_expert_sort_workspace(int64_t R, int E);
+MFL_API int mfl_expert_sort(const void *sel, int sel_dtype, int64_t R, int E, int32_t *counts,
                     int32_t *sort_idx, int32_t *inv_sort_idx, void *workspace, size_t ws_bytes,
                     void *stream);
 
 /* dst[j, :] = src[idx[j] / idx_div, :] * (row_scale ? row_scale[idx[j]] : 1), j < R_out.
  * With idx = sort_idx and idx_div = k this is "replicate each token k times, then gather",
  * qwen3_moe_fused/modular_qwen3_moe_fused.py:95-103.  row_scale has `dtype` elements. */
-int mfl_gather_rows(const void *src, const int32_t *idx, int idx_div, const void *row_scale,
+MFL_API int mfl_gather_rows(const void *src, const int32_t *idx, int idx_div, const void *row_scale,
                     void *dst, int64_t R_out, int H, int dtype, void *stream);
 
 /* dst[t, :] = sum_{j<k} src[pos[t*k+j], :] * (weights ? weights[t*k+j] : 1), fp32 accumulate.
  * With pos = inv_sort_idx this is "un-sort, then weighted sum over the k selections",
  * qwen3_moe_fused/modular_qwen3_moe_fused.py:112-115. */
-int mfl_combine_rows(const void *src, const int32_t *pos, const void *weights, void *dst,
+MFL_API int mfl_combine_rows(const void *src, const int32_t *pos, const void *weights, void *dst,
                      int64_t T, int k, int H, int dtype, void *stream);
 
 /* dots[t*k+j] = <a[t, :], b[pos[t*k+j], :]>  (gradient of mfl_combine_rows w.r.t. weights). */
-int mfl_rows_dot(const void *a, const void *b, const int32_t *pos, void *dots, int64_t T, int k,
+MFL_API int mfl_rows_dot(const void *a, const void *b, const int32_t *pos, void *dots, int64_t T, int k,
                  int H, int dtype, void *stream);
 
 /* ---- SiLU-mul --------------------------------------------------------------------- */
 
 /* h = T(f32(e) * sigmoid(f32(e))) * g.  Replaces silu_mul_forward,
  * qwen3_moe_fused/kernels/silu_mul.py:114-125. */
-int mfl_silu_mul_fwd(const void *e, const void *g, void *h, int64_t n, int dtype, void *stream);
+MFL_API int mfl_silu_mul_fwd(const void *e, const void *g, void *h, int64_t n, int dtype, void *stream);
 
 /* de, dg (and h when h_out != NULL) from dh, e, g.  Outputs may alias inputs element for
  * element (dh->h_out, e->de, g->dg gives the reference's in-place variant).  Replaces
  * silu_mul_backward and silu_mul_backward_inplace,
  * qwen3_moe_fused/kernels/silu_mul.py:128-159. */
-int mfl_silu_mul_bwd(const void *dh, const void *e, const void *g, void *de, void *dg, void *h_out,
+MFL_API int mfl_silu_mul_bwd(const void *dh, const void *e, const void *g, void *de, void *dg, void *h_out,
                      int64_t n, int dtype, void *stream);
 
 #ifdef __cplusplus

@@ -278,3 +278,49 @@ def moe_block_fwd(hidden, gate_w, w_gate, w_up, w_down, k: int, renorm: bool, ac
 def lora_linear_fwd(x, w, a, b, scale: float, sel) -> np.ndarray:
     """lora.py:134 -- base(x) + lora_B(lora_A(x)) * scaling, per-row expert ``sel``."""
     return linear_fwd(x, w, sel) + np.float32(scale) * linear_fwd(linear_fwd(x, a, sel), b, sel)
+
+
+def lora_mlp_fwd_bwd(x, G, Ag, Bg, Sg, U, Au, Bu, Su, W, Aw, Bw, Sw, sel, dy, act_round=None):
+    """kernels/fast_lora.py:3-46 (the formulas) and :68-172 (what is materialised) -- the expert MLP
+    with LoRA on its three projections, forward and every gradient the reference returns:
+
+        e = G'x, g = U'x, h = silu(e) g, y = W'h          with P' = P + S * B A per projection
+        dh = dy W',  (h, de, dg) = silu_mul_bwd(dh, e, g),  dx = de G' + dg U'
+        dA = S (dOut B)^T In,  dB = S dOut^T (In A^T)     per projection (Out = P' In)
+
+    ``act_round`` (e.g. ``round_bf16``) is applied where the reference's low-precision run
+    materialises a tensor (:96-99, :133-152).  Returns a dict of fp32 arrays."""
+    rnd = (lambda a: a) if act_round is None else act_round
+    f = np.float32
+
+    def proj(inp, P, A, B, S):                     # mv_lora, fast_lora.py:90-94
+        u = rnd(linear_fwd(inp, A, sel))
+        return rnd(rnd(linear_fwd(inp, P, sel)) + f(S) * rnd(linear_fwd(u, B, sel))), u
+
+    def proj_t(dout, P, A, B, S):                  # vm_lora, fast_lora.py:127-131
+        t = rnd(linear_bwd_input(dout, B, sel))
+        return rnd(rnd(linear_bwd_input(dout, P, sel)) + f(S) * rnd(linear_bwd_input(t, A, sel))), t
+
+    E = G.shape[0]
+    e, ug = proj(x, G, Ag, Bg, Sg)
+    g, uu = proj(x, U, Au, Bu, Su)
+    h = rnd(silu_mul_fwd_f32(e, g)) if act_round is None else from_bf16_bits(
+        silu_mul_fwd_bf16(to_bf16_bits(e), to_bf16_bits(g)))
+    y, uw = proj(h, W, Aw, Bw, Sw)
+    dh, tw = proj_t(dy, W, Aw, Bw, Sw)
+    if act_round is None:
+        h2, de, dg = silu_mul_bwd_f32(dh, e, g)
+    else:
+        h2, de, dg = (from_bf16_bits(a) for a in silu_mul_bwd_bf16(to_bf16_bits(dh), to_bf16_bits(e), to_bf16_bits(g)))
+    tg = rnd(linear_bwd_input(de, Bg, sel))
+    tu = rnd(linear_bwd_input(dg, Bu, sel))
+    out = {
+        "y": y, "e": e, "g": g, "h": h,
+        "dAw": f(Sw) * linear_bwd_weight(tw, h2, sel, E), "dBw": f(Sw) * linear_bwd_weight(dy, uw, sel, E),
+        "dAu": f(Su) * linear_bwd_weight(tu, x, sel, E), "dBu": f(Su) * linear_bwd_weight(dg, uu, sel, E),
+        "dAg": f(Sg) * linear_bwd_weight(tg, x, sel, E), "dBg": f(Sg) * linear_bwd_weight(de, ug, sel, E),
+    }
+    dx = linear_bwd_input(de, G, sel) + f(Sg) * linear_bwd_input(tg, Ag, sel)
+    dx = dx + linear_bwd_input(dg, U, sel) + f(Su) * linear_bwd_input(tu, Au, sel)
+    out["dx"] = dx
+    return out

@@ -16,6 +16,16 @@ def _declared():
     return sorted(set(re.findall(r"\b(mfl_[a-z0-9_]+)\s*\(", text)))
 
 
+def _exported():
+    """Dynamic symbols the shared object defines (nm -D), without the per-object identifiers that
+    hipcc itself emits (__hip_cuid_*)."""
+    import subprocess
+
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], check=True, capture_output=True, text=True)
+    names = [line.split()[-1] for line in out.stdout.splitlines() if line.strip()]
+    return sorted(n for n in names if not n.startswith("__hip_"))
+
+
 def test_every_declared_symbol_is_exported_and_bound():
     names = _declared()
     assert len(names) >= 17
@@ -23,6 +33,11 @@ def test_every_declared_symbol_is_exported_and_bound():
     for n in names:
         assert hasattr(raw, n), f"{n} is declared in the header but not exported"
     assert sorted(_lib.ABI_SYMBOLS) == names, "python binding table and header disagree"
+
+
+def test_exported_symbols_are_exactly_the_declared_ones():
+    """Nothing undeclared leaves the library: no tuning hook, no internal C++ symbol."""
+    assert _exported() == _declared()
 
 
 def test_version_and_strerror():

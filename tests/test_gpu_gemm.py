@@ -118,6 +118,32 @@ def test_edge_cases_empty_and_single_expert():
     check_close(y, oracle.linear_fwd(to_np32(x), to_np32(w4), sel), what="last expert only")
 
 
+@pytest.mark.parametrize("R,N,K,E,dtype", [(600, 192, 128, 4, torch.bfloat16),   # pipelined kernel
+                                           (90, 24, 40, 3, torch.bfloat16),      # register-staged kernel
+                                           (90, 3, 16, 3, torch.float32)])       # generic kernel
+def test_rows_past_the_sum_of_m_sizes_stay_unwritten(R, N, K, E, dtype):
+    """sum(m_sizes) < R: the products cover the first sum(m_sizes) rows only; the reference's
+    wrappers leave the rest of the freshly allocated output as it is (forward.py:136)."""
+    x, w, dy, _, _ = _case(21, R, N, K, E, dtype)
+    ms = torch.full((E,), (R - 37) // E, dtype=torch.int32)
+    used = int(ms.sum())
+    assert used < R
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    rtol, atol = _tol(dtype)
+    sentinel = 12345.0
+    out = torch.full((R, N), sentinel, dtype=dtype, device=DEV)
+    grouped_gemm_forward(x.to(DEV), w.to(DEV), ms.to(DEV), out=out)
+    check_close(out[:used], oracle.linear_fwd(to_np32(x[:used]), to_np32(w), sel), rtol, atol, "fwd, used rows")
+    assert (out[used:] == sentinel).all(), "forward wrote past sum(m_sizes)"
+    dx = torch.full((R, K), sentinel, dtype=dtype, device=DEV)
+    grouped_gemm_forward_transposed(dy.to(DEV), w.to(DEV), ms.to(DEV), out=dx)
+    check_close(dx[:used], oracle.linear_bwd_input(to_np32(dy[:used]), to_np32(w), sel), rtol, atol, "dx, used rows")
+    assert (dx[used:] == sentinel).all(), "input gradient wrote past sum(m_sizes)"
+    dw = grouped_gemm_backward_dw(x.to(DEV), dy.to(DEV), ms.to(DEV), dtype)
+    exp_dw = oracle.linear_bwd_weight(to_np32(dy[:used]), to_np32(x[:used]), sel, E)
+    check_close(dw, exp_dw, rtol, atol * max(1.0, np.abs(exp_dw).max()), "dw ignores the trailing rows")
+
+
 def test_alpha_and_accumulate():
     x, w, dy, ms, sel = _case(5, 300, 64, 128, 6, torch.bfloat16)
     base = randn((300, 64), gen(6), 1.0, torch.bfloat16)

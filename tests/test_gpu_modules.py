@@ -68,6 +68,13 @@ def test_sparse_block_forward(T, E, k, H, I, dtype):
         same = (np.sort(sel_gpu, 1) == np.sort(sel_ref, 1)).all(1)
         assert same.mean() > 0.97
         check_close(out[0][torch.from_numpy(same)], out_ref[same], tol, tol, "block output")
+        # the other tokens: the two routings differ by exactly one expert, and the swapped pair's
+        # bf16 logits lie within a few units in the last place of each other
+        for t in np.nonzero(~same)[0]:
+            only_gpu, only_ref = set(sel_gpu[t]) - set(sel_ref[t]), set(sel_ref[t]) - set(sel_gpu[t])
+            assert len(only_gpu) == len(only_ref) == 1, f"token {t}: routing differs by more than one expert"
+            la, lb = float(logits_ref[t, only_gpu.pop()]), float(logits_ref[t, only_ref.pop()])
+            assert abs(la - lb) <= 2.0 ** -5 * max(abs(la), abs(lb), 1.0), f"token {t}: swapped experts are not near-tied"
     else:
         check_close(out[0], out_ref, tol, tol, "block output")
 
@@ -206,13 +213,47 @@ def test_fast_lora_block_matches_module_path(dtype, tol):
     assert qs is None and A.shape == (E, 4, H) and B.shape == (E, I, 4) and s == 4.0
 
 
+@pytest.mark.parametrize("dtype,R,E,H,M,r", [(torch.float32, 300, 5, 64, 40, 4), (torch.bfloat16, 2048, 16, 256, 96, 16),
+                                            (torch.bfloat16, 700, 8, 128, 64, 8)])
+def test_fast_lora_matches_oracle_composition(dtype, R, E, H, M, r):
+    """fast_lora (one autograd function for the expert MLP with LoRA on its three projections)
+    against the oracle's composition of the reference's formulas (kernels/fast_lora.py:3-46): the
+    output and all seven gradients, not only against the module-by-module HIP path."""
+    g = gen(R + H)
+    Sg, Su, Sw = 2.0, 0.5, 1.5
+    mk = lambda *shape, scale: randn(shape, g, scale, dtype)
+    G, U, W = mk(E, M, H, scale=0.05), mk(E, M, H, scale=0.05), mk(E, H, M, scale=0.05)
+    Ag, Bg = mk(E, r, H, scale=0.05), mk(E, M, r, scale=0.05)
+    Au, Bu = mk(E, r, H, scale=0.05), mk(E, M, r, scale=0.05)
+    Aw, Bw = mk(E, r, M, scale=0.05), mk(E, H, r, scale=0.05)
+    x, dy = mk(R, H, scale=1.0), mk(R, H, scale=1.0)
+    ms = torch.bincount(torch.randint(0, E, (R,), generator=g), minlength=E).int()
+    ms[E // 2] += ms[0]
+    ms[0] = 0                                               # one expert without rows
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    rnd = oracle.round_bf16 if dtype == torch.bfloat16 else None
+    ref = oracle.lora_mlp_fwd_bwd(to_np32(x), to_np32(G), to_np32(Ag), to_np32(Bg), Sg, to_np32(U), to_np32(Au),
+                                  to_np32(Bu), Su, to_np32(W), to_np32(Aw), to_np32(Bw), Sw, sel, to_np32(dy), rnd)
+    lora = [t.to(DEV).requires_grad_() for t in (Ag, Bg, Au, Bu, Aw, Bw)]
+    xd = x.to(DEV).requires_grad_()
+    y = fast_lora(xd, G.to(DEV), None, lora[0], lora[1], Sg, U.to(DEV), None, lora[2], lora[3], Su,
+                  W.to(DEV), None, lora[4], lora[5], Sw, ms.to(DEV))
+    y.backward(dy.to(DEV))
+    tol = 3e-2 if dtype == torch.bfloat16 else 2e-4
+    check_close(y, ref["y"], tol, tol, "fast_lora y")
+    check_close(xd.grad, ref["dx"], tol, tol * float(np.abs(ref["dx"]).max()), "fast_lora dx")
+    for t, name in zip(lora, ("dAg", "dBg", "dAu", "dBu", "dAw", "dBw")):
+        check_close(t.grad, ref[name], tol, tol * float(np.abs(ref[name]).max()), "fast_lora " + name)
+        assert torch.count_nonzero(t.grad[0]).item() == 0, "expert without rows: exact zeros"
+
+
 def test_4bit_layer_and_fast_lora_on_nf4_base():
     E, H, I, r, R = 8, 128, 64, 8, 512
     g = gen(31)
     base = MoeFusedLinear(H, I, E)
     with torch.no_grad():
         base.weight.copy_(torch.randn(base.weight.shape, generator=g) * 0.02)
-    q = MoeFusedLinear4bit(H, I, E, weight=base.weight, quant_type="nf4", blocksize=64).to(DEV)
+    q = MoeFusedLinear4bit(H, I, E, weight=base.weight, quant_type="nf4", compress_statistics=False, blocksize=64).to(DEV)
     assert q.weight.dtype == torch.uint8 and q.weight.quant_state is not None
     assert q.weight.numel() == E * I * H // 2 and not q.weight.requires_grad
     sd = q.state_dict()
@@ -241,7 +282,7 @@ def test_4bit_layer_and_fast_lora_on_nf4_base():
         m = MoeFusedLinear(in_f, out_f, E)
         with torch.no_grad():
             m.weight.copy_(torch.randn(m.weight.shape, generator=gen(seed)) * 0.05)
-        return MoeFusedLinear4bit(in_f, out_f, E, weight=m.weight, quant_type="nf4").to(DEV).weight
+        return MoeFusedLinear4bit(in_f, out_f, E, weight=m.weight, quant_type="nf4", compress_statistics=False).to(DEV).weight
 
     Gq, Uq, Wq = qbase(I, H, 1), qbase(I, H, 2), qbase(H, I, 3)
     (Ag, Bg), (Au, Bu), (Aw, Bw) = lora_params(I, H, 10), lora_params(I, H, 20), lora_params(H, I, 30)
@@ -300,7 +341,7 @@ def test_fused_front_of_block_with_4bit_projections():
     cfg = _config(E, k, H, I)
     blk = _block(cfg, torch.bfloat16, 13)
     for name, (i, o) in {"gate_proj": (H, I), "up_proj": (H, I), "down_proj": (I, H)}.items():
-        setattr(blk, name, MoeFusedLinear4bit(i, o, E, weight=getattr(blk, name).weight, quant_type="nf4"))
+        setattr(blk, name, MoeFusedLinear4bit(i, o, E, weight=getattr(blk, name).weight, quant_type="nf4", compress_statistics=False))
     blk = blk.to(DEV)
     hidden = randn((1, T, H), gen(3), 1.0, torch.bfloat16).to(DEV)
     gout = randn((1, T, H), gen(4), 1.0, torch.bfloat16).to(DEV)
@@ -352,6 +393,41 @@ def test_fused_model_matches_installed_transformers_model():
     torch.testing.assert_close(h, h_ref, rtol=1e-4, atol=1e-4)
 
 
+def test_fused_causal_lm_reports_router_logits_and_aux_loss():
+    """output_router_logits: one (tokens, experts) tensor per sparse layer, equal to that layer's
+    gate applied to its input, and a load-balancing loss that is not silently zero (the reference's
+    block hands the logits up through its return value, modular_qwen3_moe_fused.py:118; the
+    installed transformers release collects them with hooks on the router module)."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import Qwen3MoeConfig
+
+    from qwen3_moe_fused.modular_qwen3_moe_fused import Qwen3MoeFusedForCausalLM, Qwen3MoeFusedRouter
+
+    torch.manual_seed(7)
+    config = Qwen3MoeConfig(vocab_size=300, hidden_size=32, intermediate_size=24, num_hidden_layers=3,
+                            num_attention_heads=4, num_key_value_heads=2, moe_intermediate_size=16, num_experts=8,
+                            num_experts_per_tok=2, norm_topk_prob=True, mlp_only_layers=[1],
+                            output_router_logits=True, router_aux_loss_coef=0.01)
+    model = Qwen3MoeFusedForCausalLM(config).to(DEV, torch.float32).eval()
+    seen = []
+    hooks = [m.register_forward_hook(lambda mod, args, out: seen.append((args[0].detach(), out.detach())))
+             for m in model.modules() if isinstance(m, Qwen3MoeFusedRouter)]
+    assert len(hooks) == 2                                       # layers 0 and 2 are sparse, layer 1 is dense
+    ids = torch.randint(0, 300, (3, 11), generator=gen(2)).to(DEV)
+    with torch.no_grad():
+        out = model(input_ids=ids, labels=ids, output_router_logits=True)
+    for h in hooks:
+        h.remove()
+    assert out.router_logits is not None and len(out.router_logits) == 2
+    for logits, (x, recorded) in zip(out.router_logits, seen):
+        assert logits.shape == (33, 8)
+        assert torch.equal(logits, recorded)
+        torch.testing.assert_close(logits, x @ model.model.layers[0].mlp.gate.weight.t()
+                                   if recorded is seen[0][1] else x @ model.model.layers[2].mlp.gate.weight.t(),
+                                   rtol=1e-4, atol=1e-5)
+    assert out.aux_loss is not None and float(out.aux_loss) > 0.0
+
+
 @pytest.mark.parametrize("four_bit", [False, True])
 def test_block_forward_replays_from_a_hip_graph(four_bit):
     """The library only enqueues kernels (no allocation, no synchronisation, no memset), so a
@@ -362,7 +438,7 @@ def test_block_forward_replays_from_a_hip_graph(four_bit):
     blk = _block(cfg, torch.bfloat16, 17)
     if four_bit:
         for name, (i, o) in {"gate_proj": (H, I), "up_proj": (H, I), "down_proj": (I, H)}.items():
-            setattr(blk, name, MoeFusedLinear4bit(i, o, E, weight=getattr(blk, name).weight, quant_type="nf4"))
+            setattr(blk, name, MoeFusedLinear4bit(i, o, E, weight=getattr(blk, name).weight, quant_type="nf4", compress_statistics=False))
     blk = blk.to(DEV)
     static_in = randn((1, T, H), gen(0), 1.0, torch.bfloat16).to(DEV)
     with torch.no_grad():

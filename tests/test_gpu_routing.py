@@ -26,6 +26,38 @@ def _tie_free_rows(logits: np.ndarray, k: int) -> np.ndarray:
     return (gap > 1e-5).all(axis=1)
 
 
+def _check_near_tie_rows(logits: np.ndarray, idx: np.ndarray, idx_ref: np.ndarray, rows, E: int, gap=1e-5):
+    """Rows that hold a near-tie among their top k+1 probabilities: an ulp of difference between two
+    exp() implementations may order the tied experts either way.  Everything else is still fixed:
+    ids in range and distinct, and wherever the two answers differ at a position the two experts
+    named there have probabilities within `gap` (relative) of each other."""
+    p = torch.softmax(torch.from_numpy(logits).double(), -1).numpy()
+    for r in rows:
+        got, ref = idx[r], idx_ref[r]
+        assert got.min() >= 0 and got.max() < E and len(set(got.tolist())) == len(got), f"row {r}: {got}"
+        for a, b in zip(got, ref):
+            if a != b:
+                assert abs(p[r, a] - p[r, b]) <= gap * p[r, b], f"row {r}: experts {a} and {b} are not near-tied"
+
+
+def test_softmax_topk_near_ties_are_checked_too():
+    """A fixture in which every row has a near-tie inside its top k and one across the k / k+1
+    boundary (logits that differ by one fp32 ulp): ids stay in range and distinct, differ from the
+    oracle only inside a near-tied pair, and the routing weights agree on every row."""
+    T, E, k = 512, 128, 8
+    logits = randn((T, E), gen(77), 1.0).numpy()
+    order = np.argsort(-logits, axis=1)
+    rows = np.arange(T)
+    for hi, lo in ((2, 3), (k - 1, k)):                 # ranks tied inside the top k / across its edge
+        logits[rows, order[:, lo]] = np.nextafter(logits[rows, order[:, hi]], np.float32(-np.inf))
+    clear = _tie_free_rows(logits, k)
+    assert not clear.any()
+    w_ref, idx_ref = oracle.softmax_topk(logits, k, True)
+    w32, _, idx = softmax_topk_raw(torch.from_numpy(logits).to(DEV), k, True, torch.float32)
+    _check_near_tie_rows(logits, idx.cpu().numpy(), idx_ref, rows, E)
+    np.testing.assert_allclose(w32.cpu().numpy(), w_ref, rtol=2e-5, atol=1e-9)
+
+
 @pytest.mark.parametrize("T,E,k,renorm", [(256, 8, 2, False), (4096, 128, 8, True), (4096, 128, 8, False),
                                           (37, 11, 3, True), (100, 60, 4, True), (64, 256, 8, True),
                                           (16, 1000, 6, True)])
@@ -37,7 +69,9 @@ def test_softmax_topk_matches_oracle(T, E, k, renorm):
     w_ref, idx_ref = oracle.softmax_topk(lnp, k, renorm)
     w32, wc, idx = softmax_topk_raw(logits.to(DEV), k, renorm, torch.bfloat16)
     assert idx.dtype == torch.int64
-    assert np.array_equal(idx.cpu().numpy()[clear], idx_ref[clear]), "expert ids must match bit for bit"
+    idx_np = idx.cpu().numpy()
+    assert np.array_equal(idx_np[clear], idx_ref[clear]), "expert ids must match bit for bit"
+    _check_near_tie_rows(lnp, idx_np, idx_ref, np.nonzero(~clear)[0], E)
     np.testing.assert_allclose(w32.cpu().numpy(), w_ref, rtol=2e-6, atol=1e-9)
     assert torch.equal(wc, w32.to(torch.bfloat16))
 

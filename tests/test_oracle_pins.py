@@ -294,3 +294,34 @@ def test_lora_composition_equals_merged_weight():
     merged = w + s * np.einsum("enr,erk->enk", b, a)
     np.testing.assert_allclose(oracle.lora_linear_fwd(x, w, a, b, s, sel), oracle.linear_fwd(x, merged, sel),
                                rtol=1e-4, atol=1e-6)
+
+
+def test_lora_mlp_composition_matches_autograd_of_merged_weights():
+    """oracle.lora_mlp_fwd_bwd (the expert MLP with LoRA on its three projections and all its
+    gradients) against fp64 autograd of the same network written with merged weights
+    P' = P + S B A (kernels/fast_lora.py:13-19): the forward formula is not retyped with LoRA
+    terms, and no gradient formula is retyped at all."""
+    B, H, M, E, r = 90, 20, 12, 4, 3
+    Sg, Su, Sw = 0.7, 1.3, 0.5
+    g = lambda i, *s, scale=0.2: _rand(100 + i, *s, scale=scale)
+    x, dy = g(0, B, H, scale=1.0), g(1, B, H, scale=1.0)
+    G, U, W = g(2, E, M, H), g(3, E, M, H), g(4, E, H, M)
+    Ag, Bg, Au, Bu = g(5, E, r, H), g(6, E, M, r), g(7, E, r, H), g(8, E, M, r)
+    Aw, Bw = g(9, E, r, M), g(10, E, H, r)
+    sel = torch.randint(0, E, (B,), generator=torch.Generator().manual_seed(11))
+    sel = torch.sort(sel).values
+    got = oracle.lora_mlp_fwd_bwd(*(t.numpy() for t in (x, G, Ag, Bg)), Sg, *(t.numpy() for t in (U, Au, Bu)), Su,
+                                  *(t.numpy() for t in (W, Aw, Bw)), Sw, sel.numpy(), dy.numpy())
+    leaves = {n: t.double().requires_grad_() for n, t in dict(x=x, Ag=Ag, Bg=Bg, Au=Au, Bu=Bu, Aw=Aw, Bw=Bw).items()}
+    merged = lambda P, A, Bm, S: P.double() + S * torch.einsum("eor,eri->eoi", Bm, A)
+    mv = lambda Wm, v: torch.einsum("boi,bi->bo", Wm[sel], v)
+    e = mv(merged(G, leaves["Ag"], leaves["Bg"], Sg), leaves["x"])
+    gg = mv(merged(U, leaves["Au"], leaves["Bu"], Su), leaves["x"])
+    h = torch.nn.functional.silu(e) * gg
+    y = mv(merged(W, leaves["Aw"], leaves["Bw"], Sw), h)
+    y.backward(dy.double())
+    np.testing.assert_allclose(got["y"], y.detach().numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(got["h"], h.detach().numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(got["dx"], leaves["x"].grad.numpy(), rtol=1e-4, atol=1e-5)
+    for n in ("Ag", "Bg", "Au", "Bu", "Aw", "Bw"):
+        np.testing.assert_allclose(got["d" + n], leaves[n].grad.numpy(), rtol=1e-4, atol=1e-5, err_msg=n)

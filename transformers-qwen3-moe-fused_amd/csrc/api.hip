@@ -19,9 +19,6 @@ const DeviceInfo &device_info() {
     return info;
 }
 
-extern int g_mfma_config;
-extern int g_pipe_config;
-
 namespace {
 
 int check_gemm(const void *a, const void *b, const void *m_sizes, int ms_dtype, const void *c, int64_t R, int N, int K,
@@ -81,22 +78,6 @@ const char *mfl_strerror(int code) {
             return "request not supported by this build";
         default:
             return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error code";
-    }
-}
-
-/* Tuning hook (not part of the stable ABI): selects a tile configuration of the bf16 MFMA
- * kernels; 0 restores the built-in table. */
-void mfl_debug_set_mfma_config(int cfg) {
-    // 0..99: configuration of the register-staged kernels (pipelined kernels off);
-    // 100 + n: configuration n of the pipelined kernels; negative: built-in table.
-    if (cfg >= 100) {
-        g_pipe_config = cfg - 100;
-    } else if (cfg >= 0) {
-        g_pipe_config = -1;
-        g_mfma_config = cfg;
-    } else {
-        g_pipe_config = 0;
-        g_mfma_config = 0;
     }
 }
 

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/moe_fused_linear.h"
 
 namespace mfl {
@@ -85,6 +87,24 @@ inline int launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? MFL_OK : (int)e;
 }
+
+// Runs `f` (a per-device set-up call such as hipFuncSetAttribute) once for every device that a kernel
+// is launched on; safe under concurrent first calls (f must be idempotent: two threads that meet in
+// the first call on a device may both run it).
+struct PerDeviceOnce {
+    std::atomic<uint64_t> done{0};
+    template <typename F>
+    hipError_t run(F &&f) {
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        const uint64_t bit = 1ull << (dev & 63);
+        if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+        e = f();
+        if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+        return e;
+    }
+};
 
 struct DeviceInfo {
     int cu_count;

@@ -414,7 +414,14 @@ int launch_mfma(int mode, const void *a, const void *b, const void *m_sizes, int
 
 }  // namespace
 
-int g_mfma_config = 0;  // tile configuration override for tuning runs (0 = default table)
+// Tile configuration: 0 = the default below; a variable only in tuning builds.
+#ifdef MFL_TUNING_BUILD
+int g_mfma_config = 0;
+#else
+namespace {
+constexpr int g_mfma_config = 0;
+}
+#endif
 
 namespace {
 

@@ -933,13 +933,12 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
 #define MFL_PIPE(MODE, NF4, GLU)                                                                                \
     {                                                                                                           \
         auto kern = gemm_pipe_kernel<MB, NB, BK, S, WGM, WGN, MODE, NF4, GLU, TO>;                              \
-        static bool attr_set = false;                                                                           \
-        if (!attr_set) {                                                                                        \
-            hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,  \
-                                               LDS_BYTES);                                                      \
-            if (e != hipSuccess) return (int)e;                                                                 \
-            attr_set = true;                                                                                    \
-        }                                                                                                       \
+        static PerDeviceOnce attr;                                                                              \
+        const hipError_t e = attr.run([&] {                                                                     \
+            return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,          \
+                                       LDS_BYTES);                                                              \
+        });                                                                                                     \
+        if (e != hipSuccess) return (int)e;                                                                     \
         kern<<<grid, NT, LDS_BYTES, stream>>>(pa, pb, m_sizes, ms_i64, pc, R, N, K, E, alpha, accumulate,       \
                                               NF4 ? *nf4 : none, fu);                                           \
     }
@@ -978,7 +977,15 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
 
 }  // namespace
 
+// Tile configuration of every launch: 0 = the built-in table below.  A variable only in tuning builds
+// (the library proper has no switch and no mutable state here).
+#ifdef MFL_TUNING_BUILD
 int g_pipe_config = 0;
+#else
+namespace {
+constexpr int g_pipe_config = 0;
+}
+#endif
 
 namespace {
 

@@ -621,13 +621,12 @@ int expert_sort(const void *sel, int is_i64, int64_t R, int E, int32_t *counts, 
         int32_t *table = (int32_t *)workspace;
         int32_t *wg_tot = table + (size_t)n_waves * E;
         const size_t lds1 = (size_t)kFastWaves * E * 4, lds2 = (size_t)(2 * kFastWaves + 1) * E * 4;
-        static bool attr_set = false;
-        if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute((const void *)fast_scatter_kernel,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 33 * 512 * 4);
-            if (e != hipSuccess) return (int)e;
-            attr_set = true;
-        }
+        static PerDeviceOnce attr;
+        const hipError_t e = attr.run([] {
+            return hipFuncSetAttribute((const void *)fast_scatter_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       33 * 512 * 4);
+        });
+        if (e != hipSuccess) return (int)e;
         fast_count_kernel<<<n_blocks, kFastWaves * 64, lds1, stream>>>(sel, is_i64, R, E, key_bits, n_waves, table,
                                                                        wg_tot);
         int rc = launch_status();

@@ -28,7 +28,6 @@ _vp, _i, _i64, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c
 _SIGNATURES = {
     "mfl_abi_version": (_i, []),
     "mfl_strerror": (ctypes.c_char_p, [_i]),
-    "mfl_debug_set_mfma_config": (None, [_i]),
     "mfl_gemm_fwd": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "mfl_gemm_dx": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "mfl_gemm_dw": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _i, _vp]),
@@ -55,8 +54,8 @@ _SIGNATURES = {
     "mfl_silu_mul_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _vp]),
 }
 
-# entry points declared in include/moe_fused_linear.h (the debug hook is not one of them)
-ABI_SYMBOLS = tuple(n for n in _SIGNATURES if n != "mfl_debug_set_mfma_config")
+# the entry points declared in include/moe_fused_linear.h: the library exports these and nothing else
+ABI_SYMBOLS = tuple(_SIGNATURES)
 
 _lib: Optional[ctypes.CDLL] = None
 

@@ -4,7 +4,9 @@ Host wrapper over ``mfl_gemm_fwd_nf4``; contract of the reference's ``grouped_ge
 (qwen3_moe_fused/grouped_gemm/forward_4bit.py:135-208): ``w_quant`` is the packed uint8 tensor,
 ``w_quant_state`` an NF4 quant state whose ``shape`` is (E, N, K); a double-quantised absmax is
 un-nested first (:149-152); the state's own dtype is ignored and weights are rounded to
-``x.dtype`` (:103-104).
+``x.dtype`` (:103-104).  Inputs the fused kernels do not take (status UNSUPPORTED: rows that are
+not bf16, K not a multiple of 8, quantisation blocks under 8) are served by the dequantise kernel
+followed by the plain product, so the wrapper accepts what the reference's accepts.
 """
 from __future__ import annotations
 
@@ -19,7 +21,7 @@ from ._common import is_int_tensor
 
 def grouped_gemm_forward_4bit(x: torch.Tensor, w_quant: torch.Tensor, w_quant_state, m_sizes: torch.Tensor,
                               dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    assert w_quant_state.quant_type == "nf4"
+    assert w_quant_state.quant_type in ("nf4", "fp4")
     blocksize = int(w_quant_state.blocksize)
     assert blocksize > 0 and blocksize & (blocksize - 1) == 0, "blocksize must be a power of two"
     code = w_quant_state.code
@@ -47,6 +49,11 @@ def grouped_gemm_forward_4bit(x: torch.Tensor, w_quant: torch.Tensor, w_quant_st
     rc = _lib.lib().mfl_gemm_fwd_nf4(_lib.ptr(x), _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), blocksize,
                                      _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(y), rows, n, k, experts,
                                      _lib.dtype_code(x.dtype), _lib.dtype_code(y.dtype), _lib.stream())
+    if rc == -6:  # MFL_ERR_UNSUPPORTED (fp32 / fp16 rows, K % 8 != 0, blocksize < 8): dequantise, then the plain product
+        from ..quantize.nf4 import dequantize_nf4
+        from .forward import grouped_gemm_forward
+
+        return grouped_gemm_forward(x, dequantize_nf4(w_quant, w_quant_state, x.dtype), m_sizes, y.dtype)
     _lib.check(rc, "mfl_gemm_fwd_nf4")
     return y
 
@@ -62,7 +69,7 @@ def grouped_gemm_forward_transposed_4bit(dy: torch.Tensor, w_quant: torch.Tensor
     from ..quantize.nf4 import dequantize_nf4
     from .forward_transposed import grouped_gemm_forward_transposed
 
-    assert w_quant_state.quant_type == "nf4"
+    assert w_quant_state.quant_type in ("nf4", "fp4")
     blocksize = int(w_quant_state.blocksize)
     code = w_quant_state.code
     absmax = resolve_absmax(w_quant_state)

@@ -46,7 +46,7 @@ def _check_gather(x_src: torch.Tensor, row_idx: Optional[torch.Tensor], idx_div:
 
 
 def _nf4_args(w_quant: torch.Tensor, state, x: torch.Tensor, k: int):
-    assert state.quant_type == "nf4"
+    assert state.quant_type in ("nf4", "fp4")
     blocksize = int(state.blocksize)
     assert blocksize > 0 and blocksize & (blocksize - 1) == 0, "blocksize must be a power of two"
     code = state.code

@@ -57,6 +57,13 @@ def route_tokens(block, hidden_2d: torch.Tensor):
     return router_logits, routing_weights, m_sizes, sort_idx, inv_sort_idx
 
 
+class Qwen3MoeFusedRouter(nn.Linear):
+    """The block's ``gate``: a plain bias-free linear layer (modular_qwen3_moe_fused.py:72 of the
+    reference) under a class name of its own, so that transformers releases that collect
+    ``router_logits`` with a forward hook on the router module (instead of from the block's return
+    value, as the reference's release did) have a class to hook: its output is the raw logits."""
+
+
 class Qwen3MoeFusedSparseMoeBlock(nn.Module):
     """``config`` needs: num_experts, num_experts_per_tok, norm_topk_prob, hidden_size,
     moe_intermediate_size, hidden_act == "silu" (a transformers ``Qwen3MoeConfig`` has them)."""
@@ -69,7 +76,7 @@ class Qwen3MoeFusedSparseMoeBlock(nn.Module):
         self.norm_topk_prob = config.norm_topk_prob
         self.hidden_size = config.hidden_size
         self.moe_intermediate_size = config.moe_intermediate_size
-        self.gate = nn.Linear(self.hidden_size, self.num_experts, bias=False)
+        self.gate = Qwen3MoeFusedRouter(self.hidden_size, self.num_experts, bias=False)
         self.gate_proj = MoeFusedLinear(self.hidden_size, self.moe_intermediate_size, self.num_experts)
         self.up_proj = MoeFusedLinear(self.hidden_size, self.moe_intermediate_size, self.num_experts)
         self.down_proj = MoeFusedLinear(self.moe_intermediate_size, self.hidden_size, self.num_experts)
@@ -139,12 +146,26 @@ def _hf_subclasses():
             self.mlp = (block_cls(config) if sparse
                         else Qwen3MoeMLP(config, intermediate_size=config.intermediate_size))
 
+    # Releases that record outputs through forward hooks take the router logits from the stock router
+    # class; the fused block's router is hooked the same way (output_router_logits, the auxiliary
+    # load-balancing loss).  Older releases read them from the block's return value and have no table.
+    record = {}
+    if isinstance(getattr(Qwen3MoeModel, "_can_record_outputs", None), dict):
+        from transformers.utils.output_capturing import OutputRecorder
+
+        record = {"_can_record_outputs": {**Qwen3MoeModel._can_record_outputs,
+                                          "router_logits": OutputRecorder(Qwen3MoeFusedRouter, index=0)}}
+
     class Qwen3MoeFusedModel(Qwen3MoeModel):
+        locals().update(record)
+
         def __init__(self, config) -> None:
             super().__init__(config)
             self.layers = nn.ModuleList(Qwen3MoeFusedDecoderLayer(config, i) for i in range(config.num_hidden_layers))
 
     class Qwen3MoeFusedForCausalLM(Qwen3MoeForCausalLM):
+        locals().update(record)
+
         def __init__(self, config) -> None:
             super().__init__(config)
             self.model = Qwen3MoeFusedModel(config)

@@ -25,13 +25,48 @@ NF4_CODE = (
 )
 
 
+# The FP4 code book of bitsandbytes (sign, two exponent bits, one mantissa bit; values
+# 0, 0.0625, 8, 12, 4, 6, 2, 3 and their negatives, divided by 12).
+FP4_CODE = tuple(v / 12.0 for v in (0.0, 0.0625, 8.0, 12.0, 4.0, 6.0, 2.0, 3.0, -0.0, -0.0625, -8.0, -12.0, -4.0,
+                                    -6.0, -2.0, -3.0))
+
+QUANT_TYPES = ("nf4", "fp4")
+
+
 def nf4_code(device) -> torch.Tensor:
     return torch.tensor(NF4_CODE, dtype=torch.float32, device=device)
 
 
+def code_of(quant_type: str, device) -> torch.Tensor:
+    """16-entry code book of a 4-bit type; the kernels take the table as an argument."""
+    if quant_type == "nf4":
+        return nf4_code(device)
+    if quant_type == "fp4":
+        return torch.tensor(FP4_CODE, dtype=torch.float32, device=device)
+    raise NotImplementedError(f"4-bit quantisation type {quant_type!r}")
+
+
+def dynamic_map_8bit() -> torch.Tensor:
+    """The signed 8-bit "dynamic" code book that bitsandbytes uses for the second level of a
+    double quantisation (its ``create_dynamic_map(signed=True, max_exponent_bits=7, total_bits=8)``):
+    for each of seven decades 10^-6 .. 10^0, the midpoints of 2^i equal slices of [0.1, 1], both
+    signs, plus 0 and 1.  The table is stored with every quantised tensor (``nested_quant_map``),
+    so a reader never has to rebuild it."""
+    data = []
+    for i in range(7):
+        boundaries = torch.linspace(0.1, 1, 2 ** i + 1)
+        means = (boundaries[:-1] + boundaries[1:]) / 2.0
+        scale = 10.0 ** (-6 + i)
+        data += (scale * means).tolist()
+        data += (-scale * means).tolist()
+    data += [0.0, 1.0]
+    assert len(data) == 256
+    return torch.tensor(sorted(data), dtype=torch.float32)
+
+
 @dataclass
 class Nf4QuantState:
-    """Field-compatible stand-in for bitsandbytes' ``QuantState`` (NF4 only)."""
+    """Field-compatible stand-in for bitsandbytes' ``QuantState`` (the 4-bit types: NF4 and FP4)."""
 
     absmax: torch.Tensor                 # fp32 (n_blocks,), or uint8 when nested
     shape: Tuple[int, ...]               # logical shape of the unquantised weight
@@ -45,6 +80,52 @@ class Nf4QuantState:
     @property
     def nested(self) -> bool:
         return self.state2 is not None
+
+    # ---- serialisation: the entries bitsandbytes' QuantState.as_dict(packed=True) / from_dict use, which is
+    # what the reference module writes into its state dict (quantize/layer.py:76-81) and what 4-bit
+    # checkpoints on the hub hold: tensors under their own names, everything else as a JSON object
+    # packed into a uint8 tensor named "quant_state.bitsandbytes__<quant_type>".
+    def as_dict(self, packed: bool = False) -> dict:
+        import json
+
+        plain = {"quant_type": self.quant_type, "absmax": self.absmax, "blocksize": int(self.blocksize),
+                 "quant_map": self.code, "dtype": str(self.dtype).replace("torch.", ""), "shape": tuple(self.shape)}
+        if self.nested:
+            off = self.offset
+            plain.update({"nested_absmax": self.state2.absmax, "nested_blocksize": int(self.state2.blocksize),
+                          "nested_quant_map": self.state2.code.clone(),
+                          "nested_dtype": str(getattr(self.state2, "dtype", torch.float32)).replace("torch.", ""),
+                          "nested_offset": float(off.item()) if torch.is_tensor(off) else float(off)})
+        if not packed:
+            return plain
+        out = {k: v for k, v in plain.items() if torch.is_tensor(v)}
+        rest = {k: (list(v) if isinstance(v, tuple) else v) for k, v in plain.items() if not torch.is_tensor(v)}
+        blob = torch.tensor(list(json.dumps(rest).encode("utf-8")), dtype=torch.uint8)
+        out["quant_state.bitsandbytes__" + self.quant_type] = blob
+        return out
+
+    @classmethod
+    def from_dict(cls, qs_dict: dict, device) -> "Nf4QuantState":
+        import json
+
+        d = dict(qs_dict)
+        packed_keys = [k for k, v in d.items() if "quant_state" in k and torch.is_tensor(v)]
+        if not packed_keys and "quant_type" not in d:
+            raise ValueError("quant state entries hold neither a packed quant_state nor a quant_type")
+        if len(packed_keys) > 1 or (packed_keys and not any(t in packed_keys[0] for t in QUANT_TYPES)):
+            raise ValueError(f"there should be exactly one quant_state entry of a 4-bit type, found {packed_keys}")
+        if packed_keys:
+            blob = d.pop(packed_keys[0])
+            d.update(json.loads(bytes(blob.detach().cpu().to(torch.uint8).tolist()).decode("utf-8")))
+        d = {k.split(".")[-1]: v for k, v in d.items()}          # names may come with a parameter prefix
+        offset = state2 = None
+        if "nested_absmax" in d:
+            offset = torch.tensor(float(d["nested_offset"]), dtype=torch.float32, device=device)
+            state2 = BlockwiseState(absmax=d["nested_absmax"].to(device), code=d["nested_quant_map"].to(device),
+                                    blocksize=int(d["nested_blocksize"]))
+        return cls(absmax=d["absmax"].to(device), shape=tuple(int(v) for v in d["shape"]),
+                   code=d["quant_map"].to(device=device, dtype=torch.float32), blocksize=int(d["blocksize"]),
+                   quant_type=d["quant_type"], dtype=getattr(torch, d["dtype"]), offset=offset, state2=state2)
 
     def to(self, device) -> "Nf4QuantState":
         self.absmax = self.absmax.to(device)
@@ -64,6 +145,7 @@ class BlockwiseState:
     absmax: torch.Tensor
     code: torch.Tensor
     blocksize: int = 256
+    dtype: torch.dtype = torch.float32
 
 
 def resolve_absmax(quant_state) -> torch.Tensor:
@@ -88,24 +170,47 @@ def resolve_absmax(quant_state) -> torch.Tensor:
     return absmax.contiguous()
 
 
-def quantize_nf4(w: torch.Tensor, blocksize: int = 64) -> Tuple[torch.Tensor, Nf4QuantState]:
-    """Blockwise NF4 quantisation on the GPU: returns (packed uint8 (numel/2, 1), state).
-    Element 2i goes to the high nibble of byte i, 2i+1 to the low nibble."""
+def _quantize_absmax(absmax: torch.Tensor, blocksize2: int = 256):
+    """Second level of a double quantisation, as bitsandbytes does it: subtract the mean, then blockwise
+    8-bit quantisation against the dynamic code book (nearest entry of x / max|block|).  Load-time work on
+    a tensor of E*N*K / blocksize floats: plain torch ops on the device."""
+    offset = absmax.mean()
+    centred = absmax - offset
+    n = centred.numel()
+    pad = (-n) % blocksize2
+    blocks = torch.nn.functional.pad(centred, (0, pad)).view(-1, blocksize2)
+    absmax2 = blocks.abs().amax(dim=1)
+    scaled = blocks / absmax2.clamp_min(torch.finfo(torch.float32).tiny).unsqueeze(1)
+    code = dynamic_map_8bit().to(absmax.device)
+    mid = (code[:-1] + code[1:]) / 2
+    q = torch.bucketize(scaled, mid).to(torch.uint8).view(-1)[:n]
+    return q, BlockwiseState(absmax=absmax2, code=code, blocksize=blocksize2), offset
+
+
+def quantize_nf4(w: torch.Tensor, blocksize: int = 64, quant_type: str = "nf4",
+                 compress_statistics: bool = False) -> Tuple[torch.Tensor, Nf4QuantState]:
+    """Blockwise 4-bit quantisation on the GPU: returns (packed uint8 (numel/2, 1), state).
+    Element 2i goes to the high nibble of byte i, 2i+1 to the low nibble.  With
+    ``compress_statistics`` the fp32 absmax is itself quantised to 8 bits (nested state)."""
     assert w.is_cuda and w.is_contiguous()
     n = w.numel()
     assert n % blocksize == 0 and blocksize % 2 == 0
-    code = nf4_code(w.device)
+    code = code_of(quant_type, w.device)
     packed = torch.empty((n // 2, 1), device=w.device, dtype=torch.uint8)
     absmax = torch.empty(n // blocksize, device=w.device, dtype=torch.float32)
     rc = _lib.lib().mfl_nf4_quant(_lib.ptr(w), _lib.dtype_code(w.dtype), n, blocksize, _lib.ptr(code), _lib.ptr(packed),
                                   _lib.ptr(absmax), _lib.stream())
     _lib.check(rc, "mfl_nf4_quant")
-    return packed, Nf4QuantState(absmax=absmax, shape=tuple(w.shape), code=code, blocksize=blocksize, dtype=w.dtype)
+    state = Nf4QuantState(absmax=absmax, shape=tuple(w.shape), code=code, blocksize=blocksize, quant_type=quant_type,
+                          dtype=w.dtype)
+    if compress_statistics:
+        state.absmax, state.state2, state.offset = _quantize_absmax(absmax)
+    return packed, state
 
 
 def dequantize_nf4(packed: torch.Tensor, quant_state, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """``code[nibble] * absmax[block]`` in fp32, rounded once to ``dtype`` (default: the state's)."""
-    assert quant_state.quant_type == "nf4"
+    assert quant_state.quant_type in QUANT_TYPES
     assert packed.is_cuda and packed.is_contiguous()
     dtype = quant_state.dtype if dtype is None else dtype
     shape = tuple(quant_state.shape)
