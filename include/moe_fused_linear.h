@@ -47,6 +47,7 @@ extern "C" {
 #define MFL_ERR_ALIGN (-4)       /* pointer not aligned to its element size         */
 #define MFL_ERR_WORKSPACE (-5)   /* workspace missing or too small                  */
 #define MFL_ERR_UNSUPPORTED (-6) /* valid request this build has no kernel for      */
+#define MFL_ERR_LIMIT (-7)       /* size beyond a fixed maximum of the entry point   */
 
 MFL_API int mfl_abi_version(void);
 /* Static, NUL-terminated description of a return code of this library. */
@@ -205,6 +206,18 @@ MFL_API size_t mfl_expert_sort_workspace(int64_t R, int E);
 MFL_API int mfl_expert_sort(const void *sel, int sel_dtype, int64_t R, int E, int32_t *counts,
                     int32_t *sort_idx, int32_t *inv_sort_idx, void *workspace, size_t ws_bytes,
                     void *stream);
+
+/* mfl_expert_sort without a workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  Same outputs as mfl_expert_sort, bit for bit.  The tables
+ * of the sort live in a fixed array of 2 228 224 bytes of device memory that belongs to the
+ * library (one copy per GPU the library runs on, held until the process ends); the call
+ * allocates nothing, on the device or through any library.  Limit: E <= 512 (any R up to
+ * 2^31 - 1); beyond it the call returns MFL_ERR_LIMIT with nothing enqueued.  All calls on one
+ * GPU share that GPU's array: calls that may overlap in time on one GPU (different streams,
+ * different threads) race and must be serialised by the caller; calls on one stream are safe. */
+MFL_API int mfl_expert_sort_static(const void *sel, int sel_dtype, int64_t R, int E, int32_t *counts,
+                           int32_t *sort_idx, int32_t *inv_sort_idx, void *stream);
 
 /* dst[j, :] = src[idx[j] / idx_div, :] * (row_scale ? row_scale[idx[j]] : 1), j < R_out.
  * With idx = sort_idx and idx_div = k this is "replicate each token k times, then gather",

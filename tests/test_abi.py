@@ -44,7 +44,7 @@ def test_version_and_strerror():
     lib = _lib.lib()
     assert lib.mfl_abi_version() == 1
     assert lib.mfl_strerror(0) == b"ok"
-    for code in (-1, -2, -3, -4, -5, -6):
+    for code in (-1, -2, -3, -4, -5, -6, -7):
         assert lib.mfl_strerror(code) not in (b"ok", b"unknown error code")
     assert lib.mfl_strerror(-99) == b"unknown error code"
 
@@ -73,6 +73,9 @@ def test_argument_errors_without_device_work():
     assert lib.mfl_route_softmax_topk(p, _lib.F32, 4, 8, 9, 1, None, None, BF16, p, None) == -2
     assert lib.mfl_expert_sort(p, _lib.I64, 16, 4, None, None, None, None, 0, None) == -1
     assert lib.mfl_expert_sort(p, 9, 16, 4, p, None, None, None, 0, None) == -3
+    # the entry point without a workspace: same argument checks, and its fixed maximum
+    assert lib.mfl_expert_sort_static(p, _lib.I64, 16, 4, None, None, None, None) == -1
+    assert lib.mfl_expert_sort_static(p, _lib.I64, -1, 4, p, None, None, None) == -2
     assert lib.mfl_silu_mul_fwd(None, p, p, 8, BF16, None) == -1
     assert lib.mfl_gather_rows(p, p, 0, None, p, 4, 8, BF16, None) == -2
     # empty problems are accepted and do nothing

@@ -76,6 +76,8 @@ const char *mfl_strerror(int code) {
             return "workspace missing or too small";
         case MFL_ERR_UNSUPPORTED:
             return "request not supported by this build";
+        case MFL_ERR_LIMIT:
+            return "size beyond the fixed maximum of this entry point";
         default:
             return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error code";
     }
@@ -286,6 +288,14 @@ int mfl_expert_sort(const void *sel, int sel_dtype, int64_t R, int E, int32_t *c
     if (!counts || (R > 0 && !sel)) return MFL_ERR_NULL;
     return expert_sort(sel, sel_dtype == MFL_I64, R, E, counts, sort_idx, inv_sort_idx, workspace, ws_bytes,
                        (hipStream_t)stream);
+}
+
+int mfl_expert_sort_static(const void *sel, int sel_dtype, int64_t R, int E, int32_t *counts, int32_t *sort_idx,
+                           int32_t *inv_sort_idx, void *stream) {
+    if (R < 0 || E <= 0 || R > 0x7fffffff) return MFL_ERR_SHAPE;
+    if (!itype_ok(sel_dtype)) return MFL_ERR_DTYPE;
+    if (!counts || (R > 0 && !sel)) return MFL_ERR_NULL;
+    return expert_sort_static(sel, sel_dtype == MFL_I64, R, E, counts, sort_idx, inv_sort_idx, (hipStream_t)stream);
 }
 
 int mfl_gather_rows(const void *src, const int32_t *idx, int idx_div, const void *row_scale, void *dst, int64_t R_out,

@@ -28,5 +28,7 @@ int route_sort_small(const void *logits, int logits_dtype, int64_t T, int E, int
 size_t expert_sort_workspace(int64_t R, int E);
 int expert_sort(const void *sel, int is_i64, int64_t R, int E, int32_t *counts, int32_t *sort_idx,
                 int32_t *inv_sort_idx, void *workspace, size_t ws_bytes, hipStream_t stream);
+int expert_sort_static(const void *sel, int is_i64, int64_t R, int E, int32_t *counts, int32_t *sort_idx,
+                       int32_t *inv_sort_idx, hipStream_t stream);
 
 }  // namespace mfl

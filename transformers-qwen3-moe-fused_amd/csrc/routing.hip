@@ -3,6 +3,8 @@
 // Both are latency/bandwidth-bound integer-heavy kernels built from wavefront ballots,
 // cross-lane shuffles and LDS histograms; neither uses atomics, so results are
 // deterministic and the index outputs are reproducible bit for bit.
+#include <mutex>
+
 #include "common.h"
 #include "ops.h"
 
@@ -664,6 +666,49 @@ int expert_sort(const void *sel, int is_i64, int64_t R, int E, int32_t *counts, 
     if (rc || rank_buf == nullptr) return rc;
     sort_scatter_kernel<<<blocks, 256, 0, stream>>>(sel, is_i64, R, E, n_waves, table, sort_idx, rank_buf);
     return launch_status();
+}
+
+// ---- expert sort that allocates nothing ----------------------------------------------------
+//
+// The tables of the two-kernel sort (per-wave histograms and per-workgroup totals) live in a
+// file-scope device array instead of a caller-supplied workspace.  The array's name is a host-side
+// stand-in, not a device address: its address on the current device is looked up once per device
+// with hipGetSymbolAddress and kept; kernels get that pointer as an argument, like a workspace.
+// Every call on a device shares that device's array: calls that overlap in time on one device race
+// (calls on one stream are ordered and safe).  Nothing needs clearing between calls: the count
+// kernel writes every table entry that the scatter kernel reads.
+namespace {
+
+constexpr size_t kStaticSortBytes =
+    (size_t)(kFastMaxBlocks * kFastWaves + kFastMaxBlocks) * 512 * sizeof(int32_t);  // 2 228 224 bytes
+static __device__ __align__(256) unsigned char scratch[kStaticSortBytes];
+
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+}  // namespace
+
+int expert_sort_static(const void *sel, int is_i64, int64_t R, int E, int32_t *counts, int32_t *sort_idx,
+                       int32_t *inv_sort_idx, hipStream_t stream) {
+    if (!fast_sort_ok(E)) return MFL_ERR_LIMIT;  // the tables of more experts do not fit the fixed array
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return MFL_ERR_LIMIT;
+    void *ptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (g_scratch_ptr[dev] == nullptr) {
+            void *p = nullptr;
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) return (int)e;
+            if (p == nullptr) return (int)hipErrorInvalidSymbol;
+            g_scratch_ptr[dev] = p;
+        }
+        ptr = g_scratch_ptr[dev];
+    }
+    return expert_sort(sel, is_i64, R, E, counts, sort_idx, inv_sort_idx, ptr, kStaticSortBytes, stream);
 }
 
 }  // namespace mfl

@@ -47,6 +47,7 @@ _SIGNATURES = {
     "mfl_route_sort_small": (_i, [_vp, _i, _i64, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "mfl_expert_sort_workspace": (_sz, [_i64, _i]),
     "mfl_expert_sort": (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "mfl_expert_sort_static": (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _vp]),
     "mfl_gather_rows": (_i, [_vp, _vp, _i, _vp, _vp, _i64, _i, _i, _vp]),
     "mfl_combine_rows": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
     "mfl_rows_dot": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
