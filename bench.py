@@ -4,8 +4,9 @@
 A step is one forward grouped GEMM over one synthetic batch at benchmark configuration 2
 (Qwen3-30B-A3B gate_proj: 128 experts, weight (128, 768, 2048) bf16, 4096 tokens routed
 top-8 -> 32768 rows sorted by expert).  Inputs are resident in HBM before the timed region.
-One JSON line is printed; dX / dW at config 3 and the bandwidth-bound neighbours are reported
-under "extra" from separate short timed loops.
+One JSON line is printed.  The metric names forward, dX and dW: the forward product is the timed
+step ("value"), dX and dW at config 3 are first-class fields beside it ("dx", "dw"), and the
+bandwidth-bound neighbours are reported under "extra" from separate short timed loops.
 """
 from __future__ import annotations
 
@@ -22,9 +23,15 @@ for _p in (ROOT, os.path.join(ROOT, "transformers-qwen3-moe-fused_amd")):
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-# HBM bytes per launch of the benchmarked kernel, from the FETCH_SIZE / WRITE_SIZE passes summarised in
-# profiles/gemm_fwd_gate_proj_config2_hbm_traffic.txt (537.1 MB read + 50.3 MB written)
+# HBM bytes per launch of the benchmarked kernel: not measured by this run but taken from the FETCH_SIZE /
+# WRITE_SIZE counter passes summarised in profiles/gemm_fwd_gate_proj_config2_hbm_traffic.txt
+# (537.1 MB read + 53.8 MB written); the JSON line names that file as the source
 MEASURED_TRAFFIC_BYTES = 591.0e6
+TRAFFIC_SOURCE = "profiles/gemm_fwd_gate_proj_config2_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not this run)"
+# A burst of back-to-back launches starts in a transient of the board's power management (boost clocks for
+# the first ten launches, a dip around launch 20, settled after about 150): every timed loop is preceded by
+# at least this many untimed launches, whatever --warmup says.
+MIN_WARMUP = 200
 
 E, HIDDEN, INTER, TOKENS, TOPK = 128, 2048, 768, 4096, 8
 ROWS = TOKENS * TOPK
@@ -190,7 +197,8 @@ def main() -> int:
     def step(i):
         grouped_gemm_forward(xs[i % NB], ws[i % NB], m_sizes, out=ys[i % NB])
 
-    for i in range(args.warmup):
+    warmup_effective = max(args.warmup, MIN_WARMUP)
+    for i in range(warmup_effective):
         step(i)
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
@@ -216,6 +224,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "warmup_effective": warmup_effective,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -227,28 +236,51 @@ def main() -> int:
                    "routing": "softmax top-8 of N(0,1) logits, rows sorted by expert"},
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved_gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "traffic_source": TRAFFIC_SOURCE,
                      "kernel_us": round(kernel_us, 2), "algorithmic_bytes": alg_bytes,
                      "mfma_tflops": round(flop / kernel_us / 1e6, 1),
                      "mfma_frac": round(flop / kernel_us / 1e6 / PEAK_BF16_TFLOPS, 4)},
     }
 
+    # ---- the other two products of the metric, at config 3 (down_proj backward), same method: rotating buffer
+    # sets, MIN_WARMUP untimed launches, then args.steps timed ones between two events
+    dys = [torch.randn((ROWS, HIDDEN), device=dev, dtype=torch.bfloat16) for _ in range(NB)]   # grad of down_proj out
+    hs = [torch.randn((ROWS, INTER), device=dev, dtype=torch.bfloat16) for _ in range(NB)]     # down_proj input
+    wd = [w.view(E, HIDDEN, INTER) for w in ws]                                                # (128, 2048, 768)
+    dxs = [torch.empty((ROWS, INTER), device=dev, dtype=torch.bfloat16) for _ in range(NB)]
+    dws = [torch.empty((E, HIDDEN, INTER), device=dev, dtype=torch.bfloat16) for _ in range(NB)]
+
+    def product_line(us):
+        return {"us": round(us, 2), "tflops": round(flop / us / 1e6, 1),
+                "mfma_frac": round(flop / us / 1e6 / PEAK_BF16_TFLOPS, 4),
+                "hbm_gbs": round(alg_bytes / us / 1e3, 1), "hbm_frac": round(alg_bytes / us / 1e3 / PEAK_HBM_GBS, 4),
+                "algorithmic_bytes": alg_bytes, "steps": args.steps, "warmup_effective": warmup_effective}
+
+    us = _event_us(lambda i: grouped_gemm_forward_transposed(dys[i % NB], wd[i % NB], m_sizes, out=dxs[i % NB]),
+                   args.steps, warmup_effective, stream)
+    out["dx"] = dict(workload="configs[2]: down_proj input gradient, dy (32768, 2048) x w (128, 2048, 768)",
+                     **product_line(us))
+    us = _event_us(lambda i: grouped_gemm_backward_dw(hs[i % NB], dys[i % NB], m_sizes, torch.bfloat16,
+                                                      out=dws[i % NB]), args.steps, warmup_effective, stream)
+    out["dw"] = dict(workload="configs[2]: down_proj weight gradient, x (32768, 768), dy (32768, 2048)",
+                     **product_line(us))
+    out["fwd"] = dict(workload="configs[1]: gate_proj forward (the timed step)", **product_line(kernel_us))
+    del dws, dxs
+
     if not args.no_extra:
         extra = {}
-        dys = [torch.randn((ROWS, HIDDEN), device=dev, dtype=torch.bfloat16) for _ in range(NB)]   # grad of down_proj out
-        hs = [torch.randn((ROWS, INTER), device=dev, dtype=torch.bfloat16) for _ in range(NB)]     # down_proj input
-        wd = [w.view(E, HIDDEN, INTER) for w in ws]                                                # (128, 2048, 768)
-        it, wm = 50, 100      # 100 warm-up launches: a burst of launches starts in a power-management transient
-        us = _event_us(lambda i: grouped_gemm_forward_transposed(dys[i % NB], wd[i % NB], m_sizes), it, wm, stream)
-        extra["dx_down_proj"] = {"us": round(us, 1), "tflops": round(flop / us / 1e6, 1),
-                                 "mfma_frac": round(flop / us / 1e6 / PEAK_BF16_TFLOPS, 4),
-                                 "hbm_frac": round(alg_bytes / us / 1e3 / PEAK_HBM_GBS, 4)}
-        dws = [torch.empty((E, HIDDEN, INTER), device=dev, dtype=torch.bfloat16) for _ in range(NB)]
-        us = _event_us(lambda i: grouped_gemm_backward_dw(hs[i % NB], dys[i % NB], m_sizes, torch.bfloat16,
-                                                          out=dws[i % NB]), it, wm, stream)
-        extra["dw_down_proj"] = {"us": round(us, 1), "tflops": round(flop / us / 1e6, 1),
-                                 "mfma_frac": round(flop / us / 1e6 / PEAK_BF16_TFLOPS, 4),
-                                 "hbm_frac": round(alg_bytes / us / 1e3 / PEAK_HBM_GBS, 4)}
-        del dws
+        it, wm = 50, MIN_WARMUP
+        # the forward product with the replicate-and-sort folded into its operand load (rows gathered from the
+        # 4096 token rows): 470 MB algorithmic instead of 587 MB
+        from qwen3_moe_fused.grouped_gemm.fused import grouped_gemm_forward_gathered
+        toks = [torch.randn((TOKENS, HIDDEN), device=dev, dtype=torch.bfloat16) for _ in range(NB)]
+        us = _event_us(lambda i: grouped_gemm_forward_gathered(toks[i % NB], sort_idx, TOPK, ws[i % NB], m_sizes),
+                       it, wm, stream)
+        gb = 2.0 * (TOKENS * HIDDEN + E * INTER * HIDDEN + ROWS * INTER) + ROWS * 4
+        extra["fwd_gate_proj_gathered"] = {"us": round(us, 1), "tflops": round(flop / us / 1e6, 1),
+                                           "mfma_frac": round(flop / us / 1e6 / PEAK_BF16_TFLOPS, 4),
+                                           "algorithmic_bytes": gb, "hbm_frac": round(gb / us / 1e3 / PEAK_HBM_GBS, 4)}
+        del toks
         us = _event_us(lambda i: silu_mul_forward(hs[i % NB], hs[(i + 1) % NB]), it, wm, stream)
         b = 3.0 * ROWS * INTER * 2
         extra["silu_mul_fwd"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / PEAK_HBM_GBS, 4)}
@@ -261,7 +293,10 @@ def main() -> int:
         b = TOKENS * E * 4 + TOKENS * TOPK * (4 + 2 + 8)
         extra["softmax_topk_4096"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 2)}
         # NF4: fused dequant+GEMM vs dequant-then-GEMM at 16 / 256 / 16384 tokens (config 5 gate_proj)
-        packed, qstate = quantize_nf4(ws[0], 64)
+        # three packed weight sets in rotation: the 113 MB of one set would stay in the 256 MB MALL between
+        # launches, and the figure would not be an HBM figure
+        qsets = [quantize_nf4(w, 64) for w in ws]
+        packed, qstate = qsets[0]
         nf4 = {}
         for tokens in (16, 256, 16384):
             lgt = torch.randn((tokens, E), device=dev)
@@ -269,18 +304,18 @@ def main() -> int:
             ms5, _, _ = get_expert_counts_and_idx(s5.view(-1), E)
             x5 = torch.randn((tokens * TOPK, HIDDEN), device=dev, dtype=torch.bfloat16)
             n_it, n_wm = (20, 30) if tokens > 1000 else (100, 300)
-            us_f = _event_us(lambda i: grouped_gemm_forward_4bit(x5, packed, qstate, ms5), n_it, n_wm, stream)
-            us_u = _event_us(lambda i: grouped_gemm_forward(x5, dequantize_nf4(packed, qstate, torch.bfloat16), ms5),
+            us_f = _event_us(lambda i: grouped_gemm_forward_4bit(x5, *qsets[i % NB], ms5), n_it, n_wm, stream)
+            us_u = _event_us(lambda i: grouped_gemm_forward(x5, dequantize_nf4(*qsets[i % NB], torch.bfloat16), ms5),
                              n_it, n_wm, stream)
             active = int((ms5 > 0).sum().item())                       # host read outside any timed loop
             packed_bytes = active * INTER * HIDDEN * (0.5 + 4.0 / 64)
             nf4[f"tokens_{tokens}"] = {"fused_us": round(us_f, 1), "dequant_then_gemm_us": round(us_u, 1),
-                                       "active_experts": active,
+                                       "active_experts": active, "weight_sets_in_rotation": NB,
                                        "fused_packed_gbs": round(packed_bytes / us_f / 1e3, 1),
                                        "fused_tflops": round(2.0 * tokens * TOPK * INTER * HIDDEN / us_f / 1e6, 1)}
         extra["nf4_gate_proj"] = nf4
         # the dequant kernel alone: packed bytes + scales in, bf16 out (a fresh output tensor per call)
-        us = _event_us(lambda i: dequantize_nf4(packed, qstate, torch.bfloat16), 50, 100, stream)
+        us = _event_us(lambda i: dequantize_nf4(*qsets[i % NB], torch.bfloat16), 50, MIN_WARMUP, stream)
         b = E * INTER * HIDDEN * (0.5 + 4.0 / 64 + 2.0)
         extra["nf4_dequant_gate_proj"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 1),
                                           "hbm_frac": round(b / us / 1e3 / PEAK_HBM_GBS, 4)}
@@ -293,7 +328,7 @@ def main() -> int:
         extra["nf4_gate_proj_dx"] = {"fused_us": round(us_f, 1), "dequant_then_gemm_us": round(us_u, 1),
                                      "fused_tflops": round(flop / us_f / 1e6, 1)}
         del dyg
-        del packed, qstate, x5
+        del packed, qstate, qsets, x5
         # config 4: rank-16 LoRA on gate_proj, 8192 tokens, Zipf(1.2)-skewed top-8 routing (65536 rows):
         # the frozen base product and the five thin products of one forward + backward
         T4, R4, RANK = 8192, 8192 * TOPK, 16
