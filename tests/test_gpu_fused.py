@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import oracle
-from util import check_close, gen, m_sizes_uniform, randn, to_np32
+from util import check_close, gen, m_sizes_uniform, randn, to_np32, unit_scale_atol
 
 pytestmark = pytest.mark.gpu
 
@@ -35,6 +35,14 @@ def _quantised(E, N, K, blocksize, seed):
     state = Nf4QuantState(absmax=torch.from_numpy(absmax).to(DEV), shape=(E, N, K), code=nf4_code(DEV),
                           blocksize=blocksize, dtype=torch.bfloat16)
     return torch.from_numpy(q).view(-1, 1).to(DEV), state, w_deq
+
+
+def _nf4_atol(ref, K, *blocksizes):
+    """K % 128 == 0 and blocks of at least 64 weights go to the kernel that scales partial sums (see
+    unit_scale_atol); two percent of the output scale there, one percent of unit scale elsewhere."""
+    if K % 128 == 0 and min(blocksizes) >= 64:
+        return unit_scale_atol(ref, 2e-2)
+    return 1e-2
 
 
 def _oracle_glu(xg, wg, wu, sel_sorted):
@@ -70,7 +78,8 @@ def test_gathered_nf4_forward(T, E, k, N, K, blocksize):
     packed, state, w_deq = _quantised(E, N, K, blocksize, N + K)
     rows = sort_idx.numpy() // k
     y = grouped_gemm_forward_4bit_gathered(x.to(DEV), sort_idx.to(DEV), k, packed, state, ms.to(DEV))
-    check_close(y, oracle.linear_fwd(to_np32(x)[rows], w_deq, np.sort(sel, kind="stable")), what="gathered nf4 fwd")
+    ref = oracle.linear_fwd(to_np32(x)[rows], w_deq, np.sort(sel, kind="stable"))
+    check_close(y, ref, atol=_nf4_atol(ref, K, blocksize), what="gathered nf4 fwd")
     y2 = grouped_gemm_forward_4bit(x[rows.astype(np.int64)].contiguous().to(DEV), packed, state, ms.to(DEV))
     assert torch.equal(y, y2)
 
@@ -117,15 +126,45 @@ def test_glu_nf4_forward(T, E, k, N, K, bs_g, bs_u):
     h, e, g = grouped_glu_forward_4bit(x.to(DEV), pg, sg, pu, su, ms.to(DEV), sort_idx.to(DEV), k,
                                        return_products=True)
     h_ref, e_ref, g_ref = _oracle_glu(to_np32(xg), wg_deq, wu_deq, np.sort(sel, kind="stable"))
-    check_close(e, e_ref, what="gate product")
-    check_close(g, g_ref, what="up product")
-    check_close(h, h_ref, 2e-2, 2e-2, what="glu")
+    check_close(e, e_ref, atol=_nf4_atol(e_ref, K, bs_g), what="gate product")
+    check_close(g, g_ref, atol=_nf4_atol(g_ref, K, bs_u), what="up product")
+    # the oracle's e and g differ from the kernel's by a few bf16 ulps, and silu(e) * g carries that on, times
+    # the size of the other factor: h is checked against the oracle's SiLU-mul of the kernel's own e and g
+    # (one ulp), and against the oracle's h by its largest error relative to the largest value
+    h_own = oracle.from_bf16_bits(oracle.silu_mul_fwd_bf16(oracle.to_bf16_bits(to_np32(e)), oracle.to_bf16_bits(to_np32(g))))
+    check_close(h, h_own, 2e-2, 2e-2, what="glu of the kernel's own products")
+    assert np.abs(to_np32(h) - h_ref).max() <= 1e-2 * np.abs(h_ref).max(), "glu against the oracle's"
     e2 = grouped_gemm_forward_4bit(xg.to(DEV), pg, sg, ms.to(DEV))
     g2 = grouped_gemm_forward_4bit(xg.to(DEV), pu, su, ms.to(DEV))
     assert torch.equal(e, e2) and torch.equal(g, g2)
     assert torch.equal(h, silu_mul_forward(e2, g2))
     h3 = grouped_glu_forward_4bit(xg.to(DEV), pg, sg, pu, su, ms.to(DEV))
     assert torch.equal(h, h3)
+
+
+def test_decode_size_nf4_product_is_as_accurate_as_the_reference_rounding():
+    # The decode-size kernel computes sum over blocks of absmax * (x . bf16(code)), the reference x . bf16(code * absmax).
+    # Against the product with the unrounded weights code * absmax, in float64, neither is better: same rms
+    # error, same largest error, within the scatter of such figures.
+    T, E, k, N, K, blocksize = 256, 128, 8, 768, 2048, 64
+    ms, sort_idx, sel = _routing(T, E, k, 11)
+    x = randn((T, K), gen(3), 1.0, torch.bfloat16)
+    w = randn((E, N, K), gen(4), 0.05)
+    q, absmax = oracle.nf4_quant(w.numpy(), blocksize)
+    w_exact = oracle.nf4_dequant(q, absmax, blocksize).reshape(E, N, K)
+    state = Nf4QuantState(absmax=torch.from_numpy(absmax).to(DEV), shape=(E, N, K), code=nf4_code(DEV),
+                          blocksize=blocksize, dtype=torch.bfloat16)
+    rows = (sort_idx.numpy() // k).astype(np.int64)
+    xg = to_np32(x)[rows]
+    sel_sorted = np.sort(sel, kind="stable")
+    y = to_np32(grouped_gemm_forward_4bit(x[rows].contiguous().to(DEV), torch.from_numpy(q).view(-1, 1).to(DEV), state,
+                                          ms.to(DEV))).astype(np.float64)
+    exact = oracle.linear_fwd(xg, w_exact, sel_sorted).astype(np.float64)
+    reference = oracle.round_bf16(oracle.linear_fwd(xg, oracle.round_bf16(w_exact), sel_sorted)).astype(np.float64)
+    err_k, err_r = y - exact, reference - exact
+    rms_k, rms_r = np.sqrt((err_k ** 2).mean()), np.sqrt((err_r ** 2).mean())
+    assert rms_k <= 1.1 * rms_r, (rms_k, rms_r)
+    assert np.abs(err_k).max() <= 1.5 * np.abs(err_r).max(), (np.abs(err_k).max(), np.abs(err_r).max())
 
 
 def test_unsupported_requests_fall_back_to_the_separate_kernels():

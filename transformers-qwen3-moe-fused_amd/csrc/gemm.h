@@ -38,6 +38,20 @@ int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, 
                    int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream,
                    const GemmFusion *fusion = nullptr);
 
+// One packed NF4 weight matrix with its quantisation state.
+struct Nf4Matrix {
+    const uint8_t *wq;
+    const float *code16;
+    const float *absmax;
+    int bs_shift;  // log2 of the quantisation block size
+};
+
+// The streaming form of gemm_nf4_decode (all operands copied straight to LDS, scale applied per block to the
+// partial sums): K % 128 == 0 and blocks of at least 64 weights, MFL_ERR_UNSUPPORTED otherwise.
+int gemm_nf4_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
+                    bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
+                    int K, int E, int out_dtype, hipStream_t stream);
+
 // Forward with NF4 weights for decode-sized batches (at most 32 rows per expert on average):
 // weights decoded in registers, no LDS stage.
 int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,

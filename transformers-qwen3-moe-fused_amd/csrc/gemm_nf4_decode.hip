@@ -30,13 +30,6 @@ namespace {
 
 constexpr int kDepth = 4;  // steps in flight
 
-struct Nf4Matrix {
-    const uint8_t *wq;
-    const float *code16;
-    const float *absmax;
-    int bs_shift;
-};
-
 // SUPER (K % 256 == 0): the reduction index is permuted over 256-wide super-steps so that a lane
 // owns 128 consecutive weights of its column (64 packed bytes: one half of a 128-byte line) per
 // super-step and fetches them with four back-to-back loads, once every four steps.  With one
@@ -326,6 +319,11 @@ int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const
     const int64_t grid = row_tiles * tiles_n;
     if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
     const bf16_t *px = (const bf16_t *)x;
+    {
+        const int rc = gemm_nf4_stream(px, row_idx, idx_div, w0, w1, glu, m_sizes, ms_i64, y, e_out, g_out, R, N, K, E,
+                                       out_dtype, stream);
+        if (rc != MFL_ERR_UNSUPPORTED) return rc;
+    }
     const bool wide = K % 256 == 0;  // 64 packed bytes per lane and super-step
     const bool am1 = w0.bs_shift >= 5 && w1.bs_shift >= 5;  // one scale per lane and step
     const bool xstage = R > 2 * (int64_t)E;                   // rows change hands in LDS

@@ -1,0 +1,321 @@
+// Fused NF4 grouped GEMM for decode-sized batches, streaming form (K % 128 == 0, quantisation blocks of at
+// least 64 weights): everything a workgroup reads arrives in LDS by direct copies (global_load_lds), in a ring
+// of stages of 128 reduction elements, so that the only vector-memory operations in the reduction loop are
+// copies with one and the same lead.  The wave's memory counter completes in order: a register load of rows
+// or scales issued after a copy would, when waited for, hold the wave until the copy has landed too, and the
+// copies would never be further ahead than those loads.
+//
+// A workgroup (4 waves) owns 32 rows of one expert and 128 output columns, a wave 32 of the columns (of both
+// matrices in the gated linear unit).
+//   stage = rows     32 x 128 bf16 (8 KiB, shared by the four waves; chunk c of row r at c ^ (r & 15))
+//         + weights  per wave and matrix 32 columns x 64 packed bytes (2 KiB; chunk c of row r at c ^ ((r >> 2) & 3))
+//         + scales   per wave and matrix 32 columns x 2 floats (one per 64 reduction elements)
+//   One barrier per stage: it publishes the rows that the other waves copied and frees the slot of the
+//   stage before for the next copies.  Three stages are 52 KiB: three workgroups share a CU (two of the gated
+//   form), and what counts at decode sizes is that every workgroup of the launch is resident at once: a
+//   workgroup's loop is a chain of latencies (about 1.1 us per stage whatever is taken out of it), so a second
+//   round of workgroups doubles the time of the launch.
+//
+// Decoding costs about one vector instruction per weight instead of three and a half:
+//   * a byte of packed weights is two weights, and two bf16 are one dword of an MFMA operand: a 256-entry
+//     table in LDS, indexed by the byte, holds the finished pair.  One shift-by-two of a byte (SDWA) and one
+//     LDS read per pair.  (A copy of the table per bank, 64 KiB, takes the bank conflicts of the lookups
+//     away and the second and third workgroup of the CU with them: slower.)
+//   * the table holds the bare code values (rounded to bf16 once).  The scale of a quantisation block is
+//     applied to the block's partial sum in fp32: with the weights as the SECOND MFMA operand a lane's 16
+//     accumulators all belong to one output column, whose scale the lane holds, so a 64-wide step is four
+//     MFMAs into a fresh accumulator and 16 multiply-adds into the running sum.
+//   The product is therefore sum over blocks of absmax * (x . bf16(code)) instead of x . bf16(code * absmax): the
+//   same one rounding to bf16 per weight, taken before the scale rather than after it.  The two differ by
+//   rounding noise of the size that either has against exact arithmetic.
+#include "common.h"
+#include "gemm.h"
+
+namespace mfl {
+
+namespace {
+
+typedef __attribute__((address_space(3))) void *lds_void_ptr;
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | 0x70 | 0xF00 | ((N >> 4) << 14));
+}
+
+// Wave-wide copies from global memory to consecutive LDS (16 or 4 bytes per lane), written out by hand: the
+// compiler orders LDS reads behind every copy to LDS that it knows to be in flight, i.e. behind the stages
+// just requested.  M0 carries the LDS address of lane 0's piece; nothing else in the kernel uses M0.
+__device__ __forceinline__ void copy16_to_lds(const void *src, unsigned char *dst) {
+    const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void_ptr)dst);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_addr) : "memory");
+}
+__device__ __forceinline__ void copy4_to_lds(const void *src, unsigned char *dst) {
+    const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void_ptr)dst);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(src), "s"(lds_addr) : "memory");
+}
+
+// (byte `B` of w) << 2: the LDS byte offset of the pair-table entry of two packed weights, in one instruction.
+template <int B>
+__device__ __forceinline__ uint32_t byte_times_4(uint32_t w) {
+    uint32_t r;
+    const uint32_t two = 2;
+    if constexpr (B == 0)
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(r) : "v"(two), "v"(w));
+    else if constexpr (B == 1)
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(r) : "v"(two), "v"(w));
+    else if constexpr (B == 2)
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2" : "=v"(r) : "v"(two), "v"(w));
+    else
+        asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3" : "=v"(r) : "v"(two), "v"(w));
+    return r;
+}
+
+template <bool GLU>
+struct StreamShape {
+    static constexpr int CB = GLU ? 2 : 1;     // weight matrices per wave
+    static constexpr int RING = 3;             // stages in LDS; two of them in flight
+    static constexpr int kX = 32 * 256;        // rows of a stage
+    static constexpr int kW = 32 * 64;         // packed weights of a stage, per wave and matrix
+    static constexpr int kA = 32 * 2 * 4;      // scales of a stage, per wave and matrix
+    static constexpr int kStage = kX + 4 * CB * (kW + kA);
+    static constexpr int kTable = CB * 256 * 4;
+    static constexpr int kLds = RING * kStage + kTable;  // 53248: three workgroups per CU; gated: 81920, two
+    static constexpr int kOps = 2 * CB + 2 + CB;  // copies per wave and stage
+};
+
+template <bool GLU, typename TO>
+__global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restrict__ x,
+                                                         const int32_t *__restrict__ row_idx, int idx_div,
+                                                         Nf4Matrix w0, Nf4Matrix w1,
+                                                         const void *__restrict__ m_sizes, int ms_i64,
+                                                         TO *__restrict__ y, TO *__restrict__ e_out,
+                                                         TO *__restrict__ g_out, int64_t R, int N, int K, int E,
+                                                         int tiles_n) {
+    using S = StreamShape<GLU>;
+    constexpr int CB = S::CB, RING = S::RING;
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    unsigned char *const table = smem + RING * S::kStage;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31, h = lane >> 5;
+
+    // ---- pair table: entry b = bf16(code[b >> 4]) in the low half (the first of the two weights is the high
+    // nibble), bf16(code[b & 15]) in the high half
+    {
+        const Nf4Matrix *mats[2] = {&w0, &w1};
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            union {
+                bf16_t e[2];
+                uint32_t u;
+            } pr;
+            pr.e[0] = (bf16_t)mats[cb]->code16[tid >> 4];
+            pr.e[1] = (bf16_t)mats[cb]->code16[tid & 15];
+            ((uint32_t *)table)[cb * 256 + tid] = pr.u;
+        }
+    }
+
+    // ---- which 32 rows: row tile blockIdx.x / tiles_n in the order of the experts
+    const int ct = blockIdx.x % tiles_n, rt = blockIdx.x / tiles_n;
+    int expert = -1, m_start = 0, m_size = 0, t_begin = 0;
+    {
+        int row_carry = 0, tile_carry = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int m = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
+            const int t = ceil_div(m, 32);
+            const int minc = wave_inclusive_scan(m), tinc = wave_inclusive_scan(t);
+            const int tb = tile_carry + tinc - t;
+            const uint64_t hits = __ballot(rt >= tb && rt < tb + t);
+            if (hits) {
+                const int src = __ffsll((unsigned long long)hits) - 1;
+                expert = e0 + src;
+                m_start = row_carry + __shfl(minc - m, src);
+                m_size = __shfl(m, src);
+                t_begin = __shfl(tb, src);
+                break;
+            }
+            row_carry += wave_last(minc);
+            tile_carry += wave_last(tinc);
+        }
+    }
+    // every wave of the workgroup takes the same path here: the values above are the same in all of them
+    if (expert < 0) return;
+    expert = __builtin_amdgcn_readfirstlane(expert);
+    const int i0 = __builtin_amdgcn_readfirstlane(m_start) + (rt - __builtin_amdgcn_readfirstlane(t_begin)) * 32;
+    int i_end = __builtin_amdgcn_readfirstlane(m_start) + __builtin_amdgcn_readfirstlane(m_size);
+    if ((int64_t)i_end > R) i_end = (int)R;
+    const int rows = i_end - i0 < 32 ? i_end - i0 : 32;
+    if (rows <= 0) return;
+
+    // ---- sources of this lane's pieces of a stage
+    const int j0 = (ct * 4 + wave) * 32;  // first column of the wave
+    const Nf4Matrix mat[2] = {w0, w1};
+    const unsigned char *w_src[CB][2];  // copy j: columns 16j .. 16j+15 of the wave, four lanes to a column
+    int64_t a_el[CB];                   // first weight under the lane's scale of stage 0: lane i brings scale i & 1 of column i >> 1
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int r = 16 * j + (lane >> 2);
+            const int c = (lane & 3) ^ ((r >> 2) & 3);
+            int col = j0 + r;
+            if (col >= N) col = N - 1;  // copied, multiplied, never stored
+            w_src[cb][j] = mat[cb].wq + ((((int64_t)expert * N + col) * K) >> 1) + c * 16;
+        }
+        int col = j0 + (lane >> 1);
+        if (col >= N) col = N - 1;
+        a_el[cb] = ((int64_t)expert * N + col) * K + (lane & 1) * 64;
+    }
+    const bf16_t *x_src[2];  // copy j: rows 8 wave + 4j .. + 3, sixteen lanes to a row
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int r = 8 * wave + 4 * j + (lane >> 4);
+        const int c = (lane & 15) ^ (r & 15);
+        int64_t src_row = i0 + (r < rows ? r : rows - 1);
+        if (row_idx != nullptr) src_row = (uint32_t)row_idx[src_row] / (uint32_t)idx_div;
+        x_src[j] = x + src_row * K + c * 8;
+    }
+    const int NS = K / 128;
+    auto issue = [&](int stg) {
+        unsigned char *const base = smem + (stg % RING) * S::kStage;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) copy16_to_lds(x_src[j] + (int64_t)stg * 128, base + (wave * 2 + j) * 1024);
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                copy16_to_lds(w_src[cb][j] + (int64_t)stg * 64, base + S::kX + (wave * CB + cb) * S::kW + j * 1024);
+            copy4_to_lds(mat[cb].absmax + ((a_el[cb] + (int64_t)stg * 128) >> mat[cb].bs_shift),
+                         base + S::kX + 4 * CB * S::kW + (wave * CB + cb) * S::kA);
+        }
+    };
+    // ---- where this lane reads a stage: its 16 bytes of packed weights of step s2, its 16 bytes of row n for
+    // MFMA ks of step s2
+    int w_rd[2], x_rd[2][4];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+        w_rd[s2] = n * 64 + (((2 * s2 + h) ^ ((n >> 2) & 3)) << 4);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) x_rd[s2][ks] = n * 256 + (((8 * s2 + 4 * h + ks) ^ (n & 15)) << 4);
+    }
+
+    floatx16 tot[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tot[cb][r] = 0.f;
+
+    // Every wave issues the same S::kOps copies per stage, unconditionally (past the end they repeat the last
+    // stage, into a slot that is free), so "at most (RING - 2) * kOps of my copies outstanding" means that the
+    // stage about to be read has landed.
+#pragma unroll
+    for (int q = 0; q < RING - 1; ++q) issue(q < NS ? q : NS - 1);
+    for (int q = 0; q < NS; ++q) {
+        wait_vmcnt<(RING - 2) * S::kOps>();
+        __syncthreads();  // stage q is whole (the first time round: so is the pair table); nobody reads stage q - 1 any more
+        issue(q + RING - 1 < NS ? q + RING - 1 : NS - 1);
+        const unsigned char *const base = smem + (q % RING) * S::kStage;
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            uint4_t wl[CB];
+            float am[CB];
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                wl[cb] = *(const uint4_t *)(base + S::kX + (wave * CB + cb) * S::kW + w_rd[s2]);
+                am[cb] = *(const float *)(base + S::kX + 4 * CB * S::kW + (wave * CB + cb) * S::kA + (n * 2 + s2) * 4);
+            }
+            floatx16 blk[CB];
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                union {
+                    uint4_t u;
+                    bf16x8 v;
+                } xa, wf;
+                xa.u = *(const uint4_t *)(base + x_rd[s2][ks]);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const uint32_t w = wl[cb][ks];
+                    const unsigned char *const tb = table + cb * 1024;
+                    wf.u[0] = *(const uint32_t *)(tb + byte_times_4<0>(w));
+                    wf.u[1] = *(const uint32_t *)(tb + byte_times_4<1>(w));
+                    wf.u[2] = *(const uint32_t *)(tb + byte_times_4<2>(w));
+                    wf.u[3] = *(const uint32_t *)(tb + byte_times_4<3>(w));
+                    if (ks == 0) {
+                        floatx16 zero;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+                        blk[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa.v, wf.v, zero, 0, 0, 0);
+                    } else {
+                        blk[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa.v, wf.v, blk[cb], 0, 0, 0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) tot[cb][r] = __builtin_fmaf(am[cb], blk[cb][r], tot[cb][r]);
+        }
+    }
+    wait_vmcnt<0>();  // the repeated copies of the last stage must not land in LDS that another workgroup owns by then
+
+    // ---- output: a lane holds column n, rows 8g + 4h + u
+    const int col = j0 + n;
+    if (col >= N) return;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int row = 8 * (r >> 2) + 4 * h + (r & 3);
+        if (row >= rows) continue;
+        const int64_t o = (int64_t)(i0 + row) * N + col;
+        if constexpr (GLU) {
+            const bf16_t pe = (bf16_t)tot[0][r], pg = (bf16_t)tot[1][r];
+            ((bf16_t *)y)[o] = silu_fwd_one<bf16_t>(pe, pg);
+            if (e_out) ((bf16_t *)e_out)[o] = pe;
+            if (g_out) ((bf16_t *)g_out)[o] = pg;
+        } else {
+            y[o] = from_f32<TO>(tot[0][r]);
+        }
+    }
+}
+
+template <bool GLU, typename TO>
+int launch_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
+                  const void *m_sizes, int ms_i64, TO *y, TO *e_out, TO *g_out, int64_t R, int N, int K, int E,
+                  hipStream_t stream) {
+    using S = StreamShape<GLU>;
+    constexpr int kLds = S::kLds;
+    const int tiles_n = ceil_div(N, 128);
+    const int64_t row_tiles = R / 32 + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / 32)
+    const int64_t grid = row_tiles * tiles_n;
+    if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
+    auto *kernel = nf4_stream_kernel<GLU, TO>;
+    static PerDeviceOnce attr;
+    const hipError_t e = attr.run([&] {
+        return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    });
+    if (e != hipSuccess) return (int)e;
+    kernel<<<(unsigned)grid, 256, kLds, stream>>>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, y, e_out, g_out,
+                                                          R, N, K, E, tiles_n);
+    return launch_status();
+}
+
+}  // namespace
+
+int gemm_nf4_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
+                    bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
+                    int K, int E, int out_dtype, hipStream_t stream) {
+    // a 64-wide step must lie inside one quantisation block, and the scales are copied four bytes at a time
+    if (K % 128 != 0 || w0.bs_shift < 6 || w1.bs_shift < 6) return MFL_ERR_UNSUPPORTED;
+    if (!aligned(w0.absmax, 4) || !aligned(w1.absmax, 4)) return MFL_ERR_UNSUPPORTED;
+    if (glu)
+        return launch_stream<true, bf16_t>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (bf16_t *)y, (bf16_t *)e_out,
+                                           (bf16_t *)g_out, R, N, K, E, stream);
+    if (out_dtype == MFL_BF16)
+        return launch_stream<false, bf16_t>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (bf16_t *)y, nullptr, nullptr,
+                                            R, N, K, E, stream);
+    return launch_stream<false, float>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (float *)y, nullptr, nullptr, R, N,
+                                       K, E, stream);
+}
+
+}  // namespace mfl
