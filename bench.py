@@ -292,6 +292,22 @@ def main() -> int:
         us = _event_us(lambda i: softmax_topk_raw(lg, TOPK, True, torch.bfloat16), it, wm, stream)
         b = TOKENS * E * 4 + TOKENS * TOPK * (4 + 2 + 8)
         extra["softmax_topk_4096"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 2)}
+        # both as the block calls them: one library call (two launches), one allocation; eager calls are bound
+        # by the host side of the call, the graph replay is the GPU side
+        from qwen3_moe_fused.kernels.routing import route_and_sort
+        with torch.no_grad():
+            us = _event_us(lambda i: route_and_sort(lg, TOPK, True, torch.bfloat16, E), it, wm, stream)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                route_and_sort(lg, TOPK, True, torch.bfloat16, E)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                route_and_sort(lg, TOPK, True, torch.bfloat16, E)
+            us_g = _event_us(lambda i: graph.replay(), it, wm, stream)
+            del graph
+        extra["route_and_sort_4096"] = {"us": round(us, 1), "hip_graph_replay_us": round(us_g, 1)}
         # NF4: fused dequant+GEMM vs dequant-then-GEMM at 16 / 256 / 16384 tokens (config 5 gate_proj)
         # three packed weight sets in rotation: the 113 MB of one set would stay in the 256 MB MALL between
         # launches, and the figure would not be an HBM figure

@@ -193,6 +193,19 @@ MFL_API int mfl_route_sort_small(const void *logits, int logits_dtype, int64_t T
                          float *weights_f32, void *weights_cast, int cast_dtype, int64_t *idx,
                          int32_t *counts, int32_t *sort_idx, int32_t *inv_sort_idx, void *stream);
 
+/* mfl_route_softmax_topk followed by mfl_expert_sort of its T * k selections, for any T: one launch
+ * up to 64 tokens (mfl_route_sort_small), otherwise two (the top-k kernel leaves a histogram of
+ * experts per 256 selections, which is the counting pass of the sort), three where the two-launch
+ * form does not apply (E > 512, more than 1024 * 256 selections).  Same outputs as the separate
+ * calls, bit for bit; both index arrays are required.  workspace: mfl_route_sort_workspace(T, E, k)
+ * bytes, 256-byte aligned.
+ * Replaces qwen3_moe_fused/modular_qwen3_moe_fused.py:87-93 + kernels/indexing.py:48-65. */
+MFL_API size_t mfl_route_sort_workspace(int64_t T, int E, int k);
+MFL_API int mfl_route_sort(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm,
+                   float *weights_f32, void *weights_cast, int cast_dtype, int64_t *idx,
+                   int32_t *counts, int32_t *sort_idx, int32_t *inv_sort_idx, void *workspace,
+                   size_t ws_bytes, void *stream);
+
 /* Stable counting sort of expert ids sel (R,) in [0, E):
  *   counts[e]        = #{j : sel[j] == e}
  *   sort_idx[i]      = j of the i-th row in the stable ascending order
@@ -224,6 +237,13 @@ MFL_API int mfl_expert_sort_static(const void *sel, int sel_dtype, int64_t R, in
  * qwen3_moe_fused/modular_qwen3_moe_fused.py:95-103.  row_scale has `dtype` elements. */
 MFL_API int mfl_gather_rows(const void *src, const int32_t *idx, int idx_div, const void *row_scale,
                     void *dst, int64_t R_out, int H, int dtype, void *stream);
+
+/* The same copy written from the source's side: dst[pos[r*k+j], :] = src[r, :] * (row_scale ?
+ * row_scale[r*k+j] : 1) for r < R_src, j < k, with pos a permutation of [0, R_src*k) (pos =
+ * inv_sort_idx gives what mfl_gather_rows gives with idx = sort_idx, bit for bit).  Every source
+ * row is read once instead of k times.  Replaces modular_qwen3_moe_fused.py:95-103 as well. */
+MFL_API int mfl_scatter_rows(const void *src, const int32_t *pos, int k, const void *row_scale,
+                     void *dst, int64_t R_src, int H, int dtype, void *stream);
 
 /* dst[t, :] = sum_{j<k} src[pos[t*k+j], :] * (weights ? weights[t*k+j] : 1), fp32 accumulate.
  * With pos = inv_sort_idx this is "un-sort, then weighted sum over the k selections",

@@ -149,6 +149,27 @@ def test_gather_and_combine(T, k, H, dtype):
                 "combine")
 
 
+@pytest.mark.parametrize("T,k,H,dtype,scaled", [(300, 8, 2048, torch.bfloat16, False), (300, 8, 2048, torch.bfloat16, True),
+                                                  (41, 3, 100, torch.float32, True), (64, 2, 36, torch.float16, False),
+                                                  (5, 1, 8, torch.float32, True)])
+def test_scatter_form_of_the_row_copy_equals_the_gather_form(T, k, H, dtype, scaled):
+    from qwen3_moe_fused.kernels.routing import _gather, _scatter
+
+    g = gen(T + H)
+    src = randn((T, H), g, 1.0, dtype).to(DEV)
+    sort_idx = torch.randperm(T * k, generator=g).to(torch.int32)
+    inv = torch.empty_like(sort_idx)
+    inv[sort_idx.long()] = torch.arange(T * k, dtype=torch.int32)
+    scale = randn((T * k,), g, 1.0, dtype).to(DEV) if scaled else None
+    a = _gather(src, sort_idx.to(DEV), k, scale)
+    b = _scatter(src, inv.to(DEV), k, scale)
+    assert torch.equal(a, b)
+    exp = src.cpu()[(sort_idx.long() // k)]
+    if scaled:
+        exp = (exp.float() * scale.cpu().float()[sort_idx.long()][:, None]).to(dtype)
+    assert torch.equal(a.cpu(), exp)
+
+
 def test_gather_combine_autograd_fp32():
     """Gradients of gather / combine / softmax-top-k against torch autograd of the reference's
     formulation (modular_qwen3_moe_fused.py:87-115)."""
@@ -205,18 +226,7 @@ def test_rows_dot_against_numpy(T, k, H, dtype):
     check_close(dots, ref, tol, tol, "rows_dot")
 
 
-@pytest.mark.parametrize("T,E,k,dtype", [(16, 128, 8, torch.float32), (1, 128, 8, torch.bfloat16), (128, 128, 8, torch.bfloat16),
-                                         (7, 11, 3, torch.float32), (100, 512, 6, torch.float32), (33, 60, 1, torch.float32),
-                                         (129, 128, 8, torch.float32)])          # the last: past the limit, separate calls
-def test_route_and_sort_in_one_launch_equals_the_separate_calls(T, E, k, dtype, monkeypatch):
-    from qwen3_moe_fused.kernels import routing
-    from qwen3_moe_fused.kernels.routing import route_and_sort
-
-    # the wrapper switches to the separate calls earlier than the entry point must (it is slower
-    # from about 64 tokens on): lift its threshold to the entry point's limit for this test
-    monkeypatch.setattr(routing, "SMALL_ROUTE_MAX_TOKENS", 128)
-    logits = randn((T, E), gen(T + E), 2.0, dtype).to(DEV)
-    w, sel, m_sizes, sort_idx, inv = route_and_sort(logits, k, True, torch.bfloat16, E)
+def _check_route_outputs(logits, k, E, w, sel, m_sizes, sort_idx, inv):
     _, w_ref, sel_ref = softmax_topk_raw(logits, k, True, torch.bfloat16)
     c_ref, s_ref, i_ref = get_expert_counts_and_idx(sel_ref.view(-1), E)
     assert torch.equal(sel, sel_ref) and torch.equal(w, w_ref)
@@ -225,3 +235,37 @@ def test_route_and_sort_in_one_launch_equals_the_separate_calls(T, E, k, dtype, 
     c_o, s_o, i_o = oracle.expert_counts_and_idx(sel.view(-1).cpu().numpy(), E)
     assert np.array_equal(m_sizes.cpu().numpy(), c_o) and np.array_equal(sort_idx.cpu().numpy(), s_o)
     assert np.array_equal(inv.cpu().numpy(), i_o)
+
+
+# one launch up to 64 tokens; two launches (top-k that counts, scatter) above; three where the two-launch form
+# does not apply: more than 512 experts, more than 1024 segments of 256 selections
+@pytest.mark.parametrize("T,E,k,dtype", [(16, 128, 8, torch.float32), (1, 128, 8, torch.bfloat16), (64, 128, 8, torch.bfloat16),
+                                         (7, 11, 3, torch.float32), (60, 512, 6, torch.float32), (33, 60, 1, torch.float32),
+                                         (65, 128, 8, torch.float32), (129, 128, 8, torch.float32),
+                                         (4096, 128, 8, torch.bfloat16), (777, 60, 3, torch.float32),
+                                         (5000, 512, 6, torch.float32), (300, 600, 4, torch.float32),
+                                         (33000, 128, 8, torch.bfloat16), (2049, 64, 64, torch.float32)])
+def test_route_and_sort_equals_the_separate_calls(T, E, k, dtype):
+    from qwen3_moe_fused.kernels.routing import route_and_sort
+
+    logits = randn((T, E), gen(T + E), 2.0, dtype).to(DEV)
+    w, sel, m_sizes, sort_idx, inv = route_and_sort(logits, k, True, torch.bfloat16, E)
+    _check_route_outputs(logits, k, E, w, sel, m_sizes, sort_idx, inv)
+
+
+@pytest.mark.parametrize("T,E,k", [(128, 128, 8), (100, 512, 6), (65, 40, 5)])
+def test_one_launch_entry_point_up_to_its_own_limit(T, E, k):
+    # mfl_route_sort uses the one-workgroup form up to 64 tokens; the entry point itself takes up to 128
+    from qwen3_moe_fused import _lib
+
+    logits = randn((T, E), gen(T), 2.0).to(DEV)
+    w = torch.empty((T, k), device=DEV, dtype=torch.bfloat16)
+    sel = torch.empty((T, k), device=DEV, dtype=torch.int64)
+    m_sizes = torch.empty(E, device=DEV, dtype=torch.int32)
+    sort_idx = torch.empty(T * k, device=DEV, dtype=torch.int32)
+    inv = torch.empty(T * k, device=DEV, dtype=torch.int32)
+    rc = _lib.lib().mfl_route_sort_small(_lib.ptr(logits), _lib.dtype_code(logits.dtype), T, E, k, 1, None, _lib.ptr(w),
+                                         _lib.dtype_code(w.dtype), _lib.ptr(sel), _lib.ptr(m_sizes), _lib.ptr(sort_idx),
+                                         _lib.ptr(inv), _lib.stream())
+    _lib.check(rc, "mfl_route_sort_small")
+    _check_route_outputs(logits, k, E, w, sel, m_sizes, sort_idx, inv)

@@ -279,6 +279,23 @@ int mfl_route_sort_small(const void *logits, int logits_dtype, int64_t T, int E,
                             (hipStream_t)stream);
 }
 
+size_t mfl_route_sort_workspace(int64_t T, int E, int k) {
+    if (T < 0 || E <= 0 || k <= 0) return 0;
+    return route_sort_workspace(T, E, k);
+}
+
+int mfl_route_sort(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, float *weights_f32,
+                   void *weights_cast, int cast_dtype, int64_t *idx, int32_t *counts, int32_t *sort_idx,
+                   int32_t *inv_sort_idx, void *workspace, size_t ws_bytes, void *stream) {
+    if (T < 0 || E <= 0 || k <= 0 || k > E || k > 64 || T * k > 0x7fffffff) return MFL_ERR_SHAPE;
+    if (!dtype_ok(logits_dtype) || (weights_cast && !dtype_ok(cast_dtype))) return MFL_ERR_DTYPE;
+    if (!counts || (T > 0 && (!logits || !idx || !sort_idx || !inv_sort_idx))) return MFL_ERR_NULL;
+    if (T == 0) return expert_sort(idx, 1, 0, E, counts, sort_idx, inv_sort_idx, workspace, ws_bytes, (hipStream_t)stream);
+    return route_sort(logits, logits_dtype, T, E, k, renorm, weights_f32, weights_cast,
+                      weights_cast ? cast_dtype : MFL_F32, idx, counts, sort_idx, inv_sort_idx, workspace, ws_bytes,
+                      (hipStream_t)stream);
+}
+
 size_t mfl_expert_sort_workspace(int64_t R, int E) { return expert_sort_workspace(R, E); }
 
 int mfl_expert_sort(const void *sel, int sel_dtype, int64_t R, int E, int32_t *counts, int32_t *sort_idx,
@@ -304,6 +321,14 @@ int mfl_gather_rows(const void *src, const int32_t *idx, int idx_div, const void
     if (!dtype_ok(dtype)) return MFL_ERR_DTYPE;
     if (R_out > 0 && (!src || !idx || !dst)) return MFL_ERR_NULL;
     return gather_rows(src, idx, idx_div, row_scale, dst, R_out, H, dtype, (hipStream_t)stream);
+}
+
+int mfl_scatter_rows(const void *src, const int32_t *pos, int k, const void *row_scale, void *dst, int64_t R_src, int H,
+                     int dtype, void *stream) {
+    if (R_src < 0 || H <= 0 || k <= 0 || R_src * k > 0x7fffffff) return MFL_ERR_SHAPE;
+    if (!dtype_ok(dtype)) return MFL_ERR_DTYPE;
+    if (R_src > 0 && (!src || !pos || !dst)) return MFL_ERR_NULL;
+    return scatter_rows(src, pos, k, row_scale, dst, R_src, H, dtype, (hipStream_t)stream);
 }
 
 int mfl_combine_rows(const void *src, const int32_t *pos, const void *weights, void *dst, int64_t T, int k, int H,

@@ -37,7 +37,7 @@ __device__ __forceinline__ float wave_max_f32(float x) {
 
 // One wave per token.  Lane l holds experts l, l+64, l+128, ... (VPL of them).
 template <typename TI, typename TC, int VPL>
-__device__ __forceinline__ void topk_one_token(const TI *__restrict__ logits, int64_t t, int E, int k, int renorm,
+__device__ __forceinline__ int topk_one_token(const TI *__restrict__ logits, int64_t t, int E, int k, int renorm,
                                                float *__restrict__ w_f32, TC *__restrict__ w_cast,
                                                int64_t *__restrict__ idx, int lane) {
     const TI *row = logits + t * E;
@@ -110,6 +110,7 @@ __device__ __forceinline__ void topk_one_token(const TI *__restrict__ logits, in
         if (w_cast) w_cast[t * k + lane] = from_f32<TC>(w);
         idx[t * k + lane] = my_i;
     }
+    return my_i;  // lanes below k: the lane's selection
 }
 
 template <typename TI, typename TC, int VPL>
@@ -530,6 +531,180 @@ __global__ __launch_bounds__(1024) void fast_scatter_kernel(const void *__restri
     }
 }
 
+// ---- routing in two launches: softmax + top-k that also counts, then the scatter
+// route_count_kernel: one workgroup per segment of tokens_per_seg tokens (at most 256 selections, the
+// segment one wave of the scatter kernel ranks), one wave per token (in turn, where a segment has more
+// tokens than the workgroup has waves).  Besides the routing weights and the selections it leaves the
+// segment's histogram of experts in table_raw[segment][E] (LDS atomics on integers: the sums do not depend
+// on their order).
+template <typename TI, typename TC, int VPL>
+__global__ __launch_bounds__(1024) void route_count_kernel(const TI *__restrict__ logits, int64_t T, int E, int k,
+                                                           int renorm, float *__restrict__ w_f32,
+                                                           TC *__restrict__ w_cast, int64_t *__restrict__ idx,
+                                                           int tokens_per_seg, int32_t *__restrict__ table_raw) {
+    extern __shared__ int lds[];  // [E]
+    const int wib = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int i = threadIdx.x; i < E; i += blockDim.x) lds[i] = 0;
+    __syncthreads();
+    for (int tt = wib; tt < tokens_per_seg; tt += kFastWaves) {
+        const int64_t t = (int64_t)blockIdx.x * tokens_per_seg + tt;
+        if (t >= T) break;
+        const int sel = topk_one_token<TI, TC, VPL>(logits, t, E, k, renorm, w_f32, w_cast, idx, lane);
+        if (lane < k) atomicAdd(&lds[sel], 1);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < E; i += blockDim.x) table_raw[(int64_t)blockIdx.x * E + i] = lds[i];
+}
+
+// fast_scatter_kernel on the raw histograms of route_count_kernel: wave w of the launch ranks segment w
+// (seg_keys selections, at most 256).  Everything the workgroup needs from global memory is requested at the
+// start, in one go: its waves' selections, the n_segs raw histograms (for the totals per expert and the rows
+// in earlier workgroups, which fast_count_kernel would have left in its tables) and, once more, the 16
+// histograms of its own segments; what follows works in LDS.
+__global__ __launch_bounds__(1024) void route_scatter_kernel(const int64_t *__restrict__ sel, int64_t R, int E,
+                                                             int key_bits, int seg_keys, int n_segs,
+                                                             const int32_t *__restrict__ table_raw,
+                                                             int32_t *__restrict__ counts,
+                                                             int32_t *__restrict__ sort_idx,
+                                                             int32_t *__restrict__ inv_sort_idx) {
+    extern __shared__ int lds[];  // base [E], before [E], offsets [16][E], histograms [16][E]
+    int *base = lds;
+    int *befo = base + E;
+    int *offs = befo + E;
+    int *hists = offs + kFastWaves * E;
+    const int tid = threadIdx.x, wib = tid >> 6, lane = tid & 63;
+    const int seg = blockIdx.x * kFastWaves + wib;
+    const int first_seg = blockIdx.x * kFastWaves;
+    const int64_t sb = (int64_t)seg * seg_keys;
+    int64_t se = sb + seg_keys;
+    if (se > R) se = R;
+    int keys[kFastBatches];
+#pragma unroll
+    for (int u = 0; u < kFastBatches; ++u) {
+        const int64_t j = sb + u * 64 + lane;
+        int key = -1;
+        if (seg < n_segs && j < se) {
+            const int64_t k64 = sel[j];
+            key = (k64 >= 0 && k64 < E) ? (int)k64 : -1;
+        }
+        keys[u] = key;
+    }
+    // the raw histograms of this workgroup's segments
+    for (int i = tid; i < kFastWaves * E; i += blockDim.x) {
+        const int w = i / E;
+        offs[i] = first_seg + w < n_segs ? table_raw[(int64_t)first_seg * E + i] : 0;
+    }
+    // Totals and rows in earlier workgroups, per expert: column sums of the n_segs x E table.  The threads
+    // split the rows among them, load eight rows at a time before they add any (a loop of load-then-add
+    // pays the L2 latency once per row: 15 us for 256 rows) and meet in LDS (integer atomics).
+    for (int e = tid; e < 2 * E; e += blockDim.x) base[e] = 0;  // base and befo
+    __syncthreads();
+    if ((E & 3) == 0) {
+        const int EV = E >> 2, rpp = blockDim.x / EV;
+        const int r0 = tid / EV, c = tid - r0 * EV;
+        if (r0 < rpp) {
+            const int4 *t4 = (const int4 *)table_raw;
+            int4 total = {0, 0, 0, 0}, before = {0, 0, 0, 0};
+            for (int s0 = r0; s0 < n_segs; s0 += 8 * rpp) {
+                int4 v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int sgm = s0 + u * rpp;
+                    v[u] = sgm < n_segs ? t4[(int64_t)sgm * EV + c] : int4{0, 0, 0, 0};
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    total.x += v[u].x, total.y += v[u].y, total.z += v[u].z, total.w += v[u].w;
+                    if (s0 + u * rpp < first_seg)
+                        before.x += v[u].x, before.y += v[u].y, before.z += v[u].z, before.w += v[u].w;
+                }
+            }
+            atomicAdd(&base[4 * c + 0], total.x), atomicAdd(&base[4 * c + 1], total.y);
+            atomicAdd(&base[4 * c + 2], total.z), atomicAdd(&base[4 * c + 3], total.w);
+            if (first_seg > 0) {
+                atomicAdd(&befo[4 * c + 0], before.x), atomicAdd(&befo[4 * c + 1], before.y);
+                atomicAdd(&befo[4 * c + 2], before.z), atomicAdd(&befo[4 * c + 3], before.w);
+            }
+        }
+    } else {
+        const int rpp = blockDim.x / E;
+        const int r0 = tid / E, e = tid - r0 * E;
+        if (r0 < rpp) {
+            int total = 0, before = 0;
+            for (int s0 = r0; s0 < n_segs; s0 += 8 * rpp) {
+                int v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int sgm = s0 + u * rpp;
+                    v[u] = sgm < n_segs ? table_raw[(int64_t)sgm * E + e] : 0;
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    total += v[u];
+                    if (s0 + u * rpp < first_seg) before += v[u];
+                }
+            }
+            atomicAdd(&base[e], total);
+            if (first_seg > 0) atomicAdd(&befo[e], before);
+        }
+    }
+    __syncthreads();
+    if (blockIdx.x == 0)
+        for (int e = tid; e < E; e += blockDim.x) counts[e] = base[e];
+    if (sort_idx == nullptr && inv_sort_idx == nullptr) return;
+    if (wib == 0) {  // exclusive scan of the totals over the experts, plus the part of earlier workgroups
+        int carry = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int v = e < E ? base[e] : 0;
+            int inc = v;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int up = __shfl_up(inc, o);
+                if (lane >= o) inc += up;
+            }
+            if (e < E) befo[e] = carry + inc - v + befo[e];  // base stays: workgroup 0 may still be copying it to counts
+            carry += __shfl(inc, 63);
+        }
+    }
+    int *hist = hists + wib * E;
+    for (int i = lane; i < E; i += 64) hist[i] = 0;
+    __syncthreads();
+    // offsets of this workgroup's waves: first row of the expert, plus its rows in the workgroup's earlier segments
+    for (int e = tid; e < E; e += blockDim.x) {
+        int run = befo[e];
+#pragma unroll
+        for (int w = 0; w < kFastWaves; ++w) {
+            const int c = offs[w * E + e];
+            offs[w * E + e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    if (seg >= n_segs) return;
+    const int *my_off = offs + wib * E;
+    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+    for (int u = 0; u < kFastBatches; ++u) {
+        const int key = keys[u];
+        const bool valid = key >= 0;
+        uint64_t same = __ballot(valid);
+        if (same == 0) continue;  // past the end of the segment
+        for (int b = 0; b < key_bits; ++b) {
+            const uint64_t bal = __ballot((key >> b) & 1);
+            same &= ((key >> b) & 1) ? bal : ~bal;
+        }
+        if (valid) {
+            const int before = hist[key];
+            const int pos = before + __popcll(same & lt_mask) + my_off[key];
+            if ((same >> lane) == 1ull) hist[key] = before + __popcll(same);
+            const int64_t j = sb + u * 64 + lane;
+            if (inv_sort_idx) inv_sort_idx[j] = pos;
+            if (sort_idx) sort_idx[pos] = (int32_t)j;
+        }
+    }
+}
+
 inline int fast_waves(int64_t R) {
     int64_t w = (R + 64 * kFastBatches - 1) / (64 * kFastBatches);
     if (w > kFastMaxBlocks * kFastWaves) w = kFastMaxBlocks * kFastWaves;
@@ -598,6 +773,83 @@ int route_sort_small(const void *logits, int logits_dtype, int64_t T, int E, int
     MFL_DISPATCH_FLOAT(logits_dtype, TI, MFL_DISPATCH_FLOAT(cast_dtype, TC, rc = (launch_route_sort_small<TI, TC>(
         logits, T, E, k, renorm, w_f32, w_cast, idx, counts, sort_idx, inv_sort_idx, stream))));
     return rc;
+}
+
+namespace {
+
+// Segments of the two-launch routing: whole tokens, at most 256 selections; a token per wave of the top-k
+// workgroup (16) while that keeps the segments under 1024, more tokens per segment beyond.  0: does not apply.
+inline int route_tokens_per_seg(int64_t T, int E, int k) {
+    if (T <= 0 || E > 512 || k > 64 || T * k > 0x7fffffff) return 0;
+    const int most = 256 / k;  // k <= 64
+    int64_t tps = (T + kFastMaxBlocks * kFastWaves - 1) / (kFastMaxBlocks * kFastWaves);
+    if (tps < kFastWaves) tps = kFastWaves;
+    if (tps > most) tps = most;
+    return (T + tps - 1) / tps <= kFastMaxBlocks * kFastWaves ? (int)tps : 0;
+}
+
+template <typename TI, typename TC>
+int launch_route_count(const void *logits, int64_t T, int E, int k, int renorm, float *w_f32, void *w_cast,
+                       int64_t *idx, int tps, int n_segs, int32_t *table_raw, hipStream_t stream) {
+    const int vpl = ceil_div(E, 64);
+    const size_t lds = (size_t)E * 4;
+#define MFL_RC(V)                                                                                         \
+    route_count_kernel<TI, TC, V><<<n_segs, kFastWaves * 64, lds, stream>>>(                              \
+        (const TI *)logits, T, E, k, renorm, w_f32, (TC *)w_cast, idx, tps, table_raw)
+    if (vpl <= 1)
+        MFL_RC(1);
+    else if (vpl <= 2)
+        MFL_RC(2);
+    else if (vpl <= 4)
+        MFL_RC(4);
+    else
+        MFL_RC(8);
+#undef MFL_RC
+    return launch_status();
+}
+
+}  // namespace
+
+size_t route_sort_workspace(int64_t T, int E, int k) {
+    if (const int tps = route_tokens_per_seg(T, E, k)) {
+        return (((size_t)((T + tps - 1) / tps) * (size_t)E * 4) + 255) / 256 * 256;
+    }
+    return expert_sort_workspace(T * k, E);
+}
+
+int route_sort(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, float *w_f32, void *w_cast,
+               int cast_dtype, int64_t *idx, int32_t *counts, int32_t *sort_idx, int32_t *inv_sort_idx,
+               void *workspace, size_t ws_bytes, hipStream_t stream) {
+    // up to 64 tokens one workgroup does it all in one launch (above, its single workgroup is the slower way)
+    int rc = T <= 64 ? route_sort_small(logits, logits_dtype, T, E, k, renorm, w_f32, w_cast, cast_dtype, idx, counts,
+                                        sort_idx, inv_sort_idx, stream)
+                     : MFL_ERR_UNSUPPORTED;
+    if (rc != MFL_ERR_UNSUPPORTED) return rc;
+    const int tps = route_tokens_per_seg(T, E, k);
+    if (tps == 0) {
+        rc = route_softmax_topk(logits, logits_dtype, T, E, k, renorm, w_f32, w_cast, cast_dtype, idx, stream);
+        if (rc) return rc;
+        return expert_sort(idx, 1, T * k, E, counts, sort_idx, inv_sort_idx, workspace, ws_bytes, stream);
+    }
+    const int n_segs = (int)((T + tps - 1) / tps);
+    if (workspace == nullptr || ws_bytes < (size_t)n_segs * E * 4) return MFL_ERR_WORKSPACE;
+    int32_t *table_raw = (int32_t *)workspace;
+    rc = MFL_ERR_DTYPE;
+    MFL_DISPATCH_FLOAT(logits_dtype, TI, MFL_DISPATCH_FLOAT(cast_dtype, TC, rc = (launch_route_count<TI, TC>(
+        logits, T, E, k, renorm, w_f32, w_cast, idx, tps, n_segs, table_raw, stream))));
+    if (rc) return rc;
+    int key_bits = 0;
+    while ((1 << key_bits) < E) ++key_bits;
+    static PerDeviceOnce attr;
+    const hipError_t e = attr.run([] {
+        return hipFuncSetAttribute((const void *)route_scatter_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   34 * 512 * 4);
+    });
+    if (e != hipSuccess) return (int)e;
+    const size_t lds2 = (size_t)(2 * kFastWaves + 2) * E * 4;
+    route_scatter_kernel<<<ceil_div(n_segs, kFastWaves), kFastWaves * 64, lds2, stream>>>(
+        idx, T * k, E, key_bits, tps * k, n_segs, table_raw, counts, sort_idx, inv_sort_idx);
+    return launch_status();
 }
 
 size_t expert_sort_workspace(int64_t R, int E) {

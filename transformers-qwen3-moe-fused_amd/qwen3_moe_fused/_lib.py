@@ -45,10 +45,13 @@ _SIGNATURES = {
     "mfl_nf4_quant": (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _vp]),
     "mfl_route_softmax_topk": (_i, [_vp, _i, _i64, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
     "mfl_route_sort_small": (_i, [_vp, _i, _i64, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
+    "mfl_route_sort_workspace": (_sz, [_i64, _i, _i]),
+    "mfl_route_sort": (_i, [_vp, _i, _i64, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "mfl_expert_sort_workspace": (_sz, [_i64, _i]),
     "mfl_expert_sort": (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _vp, _sz, _vp]),
     "mfl_expert_sort_static": (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _vp]),
     "mfl_gather_rows": (_i, [_vp, _vp, _i, _vp, _vp, _i64, _i, _i, _vp]),
+    "mfl_scatter_rows": (_i, [_vp, _vp, _i, _vp, _vp, _i64, _i, _i, _vp]),
     "mfl_combine_rows": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
     "mfl_rows_dot": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
     "mfl_silu_mul_fwd": (_i, [_vp, _vp, _vp, _i64, _i, _vp]),

@@ -62,16 +62,18 @@ def _softmax_topk_backward(logits, idx, w32, renorm, dw):
     return dlogits.to(logits.dtype)
 
 
-# Up to this many tokens, top-k and the expert sort run as one launch of one workgroup (with the
-# wrapper: 21 us at 16 and at 64 tokens, 35 us at 128, against 36 us for the three separate launches
-# at any of these sizes, of which about 22 us are kernel time).
-SMALL_ROUTE_MAX_TOKENS = 64
+_ROUTE_WS_BYTES = {}  # (T, E, k) -> bytes of scratch mfl_route_sort asks for
+
+
+def _round256(n: int) -> int:
+    return (n + 255) // 256 * 256
 
 
 class _RouteAndSort(torch.autograd.Function):
-    """softmax + top-k and the stable expert sort of its selections.  Decode-sized batches take
-    one launch (``mfl_route_sort_small``); otherwise the two separate calls run.  Returns
-    (routing weights (T,k), expert ids (T,k) int64, m_sizes (E,), sort_idx, inv_sort_idx)."""
+    """softmax + top-k and the stable expert sort of its selections: one library call
+    (``mfl_route_sort``: one launch up to 64 tokens, two above) and ONE allocation, of which the
+    outputs and the call's scratch are views.  Returns (routing weights (T,k), expert ids (T,k) int64,
+    m_sizes (E,), sort_idx, inv_sort_idx)."""
 
     @staticmethod
     def forward(ctx, logits, k, renorm, out_dtype, num_experts):
@@ -79,24 +81,30 @@ class _RouteAndSort(torch.autograd.Function):
         T, E = logits.shape
         assert E == num_experts
         out_dtype = logits.dtype if out_dtype is None else out_dtype
-        rc = -6
-        if 0 < T <= SMALL_ROUTE_MAX_TOKENS:
-            w32 = torch.empty((T, k), device=logits.device, dtype=torch.float32)
-            wc = torch.empty((T, k), device=logits.device, dtype=out_dtype)
-            idx = torch.empty((T, k), device=logits.device, dtype=torch.int64)
-            buf = torch.empty(E + 2 * T * k, device=logits.device, dtype=torch.int32)
-            m_sizes, sort_idx, inv = buf[:E], buf[E:E + T * k], buf[E + T * k:]
-            rc = _lib.lib().mfl_route_sort_small(_lib.ptr(logits), _lib.dtype_code(logits.dtype), T, E, k,
-                                                 int(bool(renorm)), _lib.ptr(w32), _lib.ptr(wc),
-                                                 _lib.dtype_code(out_dtype), _lib.ptr(idx), _lib.ptr(m_sizes),
-                                                 _lib.ptr(sort_idx), _lib.ptr(inv), _lib.stream())
-            if rc != -6:  # MFL_ERR_UNSUPPORTED: fall through to the separate calls
-                _lib.check(rc, "mfl_route_sort_small")
-        if rc == -6:
-            from .indexing import get_expert_counts_and_idx
-
-            w32, wc, idx = softmax_topk_raw(logits, k, renorm, out_dtype)
-            m_sizes, sort_idx, inv = get_expert_counts_and_idx(idx.view(-1), E)
+        R = T * k
+        key = (T, E, k)
+        ws_bytes = _ROUTE_WS_BYTES.get(key)
+        if ws_bytes is None:
+            ws_bytes = _ROUTE_WS_BYTES[key] = int(_lib.lib().mfl_route_sort_workspace(T, E, k))
+        # 256-byte aligned pieces of one block: idx int64, w32 fp32, sort_idx / inv / m_sizes int32, weights, scratch
+        o_w32 = _round256(R * 8)
+        o_sort = o_w32 + _round256(R * 4)
+        o_inv = o_sort + _round256(R * 4)
+        o_ms = o_inv + _round256(R * 4)
+        o_wc = o_ms + _round256(E * 4)
+        o_ws = o_wc + _round256(R * out_dtype.itemsize)
+        buf = torch.empty(o_ws + ws_bytes, device=logits.device, dtype=torch.uint8)
+        idx = buf[:R * 8].view(torch.int64).view(T, k)
+        w32 = buf[o_w32:o_w32 + R * 4].view(torch.float32).view(T, k)
+        sort_idx = buf[o_sort:o_sort + R * 4].view(torch.int32)
+        inv = buf[o_inv:o_inv + R * 4].view(torch.int32)
+        m_sizes = buf[o_ms:o_ms + E * 4].view(torch.int32)
+        wc = buf[o_wc:o_wc + R * out_dtype.itemsize].view(out_dtype).view(T, k)
+        base = buf.data_ptr()
+        rc = _lib.lib().mfl_route_sort(_lib.ptr(logits), _lib.dtype_code(logits.dtype), T, E, k, int(bool(renorm)),
+                                       base + o_w32, base + o_wc, _lib.dtype_code(out_dtype), base, base + o_ms,
+                                       base + o_sort, base + o_inv, base + o_ws, ws_bytes, _lib.stream())
+        _lib.check(rc, "mfl_route_sort")
         ctx.save_for_backward(logits, idx, w32)
         ctx.renorm = renorm
         ctx.mark_non_differentiable(idx, m_sizes, sort_idx, inv)
@@ -134,6 +142,20 @@ def _gather(src: torch.Tensor, idx: torch.Tensor, div: int, row_scale: Optional[
     return out
 
 
+def _scatter(src: torch.Tensor, pos: torch.Tensor, k: int, row_scale: Optional[torch.Tensor]) -> torch.Tensor:
+    """out[pos[r * k + j]] = src[r] (* row_scale[r * k + j]): ``_gather`` with idx the inverse of ``pos``, every
+    source row read once."""
+    assert src.is_cuda and src.ndim == 2 and src.is_contiguous()
+    assert pos.dtype == torch.int32 and pos.is_contiguous() and pos.numel() == src.shape[0] * k
+    out = torch.empty((pos.numel(), src.shape[1]), device=src.device, dtype=src.dtype)
+    if row_scale is not None:
+        assert row_scale.dtype == src.dtype and row_scale.is_contiguous() and row_scale.numel() == pos.numel()
+    rc = _lib.lib().mfl_scatter_rows(_lib.ptr(src), _lib.ptr(pos), k, _lib.ptr(row_scale), _lib.ptr(out), src.shape[0],
+                                     src.shape[1], _lib.dtype_code(src.dtype), _lib.stream())
+    _lib.check(rc, "mfl_scatter_rows")
+    return out
+
+
 def _combine(src: torch.Tensor, pos: torch.Tensor, weights: Optional[torch.Tensor], T: int, k: int) -> torch.Tensor:
     assert src.is_cuda and src.ndim == 2 and src.is_contiguous()
     assert pos.dtype == torch.int32 and pos.is_contiguous() and pos.numel() == T * k
@@ -155,6 +177,8 @@ class _GatherRows(torch.autograd.Function):
         ctx.save_for_backward(inv)
         ctx.div = div
         ctx.n_src = src.shape[0]
+        if div > 1 and inv.numel() == src.shape[0] * div:
+            return _scatter(src, inv, div, None)  # every source row read once, not div times
         return _gather(src, idx, div, None)
 
     @staticmethod
@@ -188,7 +212,7 @@ class _CombineRows(torch.autograd.Function):
         dy = dw = None
         if ctx.needs_input_grad[0]:
             # dy[i] = dout[sort_idx[i] // k] * w.flat[sort_idx[i]]
-            dy = _gather(dout, sort_idx, k, w.view(-1))
+            dy = _scatter(dout, pos, k, w.view(-1)) if k > 1 else _gather(dout, sort_idx, k, w.view(-1))
         if ctx.needs_input_grad[2]:
             dw = torch.empty_like(w)
             rc = _lib.lib().mfl_rows_dot(_lib.ptr(dout), _lib.ptr(y), _lib.ptr(pos), _lib.ptr(dw), T, k, y.shape[1],
