@@ -12,9 +12,15 @@
  *     it: no synchronisation, no allocation, no host read of device data;
  *   - return value: 0 = OK, negative = argument error (MFL_ERR_*), positive =
  *     hipError_t of a failed launch;
- *   - the library keeps no mutable global state (device properties and per-kernel launch
- *     attributes are cached read-only at the first call, for the device that is current
- *     then: one device per process); calls are re-entrant.
+ *   - global state of the library, all of it: the properties of the device that is current at
+ *     the first call (cached read-only: one kind of device per process), one flag per kernel
+ *     and device saying that the kernel's launch attribute has been set there (atomic; two
+ *     threads racing through a first call both set the same value), and the fixed scratch
+ *     array of mfl_expert_sort_static, which is device memory that calls on one GPU share
+ *     (see there).  Apart from that array the calls are re-entrant and thread-safe;
+ *   - the code objects are built for gfx950 only, and the work distribution of the GEMM
+ *     kernels assumes its 8 XCDs (workgroup b runs on XCD b % 8, each XCD with an L2 of its
+ *     own): on another part the library does not load its kernels at all.
  */
 #ifndef MOE_FUSED_LINEAR_H
 #define MOE_FUSED_LINEAR_H
