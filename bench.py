@@ -70,9 +70,9 @@ def _kernel_tour(n, dev):
     from qwen3_moe_fused.grouped_gemm.forward import grouped_gemm_forward
     from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_4bit
     from qwen3_moe_fused.grouped_gemm.forward_transposed import grouped_gemm_forward_transposed
-    from qwen3_moe_fused.grouped_gemm.fused import grouped_glu_forward
+    from qwen3_moe_fused.grouped_gemm.fused import grouped_glu_forward, grouped_glu_forward_4bit
     from qwen3_moe_fused.kernels.indexing import get_expert_counts_and_idx
-    from qwen3_moe_fused.kernels.routing import combine_rows, gather_rows, softmax_topk_raw
+    from qwen3_moe_fused.kernels.routing import combine_rows, gather_rows, route_and_sort, softmax_topk_raw
     from qwen3_moe_fused.kernels.silu_mul import silu_mul_backward, silu_mul_forward
     from qwen3_moe_fused.quantize.nf4 import dequantize_nf4, quantize_nf4
 
@@ -91,28 +91,33 @@ def _kernel_tour(n, dev):
     w_down = rnd(E, HIDDEN, INTER, scale=0.02)
     h, h2, dh = rnd(ROWS, INTER), rnd(ROWS, INTER), rnd(ROWS, INTER)
     dy = rnd(ROWS, HIDDEN)
-    packed, qstate = quantize_nf4(w_gate, 64)
+    # three packed weight sets in rotation: one set (113 MB) would stay in the 256 MB MALL between launches
+    qsets = [quantize_nf4(w, 64) for w in (w_gate, w_up, rnd(E, INTER, HIDDEN, scale=0.02))]
+    packed, qstate = qsets[0]
     gemm_b = 2.0 * (ROWS * HIDDEN + E * INTER * HIDDEN + ROWS * INTER)
     gemm_f = 2.0 * ROWS * INTER * HIDDEN
     nf4_b = E * INTER * HIDDEN * (0.5 + 4.0 / 64)
     legs = [
-        ("gemm_fwd gate_proj 4096 tokens", gemm_b, gemm_f, lambda: grouped_gemm_forward(x, w_gate, m_sizes)),
-        ("gemm_dx down_proj 4096 tokens", gemm_b, gemm_f, lambda: grouped_gemm_forward_transposed(dy, w_down, m_sizes)),
-        ("gemm_dw down_proj 4096 tokens", gemm_b, gemm_f, lambda: grouped_gemm_backward_dw(h, dy, m_sizes, bf)),
+        ("gemm_fwd gate_proj 4096 tokens", gemm_b, gemm_f, lambda i: grouped_gemm_forward(x, w_gate, m_sizes)),
+        ("gemm_dx down_proj 4096 tokens", gemm_b, gemm_f, lambda i: grouped_gemm_forward_transposed(dy, w_down, m_sizes)),
+        ("gemm_dw down_proj 4096 tokens", gemm_b, gemm_f, lambda i: grouped_gemm_backward_dw(h, dy, m_sizes, bf)),
         ("glu_fwd (gather + gate + up + SiLU-mul) 4096 tokens",
          2.0 * (TOKENS * HIDDEN + 2 * E * INTER * HIDDEN + ROWS * INTER), 2 * gemm_f,
-         lambda: grouped_glu_forward(hidden, w_gate, w_up, m_sizes, sort_idx, TOPK)),
-        ("silu_mul_fwd 32768 rows", 3.0 * ROWS * INTER * 2, 0.0, lambda: silu_mul_forward(h, h2)),
-        ("silu_mul_bwd 32768 rows", 5.0 * ROWS * INTER * 2, 0.0, lambda: silu_mul_backward(dh, h, h2)),
-        ("gather_rows 4096 tokens", 2.0 * (TOKENS + ROWS) * HIDDEN, 0.0,
-         lambda: gather_rows(hidden, sort_idx, TOPK, inv_sort_idx)),
+         lambda i: grouped_glu_forward(hidden, w_gate, w_up, m_sizes, sort_idx, TOPK)),
+        ("silu_mul_fwd 32768 rows", 3.0 * ROWS * INTER * 2, 0.0, lambda i: silu_mul_forward(h, h2)),
+        ("silu_mul_bwd 32768 rows", 5.0 * ROWS * INTER * 2, 0.0, lambda i: silu_mul_backward(dh, h, h2)),
+        ("gather_rows 4096 tokens (scatter form)", 2.0 * (TOKENS + ROWS) * HIDDEN, 0.0,
+         lambda i: gather_rows(hidden, sort_idx, TOPK, inv_sort_idx)),
         ("combine_rows 4096 tokens", 2.0 * (TOKENS + ROWS) * HIDDEN, 0.0,
-         lambda: combine_rows(dy, inv_sort_idx, rw, sort_idx)),
+         lambda i: combine_rows(dy, inv_sort_idx, rw, sort_idx)),
         ("softmax_topk 4096 tokens", TOKENS * E * 4.0 + TOKENS * TOPK * (4 + 2 + 8), 0.0,
-         lambda: softmax_topk_raw(logits, TOPK, True, bf)),
+         lambda i: softmax_topk_raw(logits, TOPK, True, bf)),
         ("expert_sort 32768 rows", ROWS * 8.0 + 2 * ROWS * 4 + E * 4, 0.0,
-         lambda: get_expert_counts_and_idx(sel.view(-1), E)),
-        ("nf4_dequant gate_proj", nf4_b + 2.0 * E * INTER * HIDDEN, 0.0, lambda: dequantize_nf4(packed, qstate, bf)),
+         lambda i: get_expert_counts_and_idx(sel.view(-1), E)),
+        ("route_and_sort 4096 tokens (top-k that counts + scatter)",
+         TOKENS * E * 4.0 + TOKENS * TOPK * (4 + 2 + 8) + 2 * ROWS * 4 + E * 4, 0.0,
+         lambda i: route_and_sort(logits, TOPK, True, bf, E)),
+        ("nf4_dequant gate_proj", nf4_b + 2.0 * E * INTER * HIDDEN, 0.0, lambda i: dequantize_nf4(*qsets[i % 3], bf)),
     ]
     for tokens in (16, 256, 16384):
         lgt = torch.randn((tokens, E), device=dev, generator=g)
@@ -122,10 +127,15 @@ def _kernel_tour(n, dev):
         active = int((ms5 > 0).sum().item())
         legs.append((f"gemm_fwd_nf4 gate_proj {tokens} tokens ({active} experts hit)",
                      active * nf4_b / E + 2.0 * tokens * TOPK * (HIDDEN + INTER), 2.0 * tokens * TOPK * INTER * HIDDEN,
-                     lambda x5=x5, ms5=ms5: grouped_gemm_forward_4bit(x5, packed, qstate, ms5)))
+                     lambda i, x5=x5, ms5=ms5: grouped_gemm_forward_4bit(x5, *qsets[i % 3], ms5)))
+        if tokens <= 256:
+            legs.append((f"glu_fwd_nf4 (gate + up + SiLU-mul) {tokens} tokens ({active} experts hit)",
+                         2 * active * nf4_b / E + 2.0 * tokens * TOPK * (HIDDEN + INTER),
+                         4.0 * tokens * TOPK * INTER * HIDDEN,
+                         lambda i, x5=x5, ms5=ms5: grouped_glu_forward_4bit(x5, *qsets[i % 3], *qsets[(i + 1) % 3], ms5)))
     for name, nbytes, flops, fn in legs:
-        for _ in range(n):
-            fn()
+        for i in range(n):
+            fn(i)
         torch.cuda.synchronize()
         print(f"{name}: {n} launches, algorithmic {nbytes / 1e6:.1f} MB, {flops / 1e9:.2f} GFLOP per launch", flush=True)
 
