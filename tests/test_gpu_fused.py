@@ -71,7 +71,8 @@ def test_gathered_forward_matches_oracle_and_explicit_gather(T, E, k, N, K):
 
 
 @pytest.mark.parametrize("T,E,k,N,K,blocksize", [(512, 16, 4, 192, 256, 64), (40, 20, 2, 136, 128, 16),
-                                                 (1024, 4, 2, 264, 192, 32), (16, 128, 8, 768, 2048, 64)])
+                                                 (1024, 4, 2, 264, 192, 32), (16, 128, 8, 768, 2048, 64),
+                                                 (24, 6, 2, 136, 384, 128)])   # streaming kernel, ragged edges
 def test_gathered_nf4_forward(T, E, k, N, K, blocksize):
     ms, sort_idx, sel = _routing(T, E, k, T + N)
     x = randn((T, K), gen(T), 1.0, torch.bfloat16)
@@ -115,7 +116,8 @@ def test_glu_forward(T, E, k, N, K, gathered):
 
 @pytest.mark.parametrize("T,E,k,N,K,bs_g,bs_u", [(512, 16, 4, 192, 256, 64, 64), (40, 20, 2, 136, 128, 16, 32),
                                                  (1024, 4, 2, 264, 192, 32, 8), (16, 128, 8, 768, 2048, 64, 64),
-                                                 (256, 128, 8, 768, 2048, 64, 64)])
+                                                 (256, 128, 8, 768, 2048, 64, 64),
+                                                 (24, 6, 2, 136, 384, 64, 128)])   # streaming kernel, ragged edges
 def test_glu_nf4_forward(T, E, k, N, K, bs_g, bs_u):
     ms, sort_idx, sel = _routing(T, E, k, T + N + 2)
     x = randn((T, K), gen(T), 1.0, torch.bfloat16)

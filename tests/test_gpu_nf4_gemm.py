@@ -84,6 +84,41 @@ def test_random_shapes_fused_nf4(seed):
                 what=f"seed {seed}: E={E} N={N} K={K} blocksize={blocksize} m_sizes={ms.tolist()}")
 
 
+# The streaming decode-size kernel (K % 128 == 0, blocks of at least 64 weights, at most 32 rows per expert on
+# average): one stage, an odd number of stages, column counts that leave a wave or a workgroup partly or wholly
+# empty, experts of two and three row tiles, more than 64 experts, empty experts, large quantisation blocks,
+# 64-bit row counts, fp32 output, rows past sum(m_sizes).
+@pytest.mark.parametrize("m_sizes,N,K,blocksize,ms_dtype,out_dtype", [
+    ([3, 0, 1, 7], 8, 128, 64, torch.int32, torch.bfloat16),
+    ([5, 2], 136, 384, 64, torch.int64, torch.bfloat16),
+    ([33, 0, 70, 1, 0, 12], 200, 256, 128, torch.int32, torch.float32),
+    ([1] * 70 + [0] * 5 + [40], 64, 128, 64, torch.int32, torch.bfloat16),
+    ([9, 31, 32, 2], 264, 640, 512, torch.int64, torch.bfloat16),
+    ([0, 0, 6, 0], 768, 2048, 256, torch.int32, torch.bfloat16),
+])
+def test_streaming_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, out_dtype):
+    E = len(m_sizes)
+    ms = torch.tensor(m_sizes, dtype=ms_dtype)
+    R = int(ms.sum()) + 3                      # three rows past the last expert: not written
+    assert R <= 32 * E and K % 128 == 0 and blocksize >= 64 and (N * K) % blocksize == 0
+    packed, state, w_deq = _quantised(E, N, K, blocksize, N + K)
+    x = randn((R, K), gen(K), 1.0, torch.bfloat16)
+    sel = oracle.sel_from_m_sizes(np.asarray(m_sizes))
+    y = torch.full((R, N), 7.0, device=DEV, dtype=out_dtype)
+    from qwen3_moe_fused import _lib
+    xd, msd = x.to(DEV), ms.to(DEV)
+    rc = _lib.lib().mfl_gemm_fwd_nf4(_lib.ptr(xd), _lib.ptr(packed), _lib.ptr(state.code), _lib.ptr(state.absmax), blocksize,
+                                     _lib.ptr(msd), _lib.itype_code(ms_dtype), _lib.ptr(y), R, N, K, E,
+                                     _lib.dtype_code(torch.bfloat16), _lib.dtype_code(out_dtype), _lib.stream())
+    _lib.check(rc, "mfl_gemm_fwd_nf4")
+    ref = oracle.linear_fwd(to_np32(x)[:R - 3], w_deq, sel)
+    check_close(y[:R - 3], ref, what=f"streaming kernel m_sizes={m_sizes} N={N} K={K} blocksize={blocksize}")
+    assert torch.all(y[R - 3:] == 7.0), "rows past sum(m_sizes) stay as they were"
+    # through the wrapper, and again: the same bits
+    y2 = grouped_gemm_forward_4bit(xd, packed, state, msd, out_dtype)
+    assert torch.equal(y2[:R - 3], y[:R - 3])
+
+
 from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit  # noqa: E402
 from qwen3_moe_fused.grouped_gemm.forward_transposed import grouped_gemm_forward_transposed  # noqa: E402
 
