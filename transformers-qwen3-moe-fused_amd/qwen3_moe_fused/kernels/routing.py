@@ -69,42 +69,50 @@ def _round256(n: int) -> int:
     return (n + 255) // 256 * 256
 
 
+def _route_and_sort_raw(logits: torch.Tensor, k: int, renorm: bool, out_dtype: Optional[torch.dtype]):
+    """One library call (``mfl_route_sort``: one launch up to 64 tokens, two above) and ONE allocation, of which
+    the outputs and the call's scratch are views.  Returns (w32, weights, idx, m_sizes, sort_idx, inv_sort_idx)."""
+    assert logits.is_cuda and logits.ndim == 2 and logits.is_contiguous()
+    T, E = logits.shape
+    out_dtype = logits.dtype if out_dtype is None else out_dtype
+    R = T * k
+    key = (T, E, k)
+    ws_bytes = _ROUTE_WS_BYTES.get(key)
+    if ws_bytes is None:
+        ws_bytes = _ROUTE_WS_BYTES[key] = int(_lib.lib().mfl_route_sort_workspace(T, E, k))
+    # 256-byte aligned pieces of one block: idx int64, w32 fp32, sort_idx / inv / m_sizes int32, weights, scratch
+    o_w32 = _round256(R * 8)
+    o_sort = o_w32 + _round256(R * 4)
+    o_inv = o_sort + _round256(R * 4)
+    o_ms = o_inv + _round256(R * 4)
+    o_wc = o_ms + _round256(E * 4)
+    o_ws = o_wc + _round256(R * out_dtype.itemsize)
+    buf = torch.empty(o_ws + ws_bytes, device=logits.device, dtype=torch.uint8)
+    # one typed alias of the block per element type, then one strided view per output (every piece starts on a
+    # multiple of 256 bytes, the block's size is a multiple of 256)
+    i32 = buf.view(torch.int32)
+    idx = torch.as_strided(buf.view(torch.int64), (T, k), (k, 1), 0)
+    w32 = torch.as_strided(buf.view(torch.float32), (T, k), (k, 1), o_w32 // 4)
+    sort_idx = torch.as_strided(i32, (R,), (1,), o_sort // 4)
+    inv = torch.as_strided(i32, (R,), (1,), o_inv // 4)
+    m_sizes = torch.as_strided(i32, (E,), (1,), o_ms // 4)
+    wc = torch.as_strided(buf.view(out_dtype), (T, k), (k, 1), o_wc // out_dtype.itemsize)
+    base = buf.data_ptr()
+    rc = _lib.lib().mfl_route_sort(logits.data_ptr(), _lib.dtype_code(logits.dtype), T, E, k, int(bool(renorm)),
+                                   base + o_w32, base + o_wc, _lib.dtype_code(out_dtype), base, base + o_ms,
+                                   base + o_sort, base + o_inv, base + o_ws, ws_bytes, _lib.stream())
+    _lib.check(rc, "mfl_route_sort")
+    return w32, wc, idx, m_sizes, sort_idx, inv
+
+
 class _RouteAndSort(torch.autograd.Function):
-    """softmax + top-k and the stable expert sort of its selections: one library call
-    (``mfl_route_sort``: one launch up to 64 tokens, two above) and ONE allocation, of which the
-    outputs and the call's scratch are views.  Returns (routing weights (T,k), expert ids (T,k) int64,
-    m_sizes (E,), sort_idx, inv_sort_idx)."""
+    """softmax + top-k and the stable expert sort of its selections, differentiable in the logits.  Returns
+    (routing weights (T,k), expert ids (T,k) int64, m_sizes (E,), sort_idx, inv_sort_idx)."""
 
     @staticmethod
     def forward(ctx, logits, k, renorm, out_dtype, num_experts):
-        assert logits.is_cuda and logits.ndim == 2 and logits.is_contiguous()
-        T, E = logits.shape
-        assert E == num_experts
-        out_dtype = logits.dtype if out_dtype is None else out_dtype
-        R = T * k
-        key = (T, E, k)
-        ws_bytes = _ROUTE_WS_BYTES.get(key)
-        if ws_bytes is None:
-            ws_bytes = _ROUTE_WS_BYTES[key] = int(_lib.lib().mfl_route_sort_workspace(T, E, k))
-        # 256-byte aligned pieces of one block: idx int64, w32 fp32, sort_idx / inv / m_sizes int32, weights, scratch
-        o_w32 = _round256(R * 8)
-        o_sort = o_w32 + _round256(R * 4)
-        o_inv = o_sort + _round256(R * 4)
-        o_ms = o_inv + _round256(R * 4)
-        o_wc = o_ms + _round256(E * 4)
-        o_ws = o_wc + _round256(R * out_dtype.itemsize)
-        buf = torch.empty(o_ws + ws_bytes, device=logits.device, dtype=torch.uint8)
-        idx = buf[:R * 8].view(torch.int64).view(T, k)
-        w32 = buf[o_w32:o_w32 + R * 4].view(torch.float32).view(T, k)
-        sort_idx = buf[o_sort:o_sort + R * 4].view(torch.int32)
-        inv = buf[o_inv:o_inv + R * 4].view(torch.int32)
-        m_sizes = buf[o_ms:o_ms + E * 4].view(torch.int32)
-        wc = buf[o_wc:o_wc + R * out_dtype.itemsize].view(out_dtype).view(T, k)
-        base = buf.data_ptr()
-        rc = _lib.lib().mfl_route_sort(_lib.ptr(logits), _lib.dtype_code(logits.dtype), T, E, k, int(bool(renorm)),
-                                       base + o_w32, base + o_wc, _lib.dtype_code(out_dtype), base, base + o_ms,
-                                       base + o_sort, base + o_inv, base + o_ws, ws_bytes, _lib.stream())
-        _lib.check(rc, "mfl_route_sort")
+        assert logits.shape[1] == num_experts
+        w32, wc, idx, m_sizes, sort_idx, inv = _route_and_sort_raw(logits, k, renorm, out_dtype)
         ctx.save_for_backward(logits, idx, w32)
         ctx.renorm = renorm
         ctx.mark_non_differentiable(idx, m_sizes, sort_idx, inv)
@@ -121,6 +129,11 @@ def route_and_sort(logits: torch.Tensor, k: int, renorm: bool, out_dtype: Option
     """(routing_weights (T,k) in ``out_dtype``, selected_experts (T,k) int64, m_sizes, sort_idx,
     inv_sort_idx): ``softmax_topk`` followed by ``get_expert_counts_and_idx`` on its selections
     (modular_qwen3_moe_fused.py:87-93,102)."""
+    if not (torch.is_grad_enabled() and logits.requires_grad):
+        # nothing to differentiate (inference, frozen router): skip the autograd function, whose bookkeeping
+        # costs as much host time as the call itself
+        assert logits.shape[1] == num_experts
+        return _route_and_sort_raw(logits, k, renorm, out_dtype)[1:]
     return _RouteAndSort.apply(logits, k, renorm, out_dtype, num_experts)
 
 
