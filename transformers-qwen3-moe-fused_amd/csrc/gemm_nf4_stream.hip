@@ -215,16 +215,27 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     for (int q = 0; q < NS; ++q) {
         wait_vmcnt<(RING - 2) * S::kOps>();
         __syncthreads();  // stage q is whole (the first time round: so is the pair table); nobody reads stage q - 1 any more
-        issue(q + RING - 1 < NS ? q + RING - 1 : NS - 1);
         const unsigned char *const base = smem + (q % RING) * S::kStage;
+        // the stage's packed weights and scales are asked of the LDS before the next copies are set up (some
+        // forty scalar and vector instructions), so that their latency runs under that
+        uint4_t wl2[2][CB];
+        float am2[2][CB];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                wl2[s2][cb] = *(const uint4_t *)(base + S::kX + (wave * CB + cb) * S::kW + w_rd[s2]);
+                am2[s2][cb] = *(const float *)(base + S::kX + 4 * CB * S::kW + (wave * CB + cb) * S::kA + (n * 2 + s2) * 4);
+            }
+        issue(q + RING - 1 < NS ? q + RING - 1 : NS - 1);
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
             uint4_t wl[CB];
             float am[CB];
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
-                wl[cb] = *(const uint4_t *)(base + S::kX + (wave * CB + cb) * S::kW + w_rd[s2]);
-                am[cb] = *(const float *)(base + S::kX + 4 * CB * S::kW + (wave * CB + cb) * S::kA + (n * 2 + s2) * 4);
+                wl[cb] = wl2[s2][cb];
+                am[cb] = am2[s2][cb];
             }
             floatx16 blk[CB];
 #pragma unroll
