@@ -156,3 +156,24 @@ def test_nf4_input_gradient_falls_back_for_odd_widths():
     ms = m_sizes_uniform(R, E, g)
     dx = grouped_gemm_forward_transposed_4bit(dy.to(DEV), packed, state, ms.to(DEV))
     check_close(dx, oracle.linear_bwd_input(to_np32(dy), w_deq, oracle.sel_from_m_sizes(ms.numpy())), what="fallback")
+
+
+@pytest.mark.parametrize("R,N,K,E,blocksize,dtype", [(120, 24, 20, 3, 4, torch.bfloat16),     # K % 8 != 0, blocks under 8 weights
+                                                     (90, 40, 64, 5, 64, torch.float32),      # fp32 rows
+                                                     (64, 16, 36, 2, 2, torch.float16)])      # fp16 rows, K % 8 != 0
+def test_nf4_forward_falls_back_for_inputs_without_a_fused_kernel(R, N, K, E, blocksize, dtype):
+    # the reference's wrapper takes these (forward_4bit.py:107-160); here the wrapper dequantises and multiplies
+    w = randn((E, N, K), gen(R), 0.1)
+    q, absmax = oracle.nf4_quant(w.numpy(), blocksize)
+    w_deq = oracle.nf4_dequant(q, absmax, blocksize).reshape(E, N, K)
+    if dtype != torch.float32:
+        w_deq = to_np32(torch.from_numpy(w_deq).to(dtype))
+    state = Nf4QuantState(absmax=torch.from_numpy(absmax).to(DEV), shape=(E, N, K), code=nf4_code(DEV),
+                          blocksize=blocksize, dtype=dtype)
+    g = gen(R + 1)
+    x = randn((R, K), g, 1.0, dtype)
+    ms = m_sizes_uniform(R, E, g)
+    y = grouped_gemm_forward_4bit(x.to(DEV), torch.from_numpy(q).view(-1, 1).to(DEV), state, ms.to(DEV))
+    assert y.dtype == dtype
+    tol = 1e-4 if dtype == torch.float32 else 1e-2
+    check_close(y, oracle.linear_fwd(to_np32(x), w_deq, oracle.sel_from_m_sizes(ms.numpy())), tol, tol, "fallback forward")
