@@ -72,7 +72,8 @@ def test_gathered_forward_matches_oracle_and_explicit_gather(T, E, k, N, K):
 
 @pytest.mark.parametrize("T,E,k,N,K,blocksize", [(512, 16, 4, 192, 256, 64), (40, 20, 2, 136, 128, 16),
                                                  (1024, 4, 2, 264, 192, 32), (16, 128, 8, 768, 2048, 64),
-                                                 (24, 6, 2, 136, 384, 128)])   # streaming kernel, ragged edges
+                                                 (24, 6, 2, 136, 384, 128),    # streaming kernel, ragged edges
+                                                 (9, 12, 2, 48, 1280, 128)])   # matrix-vector kernel, lanes past K
 def test_gathered_nf4_forward(T, E, k, N, K, blocksize):
     ms, sort_idx, sel = _routing(T, E, k, T + N)
     x = randn((T, K), gen(T), 1.0, torch.bfloat16)
@@ -117,7 +118,9 @@ def test_glu_forward(T, E, k, N, K, gathered):
 @pytest.mark.parametrize("T,E,k,N,K,bs_g,bs_u", [(512, 16, 4, 192, 256, 64, 64), (40, 20, 2, 136, 128, 16, 32),
                                                  (1024, 4, 2, 264, 192, 32, 8), (16, 128, 8, 768, 2048, 64, 64),
                                                  (256, 128, 8, 768, 2048, 64, 64),
-                                                 (24, 6, 2, 136, 384, 64, 128)])   # streaming kernel, ragged edges
+                                                 (24, 6, 2, 136, 384, 64, 128),    # streaming kernel, ragged edges
+                                                 (9, 12, 2, 48, 1280, 128, 256),   # matrix-vector kernel
+                                                 (3, 5, 3, 16, 2048, 2048, 8)])
 def test_glu_nf4_forward(T, E, k, N, K, bs_g, bs_u):
     ms, sort_idx, sel = _routing(T, E, k, T + N + 2)
     x = randn((T, K), gen(T), 1.0, torch.bfloat16)
@@ -144,11 +147,12 @@ def test_glu_nf4_forward(T, E, k, N, K, bs_g, bs_u):
     assert torch.equal(h, h3)
 
 
-def test_decode_size_nf4_product_is_as_accurate_as_the_reference_rounding():
-    # The decode-size kernel computes sum over blocks of absmax * (x . bf16(code)), the reference x . bf16(code * absmax).
+@pytest.mark.parametrize("T", [256, 16])   # the streaming kernel; the matrix-vector kernel
+def test_decode_size_nf4_product_is_as_accurate_as_the_reference_rounding(T):
+    # The decode-size kernels compute sum over blocks of absmax * (x . bf16(code)), the reference x . bf16(code * absmax).
     # Against the product with the unrounded weights code * absmax, in float64, neither is better: same rms
     # error, same largest error, within the scatter of such figures.
-    T, E, k, N, K, blocksize = 256, 128, 8, 768, 2048, 64
+    E, k, N, K, blocksize = 128, 8, 768, 2048, 64
     ms, sort_idx, sel = _routing(T, E, k, 11)
     x = randn((T, K), gen(3), 1.0, torch.bfloat16)
     w = randn((E, N, K), gen(4), 0.05)

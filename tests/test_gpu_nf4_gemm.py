@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import oracle
-from util import check_close, gen, m_sizes_uniform, randn, to_np32
+from util import check_close, gen, m_sizes_uniform, randn, to_np32, unit_scale_atol
 
 pytestmark = pytest.mark.gpu
 
@@ -117,6 +117,52 @@ def test_streaming_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, out_d
     # through the wrapper, and again: the same bits
     y2 = grouped_gemm_forward_4bit(xd, packed, state, msd, out_dtype)
     assert torch.equal(y2[:R - 3], y[:R - 3])
+
+
+# The matrix-vector kernel (at most two rows per expert on average, 1024 < K <= 2048, K a multiple of the block
+# size, N a multiple of 16): lanes past the end of a row (K not a multiple of 512), experts of one to five rows
+# (up to three row groups), empty experts, more than 64 experts, more units than workgroups and fewer, one
+# block per row, 64-bit counts, fp32 output, rows past sum(m_sizes).
+@pytest.mark.parametrize("m_sizes,N,K,blocksize,ms_dtype,out_dtype", [
+    ([1, 0, 2, 1], 16, 2048, 64, torch.int32, torch.bfloat16),
+    ([5, 0, 0, 0, 1, 0, 0, 0], 48, 1280, 128, torch.int64, torch.bfloat16),
+    ([0] * 70 + [2] * 3 + [1] * 57, 32, 2048, 2048, torch.int32, torch.float32),
+    ([2, 1, 0, 1, 0, 0], 304, 1536, 512, torch.int32, torch.bfloat16),
+    ([1, 2, 0, 1, 3, 0, 0, 1], 768, 2048, 64, torch.int64, torch.bfloat16),
+    ([1, 1], 16, 1088, 64, torch.int32, torch.bfloat16),
+    ([0, 0, 0, 4], 64, 1032, 8, torch.int32, torch.float32),
+])
+def test_matrix_vector_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, out_dtype):
+    E = len(m_sizes)
+    ms = torch.tensor(m_sizes, dtype=ms_dtype)
+    pad = min(3, 2 * E - int(ms.sum()))        # rows past the last expert: not written
+    R = int(ms.sum()) + pad
+    assert R <= 2 * E and 1024 < K <= 2048 and K % blocksize == 0 and N % 16 == 0
+    packed, state, w_deq = _quantised(E, N, K, blocksize, N + K)
+    x = randn((R, K), gen(K), 1.0, torch.bfloat16)
+    sel = oracle.sel_from_m_sizes(np.asarray(m_sizes))
+    y = torch.full((R, N), 7.0, device=DEV, dtype=out_dtype)
+    from qwen3_moe_fused import _lib
+    xd, msd = x.to(DEV), ms.to(DEV)
+    rc = _lib.lib().mfl_gemm_fwd_nf4(_lib.ptr(xd), _lib.ptr(packed), _lib.ptr(state.code), _lib.ptr(state.absmax), blocksize,
+                                     _lib.ptr(msd), _lib.itype_code(ms_dtype), _lib.ptr(y), R, N, K, E,
+                                     _lib.dtype_code(torch.bfloat16), _lib.dtype_code(out_dtype), _lib.stream())
+    _lib.check(rc, "mfl_gemm_fwd_nf4")
+    ref = oracle.linear_fwd(to_np32(x)[:R - pad], w_deq, sel)
+    check_close(y[:R - pad], ref, atol=unit_scale_atol(ref),
+                what=f"matrix-vector kernel m_sizes={m_sizes} N={N} K={K} blocksize={blocksize}")
+    assert torch.all(y[R - pad:] == 7.0), "rows past sum(m_sizes) stay as they were"
+    y2 = grouped_gemm_forward_4bit(xd, packed, state, msd, out_dtype)
+    assert torch.equal(y2[:R - pad], y[:R - pad])
+    # counts that run past the rows given: the rows that exist are computed, nothing past them is touched
+    R_short = int(ms.sum()) - 1
+    if R_short >= 1:
+        y3 = torch.full((R_short + 1, N), 7.0, device=DEV, dtype=out_dtype)
+        rc = _lib.lib().mfl_gemm_fwd_nf4(_lib.ptr(xd), _lib.ptr(packed), _lib.ptr(state.code), _lib.ptr(state.absmax),
+                                         blocksize, _lib.ptr(msd), _lib.itype_code(ms_dtype), _lib.ptr(y3), R_short, N, K,
+                                         E, _lib.dtype_code(torch.bfloat16), _lib.dtype_code(out_dtype), _lib.stream())
+        _lib.check(rc, "mfl_gemm_fwd_nf4")
+        assert torch.equal(y3[:R_short], y[:R_short]) and torch.all(y3[R_short] == 7.0)
 
 
 from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit  # noqa: E402

@@ -52,6 +52,13 @@ int gemm_nf4_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const 
                     bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
                     int K, int E, int out_dtype, hipStream_t stream);
 
+// The matrix-vector form of gemm_nf4_decode for at most two rows per expert on average (R <= 2 E): lanes along
+// the reduction, rows in registers, no MFMA.  K <= 2048, K a multiple of the quantisation block size;
+// MFL_ERR_UNSUPPORTED otherwise.
+int gemm_nf4_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
+                  bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
+                  int K, int E, int out_dtype, hipStream_t stream);
+
 // Forward with NF4 weights for decode-sized batches (at most 32 rows per expert on average):
 // weights decoded in registers, no LDS stage.
 int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,

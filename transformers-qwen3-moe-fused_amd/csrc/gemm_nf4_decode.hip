@@ -320,6 +320,11 @@ int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const
     if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
     const bf16_t *px = (const bf16_t *)x;
     {
+        const int rc = gemm_nf4_gemv(px, row_idx, idx_div, w0, w1, glu, m_sizes, ms_i64, y, e_out, g_out, R, N, K, E,
+                                     out_dtype, stream);
+        if (rc != MFL_ERR_UNSUPPORTED) return rc;
+    }
+    {
         const int rc = gemm_nf4_stream(px, row_idx, idx_div, w0, w1, glu, m_sizes, ms_i64, y, e_out, g_out, R, N, K, E,
                                        out_dtype, stream);
         if (rc != MFL_ERR_UNSUPPORTED) return rc;

@@ -1,0 +1,408 @@
+// Fused NF4 grouped product for batches of a few rows per expert (1024 < K <= 2048): a matrix-vector form.
+//
+// With one or two rows per expert there is nothing for a matrix core to share: a 32-row MFMA tile would
+// be 3 to 6 % full, and what the launch has to do is pull every routed expert's packed weights through
+// the chip once.  So no tile and no LDS stage:
+//   * a wave owns one output column at a time.  Its 64 lanes lie along the reduction: load i of a column
+//     gives lane l the dword of 8 packed weights k = (64 i + l) * 8 .., i.e. a wave reads 256 consecutive
+//     bytes per load and a column of K = 2048 in four.  The scale of those 8 weights is one float (blocks
+//     of at least 8 weights, K a multiple of the block size).
+//   * the rows of the group (up to two of one expert) stay in registers for all columns of the group: 16
+//     bytes per lane, load and row.
+//   * a byte of packed weights is two weights and one dword of bf16 pairs: a 256-entry table in LDS holds
+//     the finished pair, and v_dot2_f32_bf16 multiplies it with the row's pair.  An entry is 256 bytes: 32
+//     copies for the first matrix, 32 for the second of the gated form; lane l reads copy l & 31, so the 64
+//     lookups of a wave meet no bank conflict, and the address 256 * byte + 4 * copy is ONE byte permute.
+//     One vector instruction per byte for the address, one per byte and row for the product; the scale goes
+//     onto the partial sum of the 8 weights in fp32.
+//   * the 64 partial sums of a column meet in six data-parallel-primitive adds; lane 63 stores.
+//   * one workgroup of 16 waves per CU, as many workgroups as CUs, and the (row group, 16 columns) units of
+//     the launch dealt out in equal contiguous shares: no second round of workgroups, and a workgroup
+//     changes rows once or twice.  Each wave keeps the loads of four columns ahead in registers.
+//   What the loop is short of, with 16 waves to a CU, is issue slots, scalar ones first: addresses move by
+//   increments, the row count is branched on once per column, and the lookups of a dword wait once.
+//
+// The product is sum over 8-weight pieces of absmax * (x . bf16(code)), as in the streaming form.
+#include <mutex>
+#include <type_traits>
+
+#include "common.h"
+#include "gemm.h"
+
+namespace mfl {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((address_space(3))) void *lds_void_ptr;
+typedef const __attribute__((address_space(3))) uint32_t *lds_u32_ptr;
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_fadd_step(float x) {
+    // lanes without a source, and rows that the mask leaves out, add 0
+    const int y = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xf, true);
+    return x + __builtin_bit_cast(float, y);
+}
+// sum over the 64 lanes of a wave, valid in lane 63
+__device__ __forceinline__ float wave_sum_to_last(float x) {
+    x = dpp_fadd_step<0x111, 0xf>(x);  // row_shr 1
+    x = dpp_fadd_step<0x112, 0xf>(x);  // row_shr 2
+    x = dpp_fadd_step<0x114, 0xf>(x);  // row_shr 4
+    x = dpp_fadd_step<0x118, 0xf>(x);  // row_shr 8
+    x = dpp_fadd_step<0x142, 0xa>(x);  // row_bcast 15 into rows 1 and 3
+    x = dpp_fadd_step<0x143, 0xc>(x);  // row_bcast 31 into rows 2 and 3
+    return x;
+}
+
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+}
+
+// Four table reads and one wait for all of them, written out: the compiler would wait before each use, and with
+// 16 waves to a CU the issue slots of those waits are not free.  The addresses count from LDS address 0.
+__device__ __forceinline__ void lookup4(uint32_t (&pr)[4], uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3) {
+    asm volatile(
+        "ds_read_b32 %0, %4\n\tds_read_b32 %1, %5\n\tds_read_b32 %2, %6\n\tds_read_b32 %3, %7\n\ts_waitcnt lgkmcnt(0)"
+        : "=&v"(pr[0]), "=&v"(pr[1]), "=&v"(pr[2]), "=&v"(pr[3])
+        : "v"(a0), "v"(a1), "v"(a2), "v"(a3));
+}
+
+constexpr int kGemvThreads = 1024;
+constexpr int kGemvTable = 65536;
+
+
+// The LDS address of the pair of packed byte `B` of w: 256 * byte + lane_copy (the lane's copy of the table, one
+// byte), put together by one byte permute.
+template <int B>
+__device__ __forceinline__ uint32_t pair_address(uint32_t w, uint32_t lane_copy) {
+    // byte 0 of the result: byte 0 of lane_copy; byte 1: byte B of w; bytes 2 and 3: zero
+    return __builtin_amdgcn_perm(w, lane_copy, 0x0c0c0000u | ((4u + B) << 8));
+}
+
+// NL: loads per column (K <= 512 NL); ROWS: rows per group; D: columns whose loads a wave keeps in flight
+template <int NL, int ROWS, int D, bool GLU, typename TO>
+__global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__restrict__ x,
+                                                                const int32_t *__restrict__ row_idx, int idx_div,
+                                                                Nf4Matrix w0, Nf4Matrix w1,
+                                                                const void *__restrict__ m_sizes, int ms_i64,
+                                                                TO *__restrict__ y, TO *__restrict__ e_out,
+                                                                TO *__restrict__ g_out, int64_t R, int N, int K,
+                                                                int E, int units_n, int max_groups) {
+    constexpr int CB = GLU ? 2 : 1;
+    static_assert(D % CB == 0, "the matrix of a ring slot is fixed");
+    extern __shared__ __attribute__((aligned(256))) unsigned char smem[];
+    unsigned char *const table = smem;                      // kGemvTable bytes
+    int *const grp_e = (int *)(smem + kGemvTable);          // expert | rows << 16
+    int *const grp_r = grp_e + max_groups;                  // first row
+    int *const n_groups_s = grp_r + max_groups;
+    int *const ms_s = n_groups_s + 1;                       // the E counts
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // the lookups address the table from LDS address 0 (the kernel has no static LDS in front of the dynamic)
+    if ((uint32_t)(uintptr_t)(lds_void_ptr)smem != 0) __builtin_trap();
+    // the counts, asked for first: their latency runs under the filling of the table
+    int ms_own[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int e = tid + j * kGemvThreads;
+        ms_own[j] = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
+    }
+    // ---- pair table: entry b = bf16(code[b >> 4]) in the low half (the first of the two weights is the high
+    // nibble), bf16(code[b & 15]) in the high half.  Entry b is the 256 bytes at 256 b: 32 copies for the first
+    // matrix, 32 for the second; thread t writes 64 of the bytes of entry t & 255.
+    {
+        const int b = tid & 255, part = tid >> 8;
+        if (part < 2 * CB) {
+            const float *const code = part < 2 ? w0.code16 : w1.code16;
+            union {
+                bf16_t e[2];
+                uint32_t u;
+            } pr;
+            pr.e[0] = (bf16_t)code[b >> 4];
+            pr.e[1] = (bf16_t)code[b & 15];
+            const uint4_t v = {pr.u, pr.u, pr.u, pr.u};
+            uint4_t *const dst = (uint4_t *)(table + b * 256 + part * 64);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) dst[j] = v;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int e = tid + j * kGemvThreads;
+        if (e < E) ms_s[e] = ms_own[j];
+    }
+    __syncthreads();
+    // ---- row groups in the order of the experts: group g = rows grp_r[g] .. of expert grp_e[g] & 0xffff
+    if (wave == 0) {
+        int row_carry = 0, grp_carry = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            int m = e < E ? ms_s[e] : 0;
+            if (m < 0) m = 0;
+            const int minc = wave_inclusive_scan(m);
+            const int64_t start = (int64_t)row_carry + minc - m;
+            if (start + m > R) m = start < R ? (int)(R - start) : 0;  // counts that run past the rows given
+            const int g = ceil_div(m, ROWS);
+            const int ginc = wave_inclusive_scan(g);
+            const int gb = grp_carry + ginc - g;
+            for (int q = 0; q < g && gb + q < max_groups; ++q) {
+                const int rows = m - q * ROWS < ROWS ? m - q * ROWS : ROWS;
+                grp_e[gb + q] = e | (rows << 16);
+                grp_r[gb + q] = (int)start + q * ROWS;
+            }
+            row_carry += wave_last(minc);
+            grp_carry += wave_last(ginc);
+        }
+        if (lane == 0) *n_groups_s = grp_carry < max_groups ? grp_carry : max_groups;
+    }
+    __syncthreads();
+
+    // ---- this workgroup's share of the units (row group, 16 columns), row group major
+    // (equal shares, the first U % gridDim.x workgroups one unit more; the host keeps U below 2^31)
+    const uint32_t U = (uint32_t)*n_groups_s * (uint32_t)units_n;
+    const uint32_t share = U / gridDim.x, extra = U % gridDim.x;
+    const uint32_t u_begin = blockIdx.x * share + (blockIdx.x < extra ? blockIdx.x : extra);
+    const uint32_t u_end = u_begin + share + (blockIdx.x < extra ? 1 : 0);
+    if (u_begin >= u_end) return;
+    const int n_items = (int)(u_end - u_begin) * CB;  // (unit, matrix) pairs, matrix minor
+
+    // ---- what a lane reads of a column: dword (64 i + lane) of its packed row, if that is inside the row
+    uint32_t w_idx[NL], a_off[CB][NL], x_off[NL];
+    bool inside[NL];
+    const Nf4Matrix mat[2] = {w0, w1};
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int k = (i * 64 + lane) * 8;
+        inside[i] = k < K;
+        const int kc = inside[i] ? k : 0;
+        w_idx[i] = (uint32_t)kc >> 3;
+        x_off[i] = kc;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) a_off[cb][i] = (uint32_t)kc >> mat[cb].bs_shift;
+    }
+    const uint32_t copy_off = (lane & 31) * 4;  // + 128 for the second matrix
+
+    // ---- the ring of columns ahead
+    uint32_t ring_w[D][NL];
+    float ring_a[D][NL];
+    // Cursor of the loads: the wave's column of unit ic of group ig.  The pointers move on by 16 columns per unit
+    // (N % 16 == 0: every unit is whole) and are set up afresh when the group changes: a handful of scalar
+    // instructions per column instead of the 64-bit products, which with 16 waves to a CU are what the scalar
+    // unit has no time for.
+    const int ig0 = (int)(u_begin / (uint32_t)units_n), ic0 = (int)(u_begin % (uint32_t)units_n);
+    int ig = ig0, ic = ic0;
+    int i_units_left = (int)(u_end - u_begin);
+    const uint32_t *i_wp[CB];
+    const float *i_ap[CB];
+    auto point_loads = [&]() {
+        const int expert = __builtin_amdgcn_readfirstlane(grp_e[ig]) & 0xffff;
+        const int64_t base = ((int64_t)expert * N + ic * 16 + wave) * K;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            i_wp[cb] = (const uint32_t *)(mat[cb].wq + (base >> 1));
+            i_ap[cb] = mat[cb].absmax + (base >> mat[cb].bs_shift);
+        }
+    };
+    point_loads();
+    const int w_step = 2 * K;  // dwords of 16 columns
+    int a_step[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) a_step[cb] = (16 * K) >> mat[cb].bs_shift;
+    auto issue = [&](int d) {
+        const int cb = d % CB;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            ring_w[d][i] = i_wp[cb][w_idx[i]];
+            ring_a[d][i] = i_ap[cb][a_off[cb][i]];
+        }
+        // past the end the cursor stays on the last unit: loads that nobody uses
+        if (cb == CB - 1 && i_units_left > 1) {
+            --i_units_left;
+            if (++ic == units_n) {
+                ic = 0;
+                ++ig;
+                point_loads();
+            } else {
+#pragma unroll
+                for (int c2 = 0; c2 < CB; ++c2) {
+                    i_wp[c2] += w_step;
+                    i_ap[c2] += a_step[c2];
+                }
+            }
+        }
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) issue(d);
+
+    // ---- the loop over the columns
+    uint4_t xr[ROWS][NL];
+    int cg = ig0, cc = ic0;  // cursor of the arithmetic
+    int rows = 0, row0 = 0, o_col = cc * 16;
+    int64_t o_row[ROWS];  // where the wave's column of unit 0 is in the output, per row of the group
+    bool fresh = true;
+    float first[ROWS];  // the gate projection's sums, until the up projection's are there
+    // One column: the arithmetic on ring slot d, then (in the loop) the loads of the column D further on into it.
+    auto column = [&](const int d, const bool more) {
+            const int cb = d % CB;
+            if (fresh) {
+                fresh = false;
+                const int ge = __builtin_amdgcn_readfirstlane(grp_e[cg]);
+                rows = ge >> 16;
+                row0 = __builtin_amdgcn_readfirstlane(grp_r[cg]);
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    o_row[r] = (int64_t)(row0 + r) * N + wave;
+                    int64_t src_row = row0 + (r < rows ? r : rows - 1);
+                    if (row_idx != nullptr) src_row = (uint32_t)row_idx[src_row] / (uint32_t)idx_div;
+                    const bf16_t *const xp = x + src_row * K;
+#pragma unroll
+                    for (int i = 0; i < NL; ++i) {
+                        const uint4_t v = *(const uint4_t *)(xp + x_off[i]);
+                        const uint4_t zero = {0, 0, 0, 0};
+                        xr[r][i] = inside[i] ? v : zero;
+                    }
+                }
+            }
+            const uint32_t lane_copy = copy_off + cb * 128;
+            // The slot's values move to registers of the column and the slot is asked for again right away, in one
+            // place for all row counts: were the loads issued inside the branches below, the branches would load
+            // into different registers, and the copy that reconciles them would wait for the load just issued.
+            uint32_t wv[NL];
+            float av[NL];
+#pragma unroll
+            for (int i = 0; i < NL; ++i) {
+                wv[i] = ring_w[d][i];
+                av[i] = ring_a[d][i];
+            }
+            if (more) issue(d);
+            // the arithmetic of the column for RN rows: one branch on the number of rows per column, none inside
+            auto arithmetic = [&](auto RN) {
+                constexpr int rn = decltype(RN)::value;
+                float acc[rn];
+#pragma unroll
+                for (int r = 0; r < rn; ++r) acc[r] = 0.f;
+#pragma unroll
+                for (int i = 0; i < NL; ++i) {
+                    uint32_t pr[4];
+                    lookup4(pr, pair_address<0>(wv[i], lane_copy), pair_address<1>(wv[i], lane_copy),
+                            pair_address<2>(wv[i], lane_copy), pair_address<3>(wv[i], lane_copy));
+#pragma unroll
+                    for (int r = 0; r < rn; ++r) {
+                        float s = dot2_bf16(pr[0], xr[r][i][0], 0.f);
+                        s = dot2_bf16(pr[1], xr[r][i][1], s);
+                        s = dot2_bf16(pr[2], xr[r][i][2], s);
+                        s = dot2_bf16(pr[3], xr[r][i][3], s);
+                        acc[r] = __builtin_fmaf(av[i], s, acc[r]);
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < rn; ++r) acc[r] = wave_sum_to_last(acc[r]);
+                if (GLU && cb == 0) {
+#pragma unroll
+                    for (int r = 0; r < rn; ++r) first[r] = acc[r];
+                    return;
+                }
+                if (lane == 63) {
+#pragma unroll
+                    for (int r = 0; r < rn; ++r) {
+                        const int64_t o = o_row[r] + o_col;
+                        if constexpr (GLU) {
+                            const bf16_t pe = (bf16_t)first[r], pg = (bf16_t)acc[r];
+                            ((bf16_t *)y)[o] = silu_fwd_one<bf16_t>(pe, pg);
+                            if (e_out) ((bf16_t *)e_out)[o] = pe;
+                            if (g_out) ((bf16_t *)g_out)[o] = pg;
+                        } else {
+                            y[o] = from_f32<TO>(acc[r]);
+                        }
+                    }
+                }
+            };
+            if (rows == 1)
+                arithmetic(std::integral_constant<int, 1>());
+            else if (ROWS == 2 || rows == 2)
+                arithmetic(std::integral_constant<int, 2>());
+            else if (ROWS == 4 && rows == 3)
+                arithmetic(std::integral_constant<int, (ROWS > 2 ? 3 : 1)>());
+            else
+                arithmetic(std::integral_constant<int, ROWS>());
+            if (cb == CB - 1) {
+                o_col += 16;
+                if (++cc == units_n) {
+                    cc = 0;
+                    o_col = 0;
+                    ++cg;
+                    fresh = true;
+                }
+            }
+    };
+    // Whole rounds of the ring in a loop without a way out of its middle, the rest behind it: with an exit
+    // between two columns the compiler sees a path from a column's loads straight to the head of the loop,
+    // where they would be the youngest in flight, and waits for every load at every column.
+    const int rounds = n_items / D, rest = n_items % D;
+    for (int q = 0; q < rounds; ++q) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) column(d, true);
+    }
+#pragma unroll
+    for (int d = 0; d < D - 1; ++d)
+        if (d < rest) column(d, false);
+}
+
+template <int NL, int ROWS, int D, bool GLU, typename TO>
+int launch_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
+                const void *m_sizes, int ms_i64, TO *y, TO *e_out, TO *g_out, int64_t R, int N, int K, int E,
+                hipStream_t stream) {
+    const int64_t max_groups = R / ROWS + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / ROWS)
+    const int lds = kGemvTable + (int)max_groups * 8 + 16 + E * 4;
+    auto *kernel = nf4_gemv_kernel<NL, ROWS, D, GLU, TO>;
+    static PerDeviceOnce attr;
+    const hipError_t e = attr.run([&] {
+        return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kGemvTable + 4096 * 8 + 16 + 2048 * 4);
+    });
+    if (e != hipSuccess) return (int)e;
+    kernel<<<(unsigned)device_info().cu_count, kGemvThreads, lds, stream>>>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64,
+                                                                            y, e_out, g_out, R, N, K, E,
+                                                                            ceil_div(N, 16), (int)max_groups);
+    return launch_status();
+}
+
+template <int NL, int ROWS, int D>
+int dispatch_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
+                  bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
+                  int K, int E, int out_dtype, hipStream_t stream) {
+    if (glu)
+        return launch_gemv<NL, ROWS, D, true, bf16_t>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (bf16_t *)y,
+                                                   (bf16_t *)e_out, (bf16_t *)g_out, R, N, K, E, stream);
+    if (out_dtype == MFL_BF16)
+        return launch_gemv<NL, ROWS, D, false, bf16_t>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (bf16_t *)y, nullptr,
+                                                    nullptr, R, N, K, E, stream);
+    return launch_gemv<NL, ROWS, D, false, float>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (float *)y, nullptr,
+                                               nullptr, R, N, K, E, stream);
+}
+
+}  // namespace
+
+int gemm_nf4_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
+                  bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
+                  int K, int E, int out_dtype, hipStream_t stream) {
+    if (R <= 0 || R > 2 * (int64_t)E || E > 2048) return MFL_ERR_UNSUPPORTED;  // a few rows per expert only
+    // whole units of 16 columns; fewer than 2^31 units in all
+    if (K % 8 != 0 || K > 2048 || N % 16 != 0 || N > (1 << 18)) return MFL_ERR_UNSUPPORTED;
+    const Nf4Matrix *mats[2] = {&w0, &w1};
+    for (int cb = 0; cb < (glu ? 2 : 1); ++cb) {
+        const Nf4Matrix &m = *mats[cb];
+        // a lane's 8 weights under one scale, and every column starts a quantisation block
+        if (m.bs_shift < 3 || (K & ((1 << m.bs_shift) - 1)) != 0) return MFL_ERR_UNSUPPORTED;
+        if (!aligned(m.absmax, 4) || !aligned(m.wq, 4)) return MFL_ERR_UNSUPPORTED;
+    }
+    if (!aligned(x, 16)) return MFL_ERR_UNSUPPORTED;
+    // Rows of more than 1024 elements only: with shorter ones the work per column (addresses, the sum over the
+    // lanes, the store) outweighs the column's 64 to 512 bytes, and the streaming form is faster (measured at
+    // K = 768: 43 against 27 us at 16 tokens of 8 experts each).
+    if (K <= 1024) return MFL_ERR_UNSUPPORTED;
+    return dispatch_gemv<4, 2, 4>(x, row_idx, idx_div, w0, w1, glu, m_sizes, ms_i64, y, e_out, g_out, R, N, K, E,
+                                  out_dtype, stream);
+}
+
+}  // namespace mfl
