@@ -19,7 +19,7 @@
 // Decoding costs about one vector instruction per weight instead of three and a half:
 //   * a byte of packed weights is two weights, and two bf16 are one dword of an MFMA operand: a 256-entry
 //     table in LDS, indexed by the byte, holds the finished pair.  One shift-by-two of a byte (SDWA) and one
-//     LDS read per pair.  (A copy of the table per bank, 64 KiB, takes the bank conflicts of the lookups
+//     LDS read per pair; the table lies at LDS address 0, so the shifted byte is the address.  (A copy of the table per bank, 64 KiB, takes the bank conflicts of the lookups
 //     away and the second and third workgroup of the CU with them: slower.)
 //   * the table holds the bare code values (rounded to bf16 once).  The scale of a quantisation block is
 //     applied to the block's partial sum in fp32: with the weights as the SECOND MFMA operand a lane's 16
@@ -36,6 +36,7 @@ namespace mfl {
 namespace {
 
 typedef __attribute__((address_space(3))) void *lds_void_ptr;
+typedef const __attribute__((address_space(3))) uint32_t *lds_u32_ptr;
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -95,7 +96,11 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     using S = StreamShape<GLU>;
     constexpr int CB = S::CB, RING = S::RING;
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    unsigned char *const table = smem + RING * S::kStage;
+    // the pair table first, at LDS address 0 (the kernel has no static LDS): a lookup's address is then the shifted
+    // byte itself plus a constant that fits the instruction's offset field, no add
+    unsigned char *const table = smem;
+    unsigned char *const ring = smem + S::kTable;
+    if ((uint32_t)(uintptr_t)(lds_void_ptr)smem != 0) __builtin_trap();
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
@@ -179,7 +184,7 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     }
     const int NS = K / 128;
     auto issue = [&](int stg) {
-        unsigned char *const base = smem + (stg % RING) * S::kStage;
+        unsigned char *const base = ring + (stg % RING) * S::kStage;
 #pragma unroll
         for (int j = 0; j < 2; ++j) copy16_to_lds(x_src[j] + (int64_t)stg * 128, base + (wave * 2 + j) * 1024);
 #pragma unroll
@@ -215,7 +220,7 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     for (int q = 0; q < NS; ++q) {
         wait_vmcnt<(RING - 2) * S::kOps>();
         __syncthreads();  // stage q is whole (the first time round: so is the pair table); nobody reads stage q - 1 any more
-        const unsigned char *const base = smem + (q % RING) * S::kStage;
+        const unsigned char *const base = ring + (q % RING) * S::kStage;
         // the stage's packed weights and scales are asked of the LDS before the next copies are set up (some
         // forty scalar and vector instructions), so that their latency runs under that
         uint4_t wl2[2][CB];
@@ -228,45 +233,58 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
                 am2[s2][cb] = *(const float *)(base + S::kX + 4 * CB * S::kW + (wave * CB + cb) * S::kA + (n * 2 + s2) * 4);
             }
         issue(q + RING - 1 < NS ? q + RING - 1 : NS - 1);
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
-            uint4_t wl[CB];
-            float am[CB];
+        // The eight MFMA steps of the stage in one sequence, the operands of a step (16 bytes of the rows, four
+        // table lookups per matrix) asked of the LDS one step ahead: asked for right in front of their MFMA, every
+        // step would wait out the LDS latency and the stage would be a chain of eight of them.
+        struct StepOps {
+            uint4_t xa;
+            uint4_t wf[CB];
+        };
+        auto fetch = [&](int step, StepOps &o) {
+            const int s2 = step >> 2, ks = step & 3;
+            o.xa = *(const uint4_t *)(base + x_rd[s2][ks]);
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
-                wl[cb] = wl2[s2][cb];
-                am[cb] = am2[s2][cb];
+                const uint32_t w = wl2[s2][cb][ks];
+                o.wf[cb][0] = *(lds_u32_ptr)(uintptr_t)(byte_times_4<0>(w) + cb * 1024);
+                o.wf[cb][1] = *(lds_u32_ptr)(uintptr_t)(byte_times_4<1>(w) + cb * 1024);
+                o.wf[cb][2] = *(lds_u32_ptr)(uintptr_t)(byte_times_4<2>(w) + cb * 1024);
+                o.wf[cb][3] = *(lds_u32_ptr)(uintptr_t)(byte_times_4<3>(w) + cb * 1024);
             }
-            floatx16 blk[CB];
+        };
+        constexpr int AHEAD = 1;  // two steps ahead: no faster; the gated form would pass the 15 LDS reads that can be in flight
+        StepOps ops[AHEAD + 1];
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
+        for (int a = 0; a < AHEAD; ++a) fetch(a, ops[a]);
+        floatx16 blk[CB];
+#pragma unroll
+        for (int step = 0; step < 8; ++step) {
+            if (step + AHEAD < 8) fetch(step + AHEAD, ops[(step + AHEAD) % (AHEAD + 1)]);
+            const StepOps &o = ops[step % (AHEAD + 1)];
+            const int s2 = step >> 2, ks = step & 3;
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
                 union {
                     uint4_t u;
                     bf16x8 v;
                 } xa, wf;
-                xa.u = *(const uint4_t *)(base + x_rd[s2][ks]);
+                xa.u = o.xa;
+                wf.u = o.wf[cb];
+                if (ks == 0) {
+                    floatx16 zero;
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    const uint32_t w = wl[cb][ks];
-                    const unsigned char *const tb = table + cb * 1024;
-                    wf.u[0] = *(const uint32_t *)(tb + byte_times_4<0>(w));
-                    wf.u[1] = *(const uint32_t *)(tb + byte_times_4<1>(w));
-                    wf.u[2] = *(const uint32_t *)(tb + byte_times_4<2>(w));
-                    wf.u[3] = *(const uint32_t *)(tb + byte_times_4<3>(w));
-                    if (ks == 0) {
-                        floatx16 zero;
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) zero[r] = 0.f;
-                        blk[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa.v, wf.v, zero, 0, 0, 0);
-                    } else {
-                        blk[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa.v, wf.v, blk[cb], 0, 0, 0);
-                    }
+                    for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+                    blk[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa.v, wf.v, zero, 0, 0, 0);
+                } else {
+                    blk[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa.v, wf.v, blk[cb], 0, 0, 0);
                 }
             }
+            if (ks == 3) {
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb)
+                for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) tot[cb][r] = __builtin_fmaf(am[cb], blk[cb][r], tot[cb][r]);
+                    for (int r = 0; r < 16; ++r) tot[cb][r] = __builtin_fmaf(am2[s2][cb], blk[cb][r], tot[cb][r]);
+            }
         }
     }
     wait_vmcnt<0>();  // the repeated copies of the last stage must not land in LDS that another workgroup owns by then
