@@ -122,7 +122,12 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     }
 
     // ---- which 32 rows: row tile blockIdx.x / tiles_n in the order of the experts
-    const int ct = blockIdx.x % tiles_n, rt = blockIdx.x / tiles_n;
+    // Workgroup b runs on XCD b % 8.  Row tiles are dealt to the XCDs round robin, and all column tiles of a row
+    // tile to the same XCD, one after the other: the tile's rows come over the fabric once and are shared in
+    // that XCD's L2 (dealt by workgroup number, every XCD that holds one of the column tiles fetches the rows
+    // for itself), while all XCDs still work on neighbouring experts at any one time.
+    const int xcd_idx = blockIdx.x >> 3;
+    const int ct = xcd_idx % tiles_n, rt = (xcd_idx / tiles_n) * 8 + (blockIdx.x & 7);
     int expert = -1, m_start = 0, m_size = 0, t_begin = 0;
     {
         int row_carry = 0, tile_carry = 0;
@@ -316,7 +321,7 @@ int launch_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf
     constexpr int kLds = S::kLds;
     const int tiles_n = ceil_div(N, 128);
     const int64_t row_tiles = R / 32 + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / 32)
-    const int64_t grid = row_tiles * tiles_n;
+    const int64_t grid = (row_tiles + 7) / 8 * 8 * tiles_n;  // row tiles in eights: one per XCD
     if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
     auto *kernel = nf4_stream_kernel<GLU, TO>;
     static PerDeviceOnce attr;
