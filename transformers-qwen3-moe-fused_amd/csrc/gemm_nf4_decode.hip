@@ -171,6 +171,11 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
         if (XSTAGE) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) *(uint4_t *)(xl + x_wr[u]) = s.xs[u];
+            // lanes read below what other lanes of the wave wrote: say so (no instructions; without it the compiler
+            // may treat the reads as reads of this lane's own writes only)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
