@@ -120,16 +120,16 @@ def test_streaming_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, out_d
 
 
 # The matrix-vector kernel (at most two rows per expert on average, 1024 < K <= 2048, K a multiple of the block
-# size, N a multiple of 16): lanes past the end of a row (K not a multiple of 512), experts of one to five rows
+# size, N a multiple of 32): lanes past the end of a row (K not a multiple of 512), experts of one to five rows
 # (up to three row groups), empty experts, more than 64 experts, more units than workgroups and fewer, one
 # block per row, 64-bit counts, fp32 output, rows past sum(m_sizes).
 @pytest.mark.parametrize("m_sizes,N,K,blocksize,ms_dtype,out_dtype", [
-    ([1, 0, 2, 1], 16, 2048, 64, torch.int32, torch.bfloat16),
-    ([5, 0, 0, 0, 1, 0, 0, 0], 48, 1280, 128, torch.int64, torch.bfloat16),
+    ([1, 0, 2, 1], 32, 2048, 64, torch.int32, torch.bfloat16),
+    ([5, 0, 0, 0, 1, 0, 0, 0], 96, 1280, 128, torch.int64, torch.bfloat16),
     ([0] * 70 + [2] * 3 + [1] * 57, 32, 2048, 2048, torch.int32, torch.float32),
-    ([2, 1, 0, 1, 0, 0], 304, 1536, 512, torch.int32, torch.bfloat16),
+    ([2, 1, 0, 1, 0, 0], 288, 1536, 512, torch.int32, torch.bfloat16),
     ([1, 2, 0, 1, 3, 0, 0, 1], 768, 2048, 64, torch.int64, torch.bfloat16),
-    ([1, 1], 16, 1088, 64, torch.int32, torch.bfloat16),
+    ([1, 1], 32, 1088, 64, torch.int32, torch.bfloat16),
     ([0, 0, 0, 4], 64, 1032, 8, torch.int32, torch.float32),
 ])
 def test_matrix_vector_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, out_dtype):
@@ -137,7 +137,7 @@ def test_matrix_vector_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, o
     ms = torch.tensor(m_sizes, dtype=ms_dtype)
     pad = min(3, 2 * E - int(ms.sum()))        # rows past the last expert: not written
     R = int(ms.sum()) + pad
-    assert R <= 2 * E and 1024 < K <= 2048 and K % blocksize == 0 and N % 16 == 0
+    assert R <= 2 * E and 1024 < K <= 2048 and K % blocksize == 0 and N % 32 == 0
     packed, state, w_deq = _quantised(E, N, K, blocksize, N + K)
     x = randn((R, K), gen(K), 1.0, torch.bfloat16)
     sel = oracle.sel_from_m_sizes(np.asarray(m_sizes))

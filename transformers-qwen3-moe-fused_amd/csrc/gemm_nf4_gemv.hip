@@ -3,9 +3,10 @@
 // With one or two rows per expert there is nothing for a matrix core to share: a 32-row MFMA tile would
 // be 3 to 6 % full, and what the launch has to do is pull every routed expert's packed weights through
 // the chip once.  So no tile and no LDS stage:
-//   * a wave owns one output column at a time.  Its 64 lanes lie along the reduction: load i of a column
-//     gives lane l the dword of 8 packed weights k = (64 i + l) * 8 .., i.e. a wave reads 256 consecutive
-//     bytes per load and a column of K = 2048 in four.  The scale of those 8 weights is one float (blocks
+//   * a wave owns two output columns at a time, 16 apart (one in the gated form, where the second matrix takes
+//     the registers).  Its 64 lanes lie along the reduction: load i of a column gives lane l the dword of 8
+//     packed weights k = (64 i + l) * 8 .., i.e. a wave reads 256 consecutive bytes per load and a column of
+//     K = 2048 in four.  The scale of those 8 weights is one float (blocks
 //     of at least 8 weights, K a multiple of the block size).
 //   * the rows of the group (up to two of one expert) stay in registers for all columns of the group: 16
 //     bytes per lane, load and row.
@@ -15,10 +16,13 @@
 //     lookups of a wave meet no bank conflict, and the address 256 * byte + 4 * copy is ONE byte permute.
 //     One vector instruction per byte for the address, one per byte and row for the product; the scale goes
 //     onto the partial sum of the 8 weights in fp32.
-//   * the 64 partial sums of a column meet in six data-parallel-primitive adds; lane 63 stores.
-//   * one workgroup of 16 waves per CU, as many workgroups as CUs, and the (row group, 16 columns) units of
-//     the launch dealt out in equal contiguous shares: no second round of workgroups, and a workgroup
-//     changes rows once or twice.  Each wave keeps the loads of four columns ahead in registers.
+//   * the 64 partial sums of each of the two columns become 32 + 32 in one swap of half waves
+//     (v_permlane32_swap) and an add, and five data-parallel-primitive adds finish both at once; lanes 31 and
+//     63 store.
+//   * one workgroup of 16 waves per CU, as many workgroups as CUs, and the (row group, 32 columns) units of
+//     the launch (16 columns in the gated form) dealt out in equal contiguous shares: no second round of
+//     workgroups, and a workgroup changes rows once or twice.  Each wave keeps the loads of four columns ahead
+//     in registers.
 //   What the loop is short of, with 16 waves to a CU, is issue slots, scalar ones first: addresses move by
 //   increments, the row count is branched on once per column, and the lookups of a dword wait once.
 //
@@ -43,14 +47,19 @@ __device__ __forceinline__ float dpp_fadd_step(float x) {
     const int y = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xf, true);
     return x + __builtin_bit_cast(float, y);
 }
-// sum over the 64 lanes of a wave, valid in lane 63
-__device__ __forceinline__ float wave_sum_to_last(float x) {
+// a: 64 partial sums of one column, b: of another.  Returns the first column's sum in lane 31 and the second's in
+// lane 63: v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its second, so the
+// sum of the two holds a[l] + a[l + 32] in lanes 0..31 and b[l - 32] + b[l] in lanes 32..63.  (Written out: through
+// __builtin_amdgcn_permlane32_swap, with both results feeding one add, the compiler added the first result to
+// itself.  The no-ops keep the wait states that the swap and the moves after it need from their neighbours.)
+__device__ __forceinline__ float two_sums_to_31_and_63(float a, float b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    float x = a + b;
     x = dpp_fadd_step<0x111, 0xf>(x);  // row_shr 1
     x = dpp_fadd_step<0x112, 0xf>(x);  // row_shr 2
     x = dpp_fadd_step<0x114, 0xf>(x);  // row_shr 4
     x = dpp_fadd_step<0x118, 0xf>(x);  // row_shr 8
     x = dpp_fadd_step<0x142, 0xa>(x);  // row_bcast 15 into rows 1 and 3
-    x = dpp_fadd_step<0x143, 0xc>(x);  // row_bcast 31 into rows 2 and 3
     return x;
 }
 
@@ -80,7 +89,7 @@ __device__ __forceinline__ uint32_t pair_address(uint32_t w, uint32_t lane_copy)
 }
 
 // NL: loads per column (K <= 512 NL); ROWS: rows per group; D: columns whose loads a wave keeps in flight
-template <int NL, int ROWS, int D, bool GLU, typename TO>
+template <int NL, int ROWS, int D, bool GLU, bool EXACT, typename TO>
 __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__restrict__ x,
                                                                 const int32_t *__restrict__ row_idx, int idx_div,
                                                                 Nf4Matrix w0, Nf4Matrix w1,
@@ -89,6 +98,9 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
                                                                 TO *__restrict__ g_out, int64_t R, int N, int K,
                                                                 int E, int units_n, int max_groups) {
     constexpr int CB = GLU ? 2 : 1;
+    // Columns per wave and unit: two, 16 apart, for the plain product (the loop's scalar work and the sum over the
+    // lanes are shared by both); one for the gated form, whose second matrix leaves no registers for a second column.
+    constexpr int COLS = GLU ? 1 : 2;
     static_assert(D % CB == 0, "the matrix of a ring slot is fixed");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem[];
     unsigned char *const table = smem;                      // kGemvTable bytes
@@ -168,24 +180,22 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
     const int n_items = (int)(u_end - u_begin) * CB;  // (unit, matrix) pairs, matrix minor
 
     // ---- what a lane reads of a column: dword (64 i + lane) of its packed row, if that is inside the row
-    uint32_t w_idx[NL], a_off[CB][NL], x_off[NL];
+    // EXACT (K a multiple of 512): load i is inside the row for all lanes or for none, and the lane's offsets are
+    // lane * 8 plus constants; otherwise they are kept per load, clamped to 0 where the lane is past the row.
+    uint32_t x_off[NL];
     bool inside[NL];
     const Nf4Matrix mat[2] = {w0, w1};
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
         const int k = (i * 64 + lane) * 8;
-        inside[i] = k < K;
-        const int kc = inside[i] ? k : 0;
-        w_idx[i] = (uint32_t)kc >> 3;
-        x_off[i] = kc;
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) a_off[cb][i] = (uint32_t)kc >> mat[cb].bs_shift;
+        inside[i] = EXACT ? i * 512 < K : k < K;
+        x_off[i] = EXACT ? (uint32_t)(lane * 8 + (i * 512 < K ? i * 512 : 0)) : (uint32_t)(inside[i] ? k : 0);
     }
     const uint32_t copy_off = (lane & 31) * 4;  // + 128 for the second matrix
 
     // ---- the ring of columns ahead
-    uint32_t ring_w[D][NL];
-    float ring_a[D][NL];
+    uint32_t ring_w[D][COLS][NL];  // a slot: the wave's columns of a unit
+    float ring_a[D][COLS][NL];
     // Cursor of the loads: the wave's column of unit ic of group ig.  The pointers move on by 16 columns per unit
     // (N % 16 == 0: every unit is whole) and are set up afresh when the group changes: a handful of scalar
     // instructions per column instead of the 64-bit products, which with 16 waves to a CU are what the scalar
@@ -197,7 +207,7 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
     const float *i_ap[CB];
     auto point_loads = [&]() {
         const int expert = __builtin_amdgcn_readfirstlane(grp_e[ig]) & 0xffff;
-        const int64_t base = ((int64_t)expert * N + ic * 16 + wave) * K;
+        const int64_t base = ((int64_t)expert * N + ic * (16 * COLS) + wave) * K;
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
             i_wp[cb] = (const uint32_t *)(mat[cb].wq + (base >> 1));
@@ -213,8 +223,14 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
         const int cb = d % CB;
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
-            ring_w[d][i] = i_wp[cb][w_idx[i]];
-            ring_a[d][i] = i_ap[cb][a_off[cb][i]];
+            const uint32_t w_idx = x_off[i] >> 3;
+            ring_w[d][0][i] = i_wp[cb][w_idx];
+            const uint32_t a_off = x_off[i] >> mat[cb].bs_shift;  // (computed here: a register per load and matrix less)
+            ring_a[d][0][i] = i_ap[cb][a_off];
+            if constexpr (COLS == 2) {
+                ring_w[d][1][i] = i_wp[cb][w_step + w_idx];
+                ring_a[d][1][i] = i_ap[cb][a_step[cb] + a_off];
+            }
         }
         // past the end the cursor stays on the last unit: loads that nobody uses
         if (cb == CB - 1 && i_units_left > 1) {
@@ -226,8 +242,8 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
             } else {
 #pragma unroll
                 for (int c2 = 0; c2 < CB; ++c2) {
-                    i_wp[c2] += w_step;
-                    i_ap[c2] += a_step[c2];
+                    i_wp[c2] += COLS * w_step;
+                    i_ap[c2] += COLS * a_step[c2];
                 }
             }
         }
@@ -238,7 +254,7 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
     // ---- the loop over the columns
     uint4_t xr[ROWS][NL];
     int cg = ig0, cc = ic0;  // cursor of the arithmetic
-    int rows = 0, row0 = 0, o_col = cc * 16;
+    int rows = 0, row0 = 0, o_col = cc * (16 * COLS);
     int64_t o_row[ROWS];  // where the wave's column of unit 0 is in the output, per row of the group
     bool fresh = true;
     float first[ROWS];  // the gate projection's sums, until the up projection's are there
@@ -252,7 +268,7 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
                 row0 = __builtin_amdgcn_readfirstlane(grp_r[cg]);
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r) {
-                    o_row[r] = (int64_t)(row0 + r) * N + wave;
+                    o_row[r] = (int64_t)(row0 + r) * N + wave + (COLS == 2 ? (lane >> 5) * 16 : 0);  // lanes 32..63 end up with the second column
                     int64_t src_row = row0 + (r < rows ? r : rows - 1);
                     if (row_idx != nullptr) src_row = (uint32_t)row_idx[src_row] / (uint32_t)idx_div;
                     const bf16_t *const xp = x + src_row * K;
@@ -268,52 +284,59 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
             // The slot's values move to registers of the column and the slot is asked for again right away, in one
             // place for all row counts: were the loads issued inside the branches below, the branches would load
             // into different registers, and the copy that reconciles them would wait for the load just issued.
-            uint32_t wv[NL];
-            float av[NL];
-#pragma unroll
-            for (int i = 0; i < NL; ++i) {
-                wv[i] = ring_w[d][i];
-                av[i] = ring_a[d][i];
-            }
-            if (more) issue(d);
-            // the arithmetic of the column for RN rows: one branch on the number of rows per column, none inside
+            // (the next loads are asked for behind the arithmetic, in one place for all row counts: asked for inside
+            // the branches below they would land in different registers per branch, and the copy that reconciles
+            // them would wait for the load just issued)
+            // the arithmetic of the two columns for RN rows: one branch on the number of rows per unit, none inside
             auto arithmetic = [&](auto RN) {
                 constexpr int rn = decltype(RN)::value;
-                float acc[rn];
+                float acc[COLS][rn];
 #pragma unroll
-                for (int r = 0; r < rn; ++r) acc[r] = 0.f;
+                for (int c = 0; c < COLS; ++c)
+#pragma unroll
+                    for (int r = 0; r < rn; ++r) acc[c][r] = 0.f;
 #pragma unroll
                 for (int i = 0; i < NL; ++i) {
-                    uint32_t pr[4];
-                    lookup4(pr, pair_address<0>(wv[i], lane_copy), pair_address<1>(wv[i], lane_copy),
-                            pair_address<2>(wv[i], lane_copy), pair_address<3>(wv[i], lane_copy));
 #pragma unroll
-                    for (int r = 0; r < rn; ++r) {
-                        float s = dot2_bf16(pr[0], xr[r][i][0], 0.f);
-                        s = dot2_bf16(pr[1], xr[r][i][1], s);
-                        s = dot2_bf16(pr[2], xr[r][i][2], s);
-                        s = dot2_bf16(pr[3], xr[r][i][3], s);
-                        acc[r] = __builtin_fmaf(av[i], s, acc[r]);
+                    for (int c = 0; c < COLS; ++c) {
+                        uint32_t pr[4];
+                        lookup4(pr, pair_address<0>(ring_w[d][c][i], lane_copy), pair_address<1>(ring_w[d][c][i], lane_copy),
+                                pair_address<2>(ring_w[d][c][i], lane_copy), pair_address<3>(ring_w[d][c][i], lane_copy));
+#pragma unroll
+                        for (int r = 0; r < rn; ++r) {
+                            float s = dot2_bf16(pr[0], xr[r][i][0], 0.f);
+                            s = dot2_bf16(pr[1], xr[r][i][1], s);
+                            s = dot2_bf16(pr[2], xr[r][i][2], s);
+                            s = dot2_bf16(pr[3], xr[r][i][3], s);
+                            acc[c][r] = __builtin_fmaf(ring_a[d][c][i], s, acc[c][r]);
+                        }
                     }
                 }
+                // the two columns' 64 partial sums each become 32 + 32 in one swap of half waves and one add, and
+                // five data-parallel-primitive adds finish both: the first column's sum in lane 31, the second's in 63
+                float tot[rn];
 #pragma unroll
-                for (int r = 0; r < rn; ++r) acc[r] = wave_sum_to_last(acc[r]);
+                for (int r = 0; r < rn; ++r) {
+                    // (one column: summed in the same order as each of two, so that the gated form's products are
+                    // bit for bit those of the plain one; its sum is in lane 31 and in lane 63)
+                    tot[r] = two_sums_to_31_and_63(acc[0][r], acc[COLS - 1][r]);
+                }
                 if (GLU && cb == 0) {
 #pragma unroll
-                    for (int r = 0; r < rn; ++r) first[r] = acc[r];
+                    for (int r = 0; r < rn; ++r) first[r] = tot[r];
                     return;
                 }
-                if (lane == 63) {
+                if (COLS == 2 ? (lane & 31) == 31 : lane == 63) {  // one lane per column
 #pragma unroll
                     for (int r = 0; r < rn; ++r) {
                         const int64_t o = o_row[r] + o_col;
                         if constexpr (GLU) {
-                            const bf16_t pe = (bf16_t)first[r], pg = (bf16_t)acc[r];
+                            const bf16_t pe = (bf16_t)first[r], pg = (bf16_t)tot[r];
                             ((bf16_t *)y)[o] = silu_fwd_one<bf16_t>(pe, pg);
                             if (e_out) ((bf16_t *)e_out)[o] = pe;
                             if (g_out) ((bf16_t *)g_out)[o] = pg;
                         } else {
-                            y[o] = from_f32<TO>(acc[r]);
+                            y[o] = from_f32<TO>(tot[r]);
                         }
                     }
                 }
@@ -326,8 +349,9 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
                 arithmetic(std::integral_constant<int, (ROWS > 2 ? 3 : 1)>());
             else
                 arithmetic(std::integral_constant<int, ROWS>());
+            if (more) issue(d);
             if (cb == CB - 1) {
-                o_col += 16;
+                o_col += 16 * COLS;
                 if (++cc == units_n) {
                     cc = 0;
                     o_col = 0;
@@ -349,13 +373,13 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
         if (d < rest) column(d, false);
 }
 
-template <int NL, int ROWS, int D, bool GLU, typename TO>
+template <int NL, int ROWS, int D, bool GLU, bool EXACT, typename TO>
 int launch_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
                 const void *m_sizes, int ms_i64, TO *y, TO *e_out, TO *g_out, int64_t R, int N, int K, int E,
                 hipStream_t stream) {
     const int64_t max_groups = R / ROWS + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / ROWS)
     const int lds = kGemvTable + (int)max_groups * 8 + 16 + E * 4;
-    auto *kernel = nf4_gemv_kernel<NL, ROWS, D, GLU, TO>;
+    auto *kernel = nf4_gemv_kernel<NL, ROWS, D, GLU, EXACT, TO>;
     static PerDeviceOnce attr;
     const hipError_t e = attr.run([&] {
         return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kGemvTable + 4096 * 8 + 16 + 2048 * 4);
@@ -363,22 +387,26 @@ int launch_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4M
     if (e != hipSuccess) return (int)e;
     kernel<<<(unsigned)device_info().cu_count, kGemvThreads, lds, stream>>>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64,
                                                                             y, e_out, g_out, R, N, K, E,
-                                                                            ceil_div(N, 16), (int)max_groups);
+                                                                            N / (GLU ? 16 : 32), (int)max_groups);
     return launch_status();
 }
 
-template <int NL, int ROWS, int D>
+template <int NL, int ROWS>
 int dispatch_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
                   bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
                   int K, int E, int out_dtype, hipStream_t stream) {
+    const bool exact = K % 512 == 0;
+#define MFL_GEMV(GLU, EXACT, TO, Y, EO, GO) \
+    launch_gemv<NL, ROWS, (GLU ? 4 : 2), GLU, EXACT, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream)
     if (glu)
-        return launch_gemv<NL, ROWS, D, true, bf16_t>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (bf16_t *)y,
-                                                   (bf16_t *)e_out, (bf16_t *)g_out, R, N, K, E, stream);
+        return exact ? MFL_GEMV(true, true, bf16_t, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out)
+                     : MFL_GEMV(true, false, bf16_t, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out);
     if (out_dtype == MFL_BF16)
-        return launch_gemv<NL, ROWS, D, false, bf16_t>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (bf16_t *)y, nullptr,
-                                                    nullptr, R, N, K, E, stream);
-    return launch_gemv<NL, ROWS, D, false, float>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (float *)y, nullptr,
-                                               nullptr, R, N, K, E, stream);
+        return exact ? MFL_GEMV(false, true, bf16_t, (bf16_t *)y, nullptr, nullptr)
+                     : MFL_GEMV(false, false, bf16_t, (bf16_t *)y, nullptr, nullptr);
+    return exact ? MFL_GEMV(false, true, float, (float *)y, nullptr, nullptr)
+                 : MFL_GEMV(false, false, float, (float *)y, nullptr, nullptr);
+#undef MFL_GEMV
 }
 
 }  // namespace
@@ -387,8 +415,8 @@ int gemm_nf4_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf
                   bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
                   int K, int E, int out_dtype, hipStream_t stream) {
     if (R <= 0 || R > 2 * (int64_t)E || E > 2048) return MFL_ERR_UNSUPPORTED;  // a few rows per expert only
-    // whole units of 16 columns; fewer than 2^31 units in all
-    if (K % 8 != 0 || K > 2048 || N % 16 != 0 || N > (1 << 18)) return MFL_ERR_UNSUPPORTED;
+    // whole units of 16 columns per matrix column of the wave; fewer than 2^31 units in all
+    if (K % 8 != 0 || K > 2048 || N % (glu ? 16 : 32) != 0 || N > (1 << 18)) return MFL_ERR_UNSUPPORTED;
     const Nf4Matrix *mats[2] = {&w0, &w1};
     for (int cb = 0; cb < (glu ? 2 : 1); ++cb) {
         const Nf4Matrix &m = *mats[cb];
@@ -401,7 +429,7 @@ int gemm_nf4_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf
     // lanes, the store) outweighs the column's 64 to 512 bytes, and the streaming form is faster (measured at
     // K = 768: 43 against 27 us at 16 tokens of 8 experts each).
     if (K <= 1024) return MFL_ERR_UNSUPPORTED;
-    return dispatch_gemv<4, 2, 4>(x, row_idx, idx_div, w0, w1, glu, m_sizes, ms_i64, y, e_out, g_out, R, N, K, E,
+    return dispatch_gemv<4, 2>(x, row_idx, idx_div, w0, w1, glu, m_sizes, ms_i64, y, e_out, g_out, R, N, K, E,
                                   out_dtype, stream);
 }
 
