@@ -119,8 +119,8 @@ def test_streaming_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, out_d
     assert torch.equal(y2[:R - 3], y[:R - 3])
 
 
-# The matrix-vector kernel (at most two rows per expert on average, 1024 < K <= 2048, K a multiple of the block
-# size, N a multiple of 32): lanes past the end of a row (K not a multiple of 512), experts of one to five rows
+# The matrix-vector kernel (at most two rows per expert on average, 256 < K <= 2048, K a multiple of the block
+# size, N a multiple of 32; up to K = 1024 with 32 lanes to a column): lanes past the end of a row (K not a multiple of 512), experts of one to five rows
 # (up to three row groups), empty experts, more than 64 experts, more units than workgroups and fewer, one
 # block per row, 64-bit counts, fp32 output, rows past sum(m_sizes).
 @pytest.mark.parametrize("m_sizes,N,K,blocksize,ms_dtype,out_dtype", [
@@ -131,13 +131,18 @@ def test_streaming_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, out_d
     ([1, 2, 0, 1, 3, 0, 0, 1], 768, 2048, 64, torch.int64, torch.bfloat16),
     ([1, 1], 32, 1088, 64, torch.int32, torch.bfloat16),
     ([0, 0, 0, 4], 64, 1032, 8, torch.int32, torch.float32),
+    # 32 lanes to a column (K <= 1024, at most a row per expert on average) from here on
+    ([1, 2, 0, 1, 0, 0, 0, 1], 2048, 768, 64, torch.int32, torch.bfloat16),
+    ([2, 0, 0], 32, 1024, 128, torch.int64, torch.float32),
+    ([1, 0, 1, 0, 0, 0, 3], 96, 264, 8, torch.int32, torch.bfloat16),
+    ([0] * 66 + [1, 2], 64, 520, 8, torch.int32, torch.bfloat16),
 ])
 def test_matrix_vector_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, out_dtype):
     E = len(m_sizes)
     ms = torch.tensor(m_sizes, dtype=ms_dtype)
-    pad = min(3, 2 * E - int(ms.sum()))        # rows past the last expert: not written
+    pad = min(3, (2 * E if K > 1024 else E) - int(ms.sum()))   # rows past the last expert: not written
     R = int(ms.sum()) + pad
-    assert R <= 2 * E and 1024 < K <= 2048 and K % blocksize == 0 and N % 32 == 0
+    assert R <= (2 * E if K > 1024 else E) and 256 < K <= 2048 and K % blocksize == 0 and N % 32 == 0
     packed, state, w_deq = _quantised(E, N, K, blocksize, N + K)
     x = randn((R, K), gen(K), 1.0, torch.bfloat16)
     sel = oracle.sel_from_m_sizes(np.asarray(m_sizes))

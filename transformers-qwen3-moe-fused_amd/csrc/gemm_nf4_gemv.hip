@@ -1,4 +1,4 @@
-// Fused NF4 grouped product for batches of a few rows per expert (1024 < K <= 2048): a matrix-vector form.
+// Fused NF4 grouped product for batches of a few rows per expert (256 < K <= 2048): a matrix-vector form.
 //
 // With one or two rows per expert there is nothing for a matrix core to share: a 32-row MFMA tile would
 // be 3 to 6 % full, and what the launch has to do is pull every routed expert's packed weights through
@@ -23,6 +23,8 @@
 //     the launch (16 columns in the gated form) dealt out in equal contiguous shares: no second round of
 //     workgroups, and a workgroup changes rows once or twice.  Each wave keeps the loads of four columns ahead
 //     in registers.
+//   * rows of at most 1024 elements: 32 lanes to a column, the wave's second column (16 further on) in lanes
+//     32..63, loads of 128 bytes per half wave, no swap before the five adds.
 //   What the loop is short of, with 16 waves to a CU, is issue slots, scalar ones first: addresses move by
 //   increments, the row count is branched on once per column, and the lookups of a dword wait once.
 //
@@ -63,6 +65,16 @@ __device__ __forceinline__ float two_sums_to_31_and_63(float a, float b) {
     return x;
 }
 
+// lanes 0..31 hold the partial sums of one column, lanes 32..63 of another: the sums in lanes 31 and 63
+__device__ __forceinline__ float half_sums_to_31_and_63(float x) {
+    x = dpp_fadd_step<0x111, 0xf>(x);  // row_shr 1
+    x = dpp_fadd_step<0x112, 0xf>(x);  // row_shr 2
+    x = dpp_fadd_step<0x114, 0xf>(x);  // row_shr 4
+    x = dpp_fadd_step<0x118, 0xf>(x);  // row_shr 8
+    x = dpp_fadd_step<0x142, 0xa>(x);  // row_bcast 15 into rows 1 and 3
+    return x;
+}
+
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
 }
@@ -89,7 +101,7 @@ __device__ __forceinline__ uint32_t pair_address(uint32_t w, uint32_t lane_copy)
 }
 
 // NL: loads per column (K <= 512 NL); ROWS: rows per group; D: columns whose loads a wave keeps in flight
-template <int NL, int ROWS, int D, bool GLU, bool EXACT, typename TO>
+template <int NL, int ROWS, int D, bool GLU, bool EXACT, bool HALF, typename TO>
 __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__restrict__ x,
                                                                 const int32_t *__restrict__ row_idx, int idx_div,
                                                                 Nf4Matrix w0, Nf4Matrix w1,
@@ -100,7 +112,11 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
     constexpr int CB = GLU ? 2 : 1;
     // Columns per wave and unit: two, 16 apart, for the plain product (the loop's scalar work and the sum over the
     // lanes are shared by both); one for the gated form, whose second matrix leaves no registers for a second column.
-    constexpr int COLS = GLU ? 1 : 2;
+    constexpr int COLS = (GLU || HALF) ? 1 : 2;
+    // HALF (rows of at most 1024 elements): 32 lanes to a column, the wave's second column (16 further on) in its
+    // upper 32 lanes instead of in registers of its own: a load serves both, and the sums need no swap.
+    constexpr int UCOLS = HALF ? 32 : 16 * COLS;  // columns of a unit per wave-column: 16 waves x UCOLS / 16
+    static_assert(!(HALF && EXACT), "");
     static_assert(D % CB == 0, "the matrix of a ring slot is fixed");
     extern __shared__ __attribute__((aligned(256))) unsigned char smem[];
     unsigned char *const table = smem;                      // kGemvTable bytes
@@ -187,7 +203,7 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
     const Nf4Matrix mat[2] = {w0, w1};
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-        const int k = (i * 64 + lane) * 8;
+        const int k = HALF ? (i * 32 + (lane & 31)) * 8 : (i * 64 + lane) * 8;
         inside[i] = EXACT ? i * 512 < K : k < K;
         x_off[i] = EXACT ? (uint32_t)(lane * 8 + (i * 512 < K ? i * 512 : 0)) : (uint32_t)(inside[i] ? k : 0);
     }
@@ -207,7 +223,7 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
     const float *i_ap[CB];
     auto point_loads = [&]() {
         const int expert = __builtin_amdgcn_readfirstlane(grp_e[ig]) & 0xffff;
-        const int64_t base = ((int64_t)expert * N + ic * (16 * COLS) + wave) * K;
+        const int64_t base = ((int64_t)expert * N + ic * UCOLS + wave) * K;
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
             i_wp[cb] = (const uint32_t *)(mat[cb].wq + (base >> 1));
@@ -223,9 +239,10 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
         const int cb = d % CB;
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
-            const uint32_t w_idx = x_off[i] >> 3;
+            const uint32_t w_idx = (x_off[i] >> 3) + (HALF ? (lane >> 5) * w_step : 0);
             ring_w[d][0][i] = i_wp[cb][w_idx];
-            const uint32_t a_off = x_off[i] >> mat[cb].bs_shift;  // (computed here: a register per load and matrix less)
+            // (computed here: a register per load and matrix less)
+            const uint32_t a_off = (x_off[i] >> mat[cb].bs_shift) + (HALF ? (lane >> 5) * a_step[cb] : 0);
             ring_a[d][0][i] = i_ap[cb][a_off];
             if constexpr (COLS == 2) {
                 ring_w[d][1][i] = i_wp[cb][w_step + w_idx];
@@ -242,8 +259,8 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
             } else {
 #pragma unroll
                 for (int c2 = 0; c2 < CB; ++c2) {
-                    i_wp[c2] += COLS * w_step;
-                    i_ap[c2] += COLS * a_step[c2];
+                    i_wp[c2] += (UCOLS / 16) * w_step;
+                    i_ap[c2] += (UCOLS / 16) * a_step[c2];
                 }
             }
         }
@@ -254,7 +271,7 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
     // ---- the loop over the columns
     uint4_t xr[ROWS][NL];
     int cg = ig0, cc = ic0;  // cursor of the arithmetic
-    int rows = 0, row0 = 0, o_col = cc * (16 * COLS);
+    int rows = 0, row0 = 0, o_col = cc * UCOLS;
     int64_t o_row[ROWS];  // where the wave's column of unit 0 is in the output, per row of the group
     bool fresh = true;
     float first[ROWS];  // the gate projection's sums, until the up projection's are there
@@ -268,7 +285,7 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
                 row0 = __builtin_amdgcn_readfirstlane(grp_r[cg]);
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r) {
-                    o_row[r] = (int64_t)(row0 + r) * N + wave + (COLS == 2 ? (lane >> 5) * 16 : 0);  // lanes 32..63 end up with the second column
+                    o_row[r] = (int64_t)(row0 + r) * N + wave + (UCOLS == 32 ? (lane >> 5) * 16 : 0);  // lanes 32..63 end up with the second column
                     int64_t src_row = row0 + (r < rows ? r : rows - 1);
                     if (row_idx != nullptr) src_row = (uint32_t)row_idx[src_row] / (uint32_t)idx_div;
                     const bf16_t *const xp = x + src_row * K;
@@ -319,14 +336,17 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
                 for (int r = 0; r < rn; ++r) {
                     // (one column: summed in the same order as each of two, so that the gated form's products are
                     // bit for bit those of the plain one; its sum is in lane 31 and in lane 63)
-                    tot[r] = two_sums_to_31_and_63(acc[0][r], acc[COLS - 1][r]);
+                    if constexpr (HALF)
+                        tot[r] = half_sums_to_31_and_63(acc[0][r]);
+                    else
+                        tot[r] = two_sums_to_31_and_63(acc[0][r], acc[COLS - 1][r]);
                 }
                 if (GLU && cb == 0) {
 #pragma unroll
                     for (int r = 0; r < rn; ++r) first[r] = tot[r];
                     return;
                 }
-                if (COLS == 2 ? (lane & 31) == 31 : lane == 63) {  // one lane per column
+                if (UCOLS == 32 ? (lane & 31) == 31 : lane == 63) {  // one lane per column
 #pragma unroll
                     for (int r = 0; r < rn; ++r) {
                         const int64_t o = o_row[r] + o_col;
@@ -351,7 +371,7 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
                 arithmetic(std::integral_constant<int, ROWS>());
             if (more) issue(d);
             if (cb == CB - 1) {
-                o_col += 16 * COLS;
+                o_col += UCOLS;
                 if (++cc == units_n) {
                     cc = 0;
                     o_col = 0;
@@ -373,13 +393,13 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
         if (d < rest) column(d, false);
 }
 
-template <int NL, int ROWS, int D, bool GLU, bool EXACT, typename TO>
+template <int NL, int ROWS, int D, bool GLU, bool EXACT, bool HALF, typename TO>
 int launch_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
                 const void *m_sizes, int ms_i64, TO *y, TO *e_out, TO *g_out, int64_t R, int N, int K, int E,
                 hipStream_t stream) {
     const int64_t max_groups = R / ROWS + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / ROWS)
     const int lds = kGemvTable + (int)max_groups * 8 + 16 + E * 4;
-    auto *kernel = nf4_gemv_kernel<NL, ROWS, D, GLU, EXACT, TO>;
+    auto *kernel = nf4_gemv_kernel<NL, ROWS, D, GLU, EXACT, HALF, TO>;
     static PerDeviceOnce attr;
     const hipError_t e = attr.run([&] {
         return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kGemvTable + 4096 * 8 + 16 + 2048 * 4);
@@ -387,17 +407,18 @@ int launch_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4M
     if (e != hipSuccess) return (int)e;
     kernel<<<(unsigned)device_info().cu_count, kGemvThreads, lds, stream>>>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64,
                                                                             y, e_out, g_out, R, N, K, E,
-                                                                            N / (GLU ? 16 : 32), (int)max_groups);
+                                                                            N / ((GLU && !HALF) ? 16 : 32), (int)max_groups);
     return launch_status();
 }
 
-template <int NL, int ROWS>
+template <int NL, int ROWS, bool HALF>
 int dispatch_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
                   bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
                   int K, int E, int out_dtype, hipStream_t stream) {
-    const bool exact = K % 512 == 0;
-#define MFL_GEMV(GLU, EXACT, TO, Y, EO, GO) \
-    launch_gemv<NL, ROWS, (GLU ? 4 : 2), GLU, EXACT, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream)
+    const bool exact = !HALF && K % 512 == 0;
+#define MFL_GEMV(GLU, EXACT, TO, Y, EO, GO)                                                                         \
+    launch_gemv<NL, ROWS, ((GLU || HALF) ? 4 : 2), GLU, (EXACT && !HALF), HALF, TO>(x, row_idx, idx_div, w0, w1, m_sizes, \
+                                                                                 ms_i64, Y, EO, GO, R, N, K, E, stream)
     if (glu)
         return exact ? MFL_GEMV(true, true, bf16_t, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out)
                      : MFL_GEMV(true, false, bf16_t, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out);
@@ -415,8 +436,13 @@ int gemm_nf4_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf
                   bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
                   int K, int E, int out_dtype, hipStream_t stream) {
     if (R <= 0 || R > 2 * (int64_t)E || E > 2048) return MFL_ERR_UNSUPPORTED;  // a few rows per expert only
-    // whole units of 16 columns per matrix column of the wave; fewer than 2^31 units in all
-    if (K % 8 != 0 || K > 2048 || N % (glu ? 16 : 32) != 0 || N > (1 << 18)) return MFL_ERR_UNSUPPORTED;
+    const bool half = K <= 1024;  // 32 lanes to a column
+    // (short rows: ahead of the streaming form only up to a row per expert: 23.5 against 25.5 us at 16 tokens of 8
+    // experts each for K = 768, N = 2048, 35.0 against 30.4 us at 32 tokens)
+    if (half && R > E) return MFL_ERR_UNSUPPORTED;
+    if (K % 8 != 0 || K > 2048 || K <= 256) return MFL_ERR_UNSUPPORTED;
+    // whole units (32 columns; 16 in the gated form with 64 lanes to a column); fewer than 2^31 units in all
+    if (N % ((glu && !half) ? 16 : 32) != 0 || N > (1 << 18)) return MFL_ERR_UNSUPPORTED;
     const Nf4Matrix *mats[2] = {&w0, &w1};
     for (int cb = 0; cb < (glu ? 2 : 1); ++cb) {
         const Nf4Matrix &m = *mats[cb];
@@ -425,12 +451,11 @@ int gemm_nf4_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf
         if (!aligned(m.absmax, 4) || !aligned(m.wq, 4)) return MFL_ERR_UNSUPPORTED;
     }
     if (!aligned(x, 16)) return MFL_ERR_UNSUPPORTED;
-    // Rows of more than 1024 elements only: with shorter ones the work per column (addresses, the sum over the
-    // lanes, the store) outweighs the column's 64 to 512 bytes, and the streaming form is faster (measured at
-    // K = 768: 43 against 27 us at 16 tokens of 8 experts each).
-    if (K <= 1024) return MFL_ERR_UNSUPPORTED;
-    return dispatch_gemv<4, 2>(x, row_idx, idx_div, w0, w1, glu, m_sizes, ms_i64, y, e_out, g_out, R, N, K, E,
-                                  out_dtype, stream);
+#define MFL_GEMV_D(NL, ROWS, HALF) \
+    dispatch_gemv<NL, ROWS, HALF>(x, row_idx, idx_div, w0, w1, glu, m_sizes, ms_i64, y, e_out, g_out, R, N, K, E, out_dtype, stream)
+    if (!half) return MFL_GEMV_D(4, 2, false);
+    return K <= 768 ? MFL_GEMV_D(3, 2, true) : MFL_GEMV_D(4, 2, true);
+#undef MFL_GEMV_D
 }
 
 }  // namespace mfl
