@@ -85,6 +85,19 @@ MFL_API int mfl_gemm_dw(const void *x, const void *dy, const void *m_sizes, int 
                 int64_t R, int N, int K, int E, int in_dtype, int out_dtype, float alpha,
                 int accumulate, void *stream);
 
+/* mfl_gemm_dw for a product with one thin side -- N or K equal to 16 or 32 (the rank of a LoRA adapter,
+ * qwen3_moe_fused/lora.py:71-72: the products dA and dB of qwen3_moe_fused/kernels/fast_lora.py:121-125,
+ * 139-149), the other side a multiple of 256, bf16 operands, bf16 or fp32 result, at most 512 experts.
+ * The rows are dealt out evenly over the workgroups whatever the sizes of the experts; an expert cut by
+ * such a border is summed from fp32 partial results in a fixed order (same bits from run to run).
+ * Every element of dw is written.  workspace: mfl_gemm_dw_split_workspace(R, N, K, E) bytes of device
+ * memory, contents ignored; that function returns 0 for a shape this entry point does not take, and the
+ * call then returns MFL_ERR_UNSUPPORTED: use mfl_gemm_dw. */
+MFL_API size_t mfl_gemm_dw_split_workspace(int64_t R, int N, int K, int E);
+MFL_API int mfl_gemm_dw_split(const void *x, const void *dy, const void *m_sizes, int m_sizes_dtype, void *dw,
+                      int64_t R, int N, int K, int E, int in_dtype, int out_dtype, float alpha,
+                      void *workspace, size_t ws_bytes, void *stream);
+
 /* Forward GEMM with NF4 weights decoded inside the K loop:
  * w[e, n, k] = code16[nibble] * absmax[(e*N*K + n*K + k) / blocksize], rounded once to
  * in_dtype; byte i of wq holds element 2i in its high nibble, 2i+1 in its low nibble.

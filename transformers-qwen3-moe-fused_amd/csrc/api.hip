@@ -103,6 +103,19 @@ int mfl_gemm_dw(const void *x, const void *dy, const void *m_sizes, int m_sizes_
                     stream);
 }
 
+size_t mfl_gemm_dw_split_workspace(int64_t R, int N, int K, int E) { return gemm_dw_split_workspace(R, N, K, E); }
+
+int mfl_gemm_dw_split(const void *x, const void *dy, const void *m_sizes, int m_sizes_dtype, void *dw, int64_t R, int N,
+                      int K, int E, int in_dtype, int out_dtype, float alpha, void *workspace, size_t ws_bytes,
+                      void *stream) {
+    int rc = check_gemm(dy, x, m_sizes, m_sizes_dtype, dw, R, N, K, E, in_dtype, out_dtype);
+    if (rc) return rc;
+    if (!dw || (R > 0 && !x)) return MFL_ERR_NULL;
+    if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    return gemm_dw_split(dy, x, m_sizes, m_sizes_dtype == MFL_I64, dw, R, N, K, E, out_dtype, alpha, workspace, ws_bytes,
+                         (hipStream_t)stream);
+}
+
 int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
                      const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K, int E, int in_dtype,
                      int out_dtype, void *stream) {

@@ -31,6 +31,8 @@ _SIGNATURES = {
     "mfl_gemm_fwd": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "mfl_gemm_dx": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "mfl_gemm_dw": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _i, _vp]),
+    "mfl_gemm_dw_split_workspace": (_sz, [_i64, _i, _i, _i]),
+    "mfl_gemm_dw_split": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _vp, _sz, _vp]),
     "mfl_gemm_fwd_nf4": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
     "mfl_gemm_dx_nf4": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "mfl_gemm_dx_dual": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _vp]),

@@ -11,7 +11,11 @@ from typing import Optional
 
 import torch
 
+from .. import _lib
 from ._common import check_operands, launch
+
+# below this many rows the general kernel is as fast and needs no workspace
+_SPLIT_MIN_ROWS = 4096
 
 
 def grouped_gemm_backward_dw(x: torch.Tensor, y: torch.Tensor, m_sizes: torch.Tensor, dtype: torch.dtype, *,
@@ -28,5 +32,18 @@ def grouped_gemm_backward_dw(x: torch.Tensor, y: torch.Tensor, m_sizes: torch.Te
         out = torch.empty((experts, n, k), device=x.device, dtype=dtype)
     else:
         assert out.shape == (experts, n, k) and out.is_contiguous() and out.device == x.device
+    if not accumulate and rows >= _SPLIT_MIN_ROWS and x.dtype == torch.bfloat16:
+        # one side as thin as a LoRA rank: the rows are dealt out evenly over the workgroups, so that the
+        # expert with the most rows does not decide the time of the launch
+        ws_bytes = int(_lib.lib().mfl_gemm_dw_split_workspace(rows, n, k, experts))
+        if ws_bytes > 0 and out.dtype in (torch.bfloat16, torch.float32):
+            ws = torch.empty(ws_bytes, device=x.device, dtype=torch.uint8)
+            ms = _lib.as_index_tensor(m_sizes)
+            rc = _lib.lib().mfl_gemm_dw_split(_lib.ptr(x), _lib.ptr(y), _lib.ptr(ms), _lib.itype_code(ms.dtype),
+                                              _lib.ptr(out), rows, n, k, experts, _lib.dtype_code(x.dtype),
+                                              _lib.dtype_code(out.dtype), float(alpha), _lib.ptr(ws), ws_bytes,
+                                              _lib.stream())
+            _lib.check(rc, "mfl_gemm_dw_split")
+            return out
     # the C entry point takes (x, dy); launch() passes its first two tensors in order
     return launch("mfl_gemm_dw", x, y, m_sizes, out, rows, n, k, experts, alpha, accumulate)
