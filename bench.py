@@ -385,8 +385,36 @@ def main() -> int:
                 lora[name]["tflops"] = round(flop4 / us / 1e6, 1)
             else:
                 lora[name]["wide_operand_gbs"] = round(stream_bytes / us / 1e3, 1)
+        # the base product with the rank-16 term in the same reduction (one pass over the output), forward and
+        # input gradient, and the expert MLP with adapters on all three projections, forward + backward
+        from qwen3_moe_fused.grouped_gemm.fused import grouped_gemm_forward_lora, grouped_gemm_forward_transposed_lora
+        from qwen3_moe_fused.kernels.fast_lora import fast_lora
+        us = _event_us(lambda i: grouped_gemm_forward_lora(x4, ws[0], u4, lb, ms4), 50, 100, stream)
+        lora["base_fwd_with_lora_term"] = {"us": round(us, 1), "tflops": round(flop4 / us / 1e6, 1)}
+        us = _event_us(lambda i: grouped_gemm_forward_transposed_lora(dy4, ws[0].view(E, INTER, HIDDEN), t4, la, ms4),
+                       50, 100, stream)
+        lora["base_dx_with_lora_term"] = {"us": round(us, 1), "tflops": round(flop4 / us / 1e6, 1)}
+        del u4, y4, t4
+        adapters = []
+        for n_in, n_out in ((HIDDEN, INTER), (HIDDEN, INTER), (INTER, HIDDEN)):
+            adapters.append(((torch.randn((E, RANK, n_in), device=dev) * 0.01).bfloat16().requires_grad_(),
+                             (torch.randn((E, n_out, RANK), device=dev) * 0.01).bfloat16().requires_grad_()))
+        w_down = ws[2].view(E, HIDDEN, INTER)
+        x4.requires_grad_()
+        dyh = torch.randn((R4, HIDDEN), device=dev, dtype=torch.bfloat16)
+
+        def mlp_step(i):
+            (ag, bg), (au, bu), (aw, bw) = adapters
+            y = fast_lora(x4, ws[0], None, ag, bg, 2.0, ws[1], None, au, bu, 2.0, w_down, None, aw, bw, 2.0, ms4)
+            y.backward(dyh)
+            x4.grad = None
+            for a_, b_ in adapters:
+                a_.grad = b_.grad = None
+        us = _event_us(mlp_step, 10, 5, stream)
+        lora["expert_mlp_lora_fwd_bwd"] = {"us": round(us, 1), "tokens_per_s": round(T4 / us * 1e6),
+                                           "tflops": round(6 * flop4 / us / 1e6, 1)}  # 3 forward + 3 dX products
         extra["lora_rank16_zipf_config4"] = lora
-        del x4, dy4, u4, y4, t4
+        del x4, dy4, dyh, adapters
         # config 5: the whole sparse block (router -> top-k -> sort -> gather -> gate/up -> SiLU-mul -> down ->
         # weighted combine) with NF4 experts, forward only, module calls as a user makes them
         from types import SimpleNamespace

@@ -130,6 +130,24 @@ MFL_API int mfl_gemm_dx_dual(const void *dy1, const void *w1, const void *dy2, c
                      const void *m_sizes, int m_sizes_dtype, void *dx, int64_t R, int N, int K,
                      int E, int in_dtype, int out_dtype, void *stream);
 
+/* A product with the rank-r term of a LoRA adapter in the same reduction: one accumulator, one
+ * rounding, one pass over the output, where the reference adds the two products
+ * (qwen3_moe_fused/lora.py:134; matmul_lora at kernels/fast_lora.py:65-88,127-131,151-152).
+ *   mfl_gemm_fwd_lora:  y = x w^T + xt wt^T      x (R,K), w (E,N,K), xt (R,KT), wt (E,N,KT)
+ *   mfl_gemm_dx_lora:  dx = dy w (+ dy2 w2) + xt wt    dy, dy2 (R,K), w, w2 (E,K,N), xt (R,KT),
+ *                      wt (E,KT,N); dy2 and w2 both NULL or both given (the gated unit's two terms)
+ * xt is x A^T (or dy B) already multiplied by the adapter's scaling; KT is the rank, a multiple
+ * of 8.  Both return MFL_ERR_UNSUPPORTED, with nothing enqueued, unless the element type is bf16,
+ * N, K and KT are multiples of 8 (K % 64 == 0 with dy2), E <= 512 and the pointers are 16-byte
+ * aligned; the caller then adds the thin product with a second call (accumulate = 1). */
+MFL_API int mfl_gemm_fwd_lora(const void *x, const void *w, const void *xt, const void *wt, int KT,
+                      const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K,
+                      int E, int in_dtype, int out_dtype, void *stream);
+MFL_API int mfl_gemm_dx_lora(const void *dy, const void *w, const void *dy2, const void *w2,
+                     const void *xt, const void *wt, int KT, const void *m_sizes, int m_sizes_dtype,
+                     void *dx, int64_t R, int N, int K, int E, int in_dtype, int out_dtype,
+                     void *stream);
+
 /* ---- forward products fused with their neighbours in the sparse MLP block ---------
  * The reference names these fusions as future work (modular_qwen3_moe_fused.py:100-101,105).
  * Each call returns MFL_ERR_UNSUPPORTED, with nothing enqueued, for a request the pipelined

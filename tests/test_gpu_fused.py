@@ -269,3 +269,84 @@ def test_two_term_input_gradient(R, N, K, E):
         assert torch.equal(dx, dx_cat), "the same reduction in the same order"
     else:
         check_close(dx, to_np32(dx_cat), what="two-term dx vs concatenated product")
+
+
+from qwen3_moe_fused.grouped_gemm.fused import (grouped_gemm_forward_lora,  # noqa: E402
+                                                grouped_gemm_forward_transposed_lora)
+
+# R, N, K, E, rank.  The rank-r term of a LoRA adapter in the reduction of the base product
+# (qwen3_moe_fused/lora.py:134): y = x w^T + xt wt^T.
+LORA_CASES = [(4096, 768, 2048, 16, 16),     # the 320 x 192 tiles of the expert shapes
+              (9000, 512, 256, 4, 32),       # more than 512 rows per expert: 256 x 256 tiles
+              (700, 200, 64, 5, 8),
+              (300, 72, 128, 3, 24),         # rank not a multiple of 16
+              (600, 136, 192, 6, 72),        # rank beyond one reduction step
+              (33, 8, 192, 40, 16),          # a row or none per expert: the flat decode tiles
+              (500, 40, 256, 3, 16),         # thin output: 128 x 64 tiles
+              (64, 24, 72, 4, 16)]           # K % 64 != 0: a partial last step before the thin term
+
+
+@pytest.mark.parametrize("R,N,K,E,r", LORA_CASES)
+def test_forward_with_lora_term(R, N, K, E, r):
+    g = gen(R + N + r)
+    x, xt = randn((R, K), g, 1.0, torch.bfloat16), randn((R, r), g, 1.0, torch.bfloat16)
+    w, wt = randn((E, N, K), g, 0.05, torch.bfloat16), randn((E, N, r), g, 0.2, torch.bfloat16)
+    ms = m_sizes_uniform(R, E, g)
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    y = grouped_gemm_forward_lora(x.to(DEV), w.to(DEV), xt.to(DEV), wt.to(DEV), ms.to(DEV))
+    ref = (oracle.linear_fwd(to_np32(x), to_np32(w), sel).astype(np.float64)
+           + oracle.linear_fwd(to_np32(xt), to_np32(wt), sel))
+    check_close(y, ref, what="forward with a rank-r term vs oracle")
+    # closed form: one product over the concatenated reduction
+    y_cat = grouped_gemm_forward(torch.cat([x, xt], 1).contiguous().to(DEV), torch.cat([w, wt], 2).contiguous().to(DEV),
+                                 ms.to(DEV))
+    if K % 64 == 0:
+        assert torch.equal(y, y_cat), "the same reduction in the same order"
+    else:
+        check_close(y, to_np32(y_cat), what="forward with a rank-r term vs concatenated product")
+
+
+@pytest.mark.parametrize("dual", [False, True])
+@pytest.mark.parametrize("R,N,K,E,r", LORA_CASES)
+def test_input_gradient_with_lora_term(R, N, K, E, r, dual):
+    # dx (R, N) = dy (R, K) @ w[e] (+ dy2 @ w2[e]) + xt (R, r) @ wt[e],  w (E, K, N), wt (E, r, N)
+    g = gen(R + N + r + 1)
+    dy, dy2 = randn((R, K), g, 1.0, torch.bfloat16), randn((R, K), g, 1.0, torch.bfloat16)
+    xt = randn((R, r), g, 1.0, torch.bfloat16)
+    w, w2 = randn((E, K, N), g, 0.05, torch.bfloat16), randn((E, K, N), g, 0.05, torch.bfloat16)
+    wt = randn((E, r, N), g, 0.2, torch.bfloat16)
+    ms = m_sizes_uniform(R, E, g)
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    kw = dict(dy2=dy2.to(DEV), w2=w2.to(DEV)) if dual else {}
+    dx = grouped_gemm_forward_transposed_lora(dy.to(DEV), w.to(DEV), xt.to(DEV), wt.to(DEV), ms.to(DEV), **kw)
+    ref = (oracle.linear_bwd_input(to_np32(dy), to_np32(w), sel).astype(np.float64)
+           + oracle.linear_bwd_input(to_np32(xt), to_np32(wt), sel))
+    if dual:
+        ref = ref + oracle.linear_bwd_input(to_np32(dy2), to_np32(w2), sel)
+    check_close(dx, ref, what="input gradient with a rank-r term vs oracle")
+    terms_a = [dy] + ([dy2] if dual else []) + [xt]
+    terms_w = [w] + ([w2] if dual else []) + [wt]
+    dx_cat = grouped_gemm_forward_transposed(torch.cat(terms_a, 1).contiguous().to(DEV),
+                                             torch.cat(terms_w, 1).contiguous().to(DEV), ms.to(DEV))
+    if K % 64 == 0:
+        assert torch.equal(dx, dx_cat), "the same reduction in the same order"
+    else:
+        check_close(dx, to_np32(dx_cat), what="input gradient with a rank-r term vs concatenated product")
+
+
+def test_lora_term_of_other_element_types_runs_as_two_products():
+    g = gen(77)
+    R, N, K, E, r = 90, 12, 20, 3, 4                     # fp32, odd sizes: no fused kernel
+    x, xt = randn((R, K), g), randn((R, r), g)
+    w, wt = randn((E, N, K), g, 0.1), randn((E, N, r), g, 0.1)
+    ms = m_sizes_uniform(R, E, g)
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    y = grouped_gemm_forward_lora(x.to(DEV), w.to(DEV), xt.to(DEV), wt.to(DEV), ms.to(DEV))
+    ref = oracle.linear_fwd(to_np32(x), to_np32(w), sel).astype(np.float64) + oracle.linear_fwd(to_np32(xt), to_np32(wt), sel)
+    check_close(y, ref, rtol=1e-4, atol=1e-4, what="fp32 forward with a rank-r term")
+    dy = randn((R, N), g)
+    wa = randn((E, r, K), g, 0.1)
+    dx = grouped_gemm_forward_transposed_lora(dy.to(DEV), w.to(DEV), xt.to(DEV), wa.to(DEV), ms.to(DEV))
+    ref = (oracle.linear_bwd_input(to_np32(dy), to_np32(w), sel).astype(np.float64)
+           + oracle.linear_bwd_input(to_np32(xt), to_np32(wa), sel))
+    check_close(dx, ref, rtol=1e-4, atol=1e-4, what="fp32 input gradient with a rank-r term")

@@ -163,6 +163,37 @@ int mfl_gemm_dx_dual(const void *dy1, const void *w1, const void *dy2, const voi
                           (hipStream_t)stream, &fu);
 }
 
+int mfl_gemm_fwd_lora(const void *x, const void *w, const void *xt, const void *wt, int KT, const void *m_sizes,
+                      int m_sizes_dtype, void *y, int64_t R, int N, int K, int E, int in_dtype, int out_dtype,
+                      void *stream) {
+    int rc = check_gemm(x, w, m_sizes, m_sizes_dtype, y, R, N, K, E, in_dtype, out_dtype);
+    if (rc) return rc;
+    if (KT <= 0) return MFL_ERR_SHAPE;
+    if (R > 0 && (!xt || !wt)) return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    GemmFusion fu = {nullptr, 1, 0, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr};
+    fu.xt = xt, fu.wt = wt, fu.kt = KT;
+    return gemm_bf16_pipe(MODE_FWD, x, w, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E, out_dtype, 1.0f, 0,
+                          (hipStream_t)stream, &fu);
+}
+
+int mfl_gemm_dx_lora(const void *dy, const void *w, const void *dy2, const void *w2, const void *xt, const void *wt,
+                     int KT, const void *m_sizes, int m_sizes_dtype, void *dx, int64_t R, int N, int K, int E,
+                     int in_dtype, int out_dtype, void *stream) {
+    int rc = check_gemm(dy, w, m_sizes, m_sizes_dtype, dx, R, N, K, E, in_dtype, out_dtype);
+    if (rc) return rc;
+    if (KT <= 0) return MFL_ERR_SHAPE;
+    if ((dy2 == nullptr) != (w2 == nullptr)) return MFL_ERR_NULL;
+    if (R > 0 && (!xt || !wt)) return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    GemmFusion fu = {nullptr, 1, 0, w2, nullptr, nullptr, 0, nullptr, nullptr, dy2};
+    fu.xt = xt, fu.wt = wt, fu.kt = KT;
+    return gemm_bf16_pipe(MODE_DX, dy, w, m_sizes, m_sizes_dtype == MFL_I64, dx, R, N, K, E, out_dtype, 1.0f, 0,
+                          (hipStream_t)stream, &fu);
+}
+
 /* ---- forward products fused with their neighbours in the sparse MLP block ---- */
 
 namespace {

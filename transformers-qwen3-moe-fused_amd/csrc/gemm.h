@@ -30,6 +30,10 @@ struct GemmFusion {
     void *e_out, *g_out;
     // input gradient with two terms (DX only): dx = dy w + x2 w2, x2 and w2 shaped like dy and w
     const void *x2;
+    // a last term with a reduction length of its own (FWD, DX; bf16 weights): c += xt wt with xt (R, kt) and
+    // wt (E, N, kt) in FWD, (E, kt, N) in DX; kt a multiple of 8.  The rank-r term of a LoRA adapter.
+    const void *xt, *wt;
+    int kt;
 };
 
 // Pipelined bf16 MFMA kernels (direct global->LDS copies, multi-stage) for aligned shapes.

@@ -228,15 +228,24 @@ struct FwdFusion {
     // Two-term input gradient (DX only): the reduction runs over (a, b) and then over (a2, b2),
     // same shapes, one accumulator, one epilogue: dx = a b + a2 b2.
     const void *a2;
+    // A last term with a reduction length of its own (FWD, DX; the rank of a LoRA adapter), after the one or
+    // two terms above, in the same accumulator: c += at bt, at (R, kt), bt (E, N, kt) in FWD and (E, kt, N)
+    // in DX.
+    const void *at, *bt;
+    int kthin;
 };
 
-template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODE, bool NF4, bool GLU, typename TO>
+// FUSE: 0 plain, 1 two weight matrices and the silu(gate) * up epilogue, 2 a thin last term in the reduction (built
+// as a kernel of its own: the test for it in every step cost the plain products 3-5 %).
+template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODE, bool NF4, int FUSE, typename TO>
 __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *__restrict__ a,
                                                                   const bf16_t *__restrict__ b,
                                                                   const void *__restrict__ m_sizes, int ms_i64,
                                                                   TO *__restrict__ c, int64_t R, int N, int K, int E,
                                                                   float alpha, int accumulate, Nf4Params nf4,
                                                                   FwdFusion fu) {
+    constexpr bool GLU = FUSE == 1, THIN = FUSE == 2;
+    static_assert(!THIN || (MODE != MODE_DW && !NF4), "the thin last term belongs to the row-grouped bf16 products");
     static_assert(!NF4 || (MODE != MODE_DW && S == 2 && BK == 64), "NF4 weights: row-grouped products, two stages");
     static_assert(!GLU || (MODE == MODE_FWD && WGN % 2 == 0 && sizeof(TO) == 2 && BK == 64),
                   "GLU: forward product, bf16 output, the waves along N split in a gate half and an up half");
@@ -360,6 +369,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
     const unsigned char *a_tile = nullptr, *b_tile = nullptr;
     const unsigned char *b2_tile = nullptr;
     const unsigned char *a2_tile = nullptr;  // two-term DX: second pair of operands
+    const unsigned char *at_tile = nullptr, *bt_tile = nullptr;  // the thin last term
+    int KT_thin = 0;
     int lda = 0, ldb = 0;
     int64_t ldc = 0, nf4_base = 0;
     TO *c_base = nullptr;
@@ -423,11 +434,18 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                     b2_tile = (const unsigned char *)((const bf16_t *)fu.b2 + (int64_t)expert * N * K + j0);
                 }
             }
+            if constexpr (THIN) {
+                at_tile = (const unsigned char *)((const bf16_t *)fu.at + (int64_t)i0 * fu.kthin);
+                bt_tile = (const unsigned char *)((const bf16_t *)fu.bt + (B_RC ? ((int64_t)expert * N + j0) * fu.kthin
+                                                                               : (int64_t)expert * N * fu.kthin + j0));
+            }
             c_base = c;
         }
         red = r_end - r_begin;
         KT1 = ceil_div(red, BK);                                      // steps of one term
         KT = MODE == MODE_DX && fu.a2 != nullptr ? 2 * KT1 : KT1;  // the host checked K % BK == 0
+        KT_thin = KT;  // first step of the thin term
+        if constexpr (THIN) KT += ceil_div(fu.kthin, BK);
         i_lim = i_end - i0 < BM ? i_end - i0 : BM;  // valid rows (or columns) of A from the tile origin
         j_lim = j_end - j0 < BNH ? j_end - j0 : BNH;
 
@@ -487,8 +505,55 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         // products with a reduction-strided operand read it with transposing LDS reads
         constexpr bool ASM_COPY = MODE != MODE_FWD;
         constexpr int SA_ROWS_PER_COPY = 64 / SA::kChunksPerRow;
+        // A step of the last term, the one with a reduction length of its own: source offsets from that term's leading
+        // dimensions, worked out here (the term is one or two steps of a tile's many); chunks past the end of a
+        // reduction-contiguous row come from a chunk of zeros, rows past the end of a reduction-strided operand
+        // re-read its last row (they meet zeros of the other operand).
+        auto issue_second = [&](int ks, unsigned char *st) {
+            static_assert(MODE == MODE_DW || A_RC, "the left operand of a row-grouped product");
+            const int k2 = fu.kthin;
+            // the lane number behind a barrier for the optimiser: what follows is worked out here, once or twice
+            // per tile, and not kept in registers across the tile's other steps
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+#pragma unroll
+            for (int q = 0; q < LA; ++q) {
+                const int load = wave * LA + q;
+                int i = SA::row_of(load, ln);
+                const int c = SA::swz(i, SA::phys_of(load, ln));
+                if (i >= i_lim) i = i_lim - 1;
+                const int r = ks * BK + c * 8;
+                const unsigned char *p = r >= k2 ? (const unsigned char *)&g_zero_chunk : at_tile + ((int64_t)i * k2 + r) * 2;
+                copy_to_lds<0, ASM_COPY>(p, st + load * 1024);
+            }
+#pragma unroll
+            for (int q = 0; q < LB; ++q) {
+                const int load = wave * LB + q;
+                const int row = SB::row_of(load, ln);
+                const int c = SB::swz(row, SB::phys_of(load, ln));
+                const unsigned char *p;
+                if (B_RC) {
+                    const int j = row < j_lim ? row : j_lim - 1;
+                    const int r = ks * BK + c * 8;
+                    p = r >= k2 ? (const unsigned char *)&g_zero_chunk : bt_tile + ((int64_t)j * k2 + r) * 2;
+                } else {
+                    int r = ks * BK + row;
+                    if (r >= k2) r = k2 - 1;
+                    int j = c * 8;
+                    if (j >= j_lim) j = j_lim - 8;
+                    p = bt_tile + ((int64_t)r * N + j) * 2;
+                }
+                copy_to_lds<0, ASM_COPY>(p, st + SA::kBytes + load * 1024);
+            }
+        };
         auto issue = [&](int kt) {
             unsigned char *st = smem + (kt % S) * STAGE_BYTES;
+            if constexpr (THIN) {
+                if (kt >= KT_thin) {
+                    issue_second(kt - KT_thin, st);
+                    return;
+                }
+            }
             // step of the term that is being reduced (two-term DX: the second term follows the first)
             int ks = kt;
             const unsigned char *a_term = a_tile, *b_term = b_tile;
@@ -927,11 +992,12 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
     constexpr int PER_CU = LDS_BYTES <= 80 * 1024 ? 2 : 1;
     const int grid = device_info().cu_count / kXcd * kXcd * PER_CU;
     const Nf4Params none = {nullptr, nullptr, 0};
-    const FwdFusion no_fusion = {nullptr, 1, nullptr, none, nullptr, nullptr, nullptr};
+    const FwdFusion no_fusion = {nullptr, 1, nullptr, none, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     const FwdFusion fu = fusion ? *fusion : no_fusion;
     const bool glu = fu.b2 != nullptr && fu.a2 == nullptr;
     if ((glu || fu.row_idx) && mode != MODE_FWD) return MFL_ERR_UNSUPPORTED;
     if (fu.a2 != nullptr && (mode != MODE_DX || nf4 != nullptr || fu.b2 == nullptr)) return MFL_ERR_UNSUPPORTED;
+    if (fu.at != nullptr && (mode == MODE_DW || nf4 != nullptr || glu || fu.bt == nullptr)) return MFL_ERR_UNSUPPORTED;
 #define MFL_PIPE(MODE, NF4, GLU)                                                                                \
     {                                                                                                           \
         auto kern = gemm_pipe_kernel<MB, NB, BK, S, WGM, WGN, MODE, NF4, GLU, TO>;                              \
@@ -954,6 +1020,14 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
             } else {
                 MFL_PIPE(MODE_FWD, false, true)
             }
+        } else {
+            return MFL_ERR_UNSUPPORTED;
+        }
+    } else if (fu.at != nullptr) {
+        // MODES bit 4: the configuration is also built with the thin last term
+        if constexpr ((MODES & 16) != 0 && (MODES & 3) == 3) {
+            if (mode == MODE_FWD) MFL_PIPE(MODE_FWD, false, 2)
+            else MFL_PIPE(MODE_DX, false, 2)
         } else {
             return MFL_ERR_UNSUPPORTED;
         }
@@ -1026,22 +1100,22 @@ int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, i
         case 2:
             return MFL_LAUNCH(8, 4, 64, 3, 4, 2, 7);
         case 3:
-            return MFL_LAUNCH(10, 6, 64, 2, 4, 2, 15);
+            return MFL_LAUNCH(10, 6, 64, 2, 4, 2, 31);
         case 4:
             return MFL_LAUNCH(10, 4, 64, 2, 4, 2, 7);
         case 15:  // a few rows per expert (decode): the weights are all the traffic; flat 64 x 128 tiles,
                   // 3 stages of 24 KiB, two workgroups per CU (one with 6 stages: 85 instead of 77 us for
                   // 2048 rows over 128 experts, N = 768, K = 2048)
-            return MFL_LAUNCH(2, 4, 64, 3, 2, 4, 11);
+            return MFL_LAUNCH(2, 4, 64, 3, 2, 4, 27);
         case 10:  // thin output of a row-grouped product: 128 rows x 64 columns, 3 stages of 24 KiB, two
                   // workgroups per CU (one's set-up and epilogue under the other's loop; one workgroup with 6
                   // stages: x A^T 57 instead of 53 us, dy B 28.5 instead of 23.5 us at 65536 rows)
-            return MFL_LAUNCH(4, 2, 64, 3, 4, 1, 3);
+            return MFL_LAUNCH(4, 2, 64, 3, 4, 1, 19);
         case 11:  // dW with a thin side: 64 x 64 tiles (an expert's reduction is spread over as many
                   // workgroups as its wide side has 64-column slices), 8 stages of 16 KiB
             return MFL_LAUNCH(2, 2, 64, 8, 2, 2, 4);
         default:
-            return MFL_LAUNCH(8, 8, 64, 2, 2, 4, 15);
+            return MFL_LAUNCH(8, 8, 64, 2, 2, 4, 31);
     }
 #undef MFL_LAUNCH
 }
@@ -1053,7 +1127,7 @@ namespace {
 // Checks the fusion request of a forward product and translates it for the kernel.
 // Returns MFL_ERR_UNSUPPORTED for what the pipelined kernels do not take.
 int make_fusion(const GemmFusion *f, int K, bool nf4, FwdFusion *out) {
-    *out = FwdFusion{nullptr, 1, nullptr, Nf4Params{nullptr, nullptr, 0}, nullptr, nullptr, nullptr};
+    *out = FwdFusion{nullptr, 1, nullptr, Nf4Params{nullptr, nullptr, 0}, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (f == nullptr) return MFL_OK;
     if (f->row_idx != nullptr) {
         // the kernel addresses the source rows with 32-bit byte offsets
@@ -1061,6 +1135,14 @@ int make_fusion(const GemmFusion *f, int K, bool nf4, FwdFusion *out) {
             return MFL_ERR_UNSUPPORTED;
         out->row_idx = f->row_idx;
         out->idx_div = f->idx_div;
+    }
+    if (f->xt != nullptr) {
+        if (nf4 || f->wt == nullptr || f->kt < 8 || f->kt % 8 != 0 || !aligned(f->xt, 16) || !aligned(f->wt, 16) ||
+            f->row_idx != nullptr || (f->w2 != nullptr && f->x2 == nullptr))
+            return MFL_ERR_UNSUPPORTED;
+        out->at = f->xt;
+        out->bt = f->wt;
+        out->kthin = f->kt;
     }
     if (f->x2 != nullptr) {
         // two-term input gradient: whole reduction steps only, bf16 weights
@@ -1098,7 +1180,10 @@ int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, 
     if (mode == MODE_DW && (N % 8 != 0 || K % 8 != 0 || N < 8 || K < 8)) return MFL_ERR_UNSUPPORTED;
     FwdFusion fu;
     if (fusion != nullptr) {
-        if (mode != (fusion->x2 != nullptr ? MODE_DX : MODE_FWD)) return MFL_ERR_UNSUPPORTED;
+        // two full terms: DX; a thin last term: FWD or DX; everything else: FWD
+        if (mode == MODE_DW || (fusion->x2 != nullptr && mode != MODE_DX) ||
+            (mode == MODE_DX && fusion->x2 == nullptr && fusion->xt == nullptr))
+            return MFL_ERR_UNSUPPORTED;
         if (fusion->x2 == nullptr && fusion->w2 != nullptr && (out_dtype != MFL_BF16 || accumulate || alpha != 1.0f))
             return MFL_ERR_UNSUPPORTED;
         const int rc = make_fusion(fusion, K, false, &fu);

@@ -181,3 +181,61 @@ def grouped_gemm_forward_transposed_dual(dy1: torch.Tensor, w1: torch.Tensor, dy
         return grouped_gemm_forward_transposed(dy2, w2, m_sizes, dtype, out=dx, accumulate=True)
     _lib.check(rc, "mfl_gemm_dx_dual")
     return dx
+
+
+def grouped_gemm_forward_lora(x: torch.Tensor, w: torch.Tensor, xt: torch.Tensor, wt: torch.Tensor,
+                              m_sizes: torch.Tensor, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``grouped_gemm_forward(x, w, m_sizes) + grouped_gemm_forward(xt, wt, m_sizes)`` in one kernel: a product
+    with the rank-r term of a LoRA adapter in the same reduction (``xt = s * x A^T`` (rows, r), ``wt = B``
+    (E, N, r)); the reference adds the two (qwen3_moe_fused/lora.py:134, kernels/fast_lora.py:65-88)."""
+    check_operands(m_sizes, x, w, xt, wt)
+    assert x.ndim == 2 and w.ndim == 3 and xt.ndim == 2 and wt.ndim == 3
+    rows, k = x.shape
+    experts, n, k_w = w.shape
+    r = xt.shape[1]
+    assert k_w == k and m_sizes.numel() == experts and xt.shape[0] == rows and wt.shape == (experts, n, r)
+    y = torch.empty((rows, n), device=x.device, dtype=x.dtype if dtype is None else dtype)
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_gemm_fwd_lora(_lib.ptr(x), _lib.ptr(w), _lib.ptr(xt), _lib.ptr(wt), r, _lib.ptr(ms),
+                                      _lib.itype_code(ms.dtype), _lib.ptr(y), rows, n, k, experts,
+                                      _lib.dtype_code(x.dtype), _lib.dtype_code(y.dtype), _lib.stream())
+    if rc == UNSUPPORTED:
+        grouped_gemm_forward(x, w, m_sizes, dtype, out=y)
+        return grouped_gemm_forward(xt, wt, m_sizes, dtype, out=y, accumulate=True)
+    _lib.check(rc, "mfl_gemm_fwd_lora")
+    return y
+
+
+def grouped_gemm_forward_transposed_lora(dy: torch.Tensor, w: torch.Tensor, xt: torch.Tensor, wt: torch.Tensor,
+                                         m_sizes: torch.Tensor, dtype: Optional[torch.dtype] = None, *,
+                                         dy2: Optional[torch.Tensor] = None,
+                                         w2: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``dy @ w (+ dy2 @ w2) + xt @ wt`` per expert in one kernel: an input gradient with the rank-r term of a
+    LoRA adapter in the same reduction (``xt = s * dy B`` (rows, r), ``wt = A`` (E, r, N)), optionally over
+    both weights of the gated unit (qwen3_moe_fused/kernels/fast_lora.py:127-131,151-152)."""
+    from .forward_transposed import grouped_gemm_forward_transposed
+
+    check_operands(m_sizes, dy, w, xt, wt)
+    assert dy.ndim == 2 and w.ndim == 3 and xt.ndim == 2 and wt.ndim == 3
+    rows, k = dy.shape
+    experts, k_w, n = w.shape
+    r = xt.shape[1]
+    assert k_w == k and m_sizes.numel() == experts and xt.shape[0] == rows and wt.shape == (experts, r, n)
+    assert (dy2 is None) == (w2 is None)
+    if dy2 is not None:
+        check_operands(m_sizes, dy, dy2, w2)
+        assert dy2.shape == dy.shape and w2.shape == w.shape
+    dx = torch.empty((rows, n), device=dy.device, dtype=dy.dtype if dtype is None else dtype)
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_gemm_dx_lora(_lib.ptr(dy), _lib.ptr(w), _lib.ptr(dy2) if dy2 is not None else None,
+                                     _lib.ptr(w2) if w2 is not None else None, _lib.ptr(xt), _lib.ptr(wt), r,
+                                     _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(dx), rows, n, k, experts,
+                                     _lib.dtype_code(dy.dtype), _lib.dtype_code(dx.dtype), _lib.stream())
+    if rc == UNSUPPORTED:
+        if dy2 is None:
+            grouped_gemm_forward_transposed(dy, w, m_sizes, dtype, out=dx)
+        else:
+            dx = grouped_gemm_forward_transposed_dual(dy, w, dy2, w2, m_sizes, dtype)
+        return grouped_gemm_forward_transposed(xt, wt, m_sizes, dtype, out=dx, accumulate=True)
+    _lib.check(rc, "mfl_gemm_dx_lora")
+    return dx

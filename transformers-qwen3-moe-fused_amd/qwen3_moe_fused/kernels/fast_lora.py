@@ -4,7 +4,7 @@
 Shapes (rows B, hidden H, intermediate M, rank r, experts E):
     x (B,H);  G,U (E,M,H);  W (E,H,M);  Ag,Au (E,r,H);  Bg,Bu (E,M,r);  Aw (E,r,M);  Bw (E,H,r)
     e = G x + Sg Bg (Ag x),  g = U x + Su Bu (Au x),  h = silu(e) g,  y = W h + Sw Bw (Aw h)
-Only e, g and the two rank-r activations Ag x, Au x are kept for the backward pass.
+Only e, g and the two rank-r activations Sg Ag x, Su Au x are kept for the backward pass.
 
 Gradients.  With t = dOut Bproj (rows x r) and u = In Aproj^T (rows x r) for a projection
 Out = (Wp + S Bp Ap) In:
@@ -23,7 +23,8 @@ from ..grouped_gemm.forward import grouped_gemm_forward as _fwd
 from ..grouped_gemm.forward_4bit import grouped_gemm_forward_4bit as _fwd4
 from ..grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit as _dx4
 from ..grouped_gemm.forward_transposed import grouped_gemm_forward_transposed as _dx
-from ..grouped_gemm.fused import grouped_gemm_forward_transposed_dual as _dx_dual
+from ..grouped_gemm.fused import grouped_gemm_forward_lora as _fwd_lora
+from ..grouped_gemm.fused import grouped_gemm_forward_transposed_lora as _dx_lora
 from ..quantize.nf4 import dequantize_nf4
 from .silu_mul import silu_mul_backward_inplace, silu_mul_forward
 
@@ -41,19 +42,25 @@ def _dense(wq, wqs, dtype):
 
 
 def _proj_fwd(x, wq, wqs, a, b, s, m_sizes):
+    """y = x W^T + (s x A^T) B^T; returns y and the scaled rank-r activation s x A^T (rows x r)."""
+    us = _fwd(x, a, m_sizes, alpha=s)
+    if wqs is None and x.dtype == torch.bfloat16:
+        # bf16 weights: the rank-r term rides in the reduction of the base product (no second pass over y)
+        return _fwd_lora(x, wq.to(x.dtype), us, b, m_sizes), us
     y = _base_fwd(x, wq, wqs, m_sizes)
-    u = _fwd(x, a, m_sizes)                                   # rows x r
-    _fwd(u, b, m_sizes, out=y, alpha=s, accumulate=True)      # y += s * u b^T
-    return y, u
+    _fwd(us, b, m_sizes, out=y, accumulate=True)             # y += us b^T
+    return y, us
 
 
-def _proj_bwd_input(dout, t, wq, wqs, a, s, m_sizes, out=None):
-    """dIn (+)= dOut W + s * t A."""
+def _proj_bwd_input(dout, ts, wq, wqs, a, m_sizes, out=None):
+    """dIn (+)= dOut W + ts A with ts = s dOut B (rows x r)."""
+    if wqs is None and dout.dtype == torch.bfloat16 and out is None:
+        return _dx_lora(dout, wq.to(dout.dtype), ts, a, m_sizes)
     if wqs is not None and dout.dtype == torch.bfloat16:
         out = _dx4(dout, wq, wqs, m_sizes, out=out, accumulate=out is not None)
     else:
         out = _dx(dout, _dense(wq, wqs, dout.dtype), m_sizes, out=out, accumulate=out is not None)
-    return _dx(t, a, m_sizes, out=out, alpha=s, accumulate=True)
+    return _dx(ts, a, m_sizes, out=out, accumulate=True)
 
 
 class FastLora(torch.autograd.Function):
@@ -77,34 +84,34 @@ class FastLora(torch.autograd.Function):
         dt = x.dtype
         dy = dy.contiguous()
 
+        # The rank-r activations carry the adapter's scaling (ug, uu from the forward pass; tw, tu, tg here),
+        # so every product below takes them as they are.
         # down projection
-        tw = _dx(dy, Bw, m_sizes)                                     # dy Bw, rows x r
-        dh = _proj_bwd_input(dy, tw, Wq, Wqs, Aw, Sw, m_sizes)
+        tw = _dx(dy, Bw, m_sizes, alpha=Sw)                            # Sw dy Bw, rows x r
+        dh = _proj_bwd_input(dy, tw, Wq, Wqs, Aw, m_sizes)
         silu_mul_backward_inplace(dh, e, g)                            # (dh, e, g) <- (h, de, dg)
         h, de, dg = dh, e, g
-        dAw = _dw(h, tw, m_sizes, dt, alpha=Sw)                        # (E, r, M)
-        dBw = _dw(_fwd(h, Aw, m_sizes), dy, m_sizes, dt, alpha=Sw)     # (E, H, r)
+        dAw = _dw(h, tw, m_sizes, dt)                                  # (E, r, M)
+        dBw = _dw(_fwd(h, Aw, m_sizes, alpha=Sw), dy, m_sizes, dt)     # (E, H, r)
 
         # up projection
-        tu = _dx(dg, Bu, m_sizes)
-        dAu = _dw(x, tu, m_sizes, dt, alpha=Su)                        # (E, r, H)
-        dBu = _dw(uu, dg, m_sizes, dt, alpha=Su)                       # (E, M, r)
+        tu = _dx(dg, Bu, m_sizes, alpha=Su)
+        dAu = _dw(x, tu, m_sizes, dt)                                  # (E, r, H)
+        dBu = _dw(uu, dg, m_sizes, dt)                                 # (E, M, r)
 
         # gate projection
-        tg = _dx(de, Bg, m_sizes)
-        dAg = _dw(x, tg, m_sizes, dt, alpha=Sg)
-        dBg = _dw(ug, de, m_sizes, dt, alpha=Sg)
+        tg = _dx(de, Bg, m_sizes, alpha=Sg)
+        dAg = _dw(x, tg, m_sizes, dt)
+        dBg = _dw(ug, de, m_sizes, dt)
 
         dx = None
         if ctx.needs_input_grad[0]:
             if Gqs is None and Uqs is None and dt == torch.bfloat16 and Gq.dtype == dt and Uq.dtype == dt:
-                # both base terms in one reduction, then the two rank-r terms on top
-                dx = _dx_dual(de, Gq, dg, Uq, m_sizes)
-                _dx(tg, Ag, m_sizes, out=dx, alpha=Sg, accumulate=True)
-                _dx(tu, Au, m_sizes, out=dx, alpha=Su, accumulate=True)
+                # both base terms and both rank-r terms (side by side as one term of rank 2 r) in one reduction
+                dx = _dx_lora(de, Gq, torch.cat((tg, tu), dim=1), torch.cat((Ag, Au), dim=1), m_sizes, dy2=dg, w2=Uq)
             else:
-                dx = _proj_bwd_input(de, tg, Gq, Gqs, Ag, Sg, m_sizes)
-                dx = _proj_bwd_input(dg, tu, Uq, Uqs, Au, Su, m_sizes, out=dx)
+                dx = _proj_bwd_input(de, tg, Gq, Gqs, Ag, m_sizes)
+                dx = _proj_bwd_input(dg, tu, Uq, Uqs, Au, m_sizes, out=dx)
 
         return (dx, None, None, dAg, dBg, None, None, None, dAu, dBu, None, None, None, dAw, dBw, None, None)
 
