@@ -133,6 +133,29 @@ def _kernel_tour(n, dev):
                          2 * active * nf4_b / E + 2.0 * tokens * TOPK * (HIDDEN + INTER),
                          4.0 * tokens * TOPK * INTER * HIDDEN,
                          lambda i, x5=x5, ms5=ms5: grouped_glu_forward_4bit(x5, *qsets[i % 3], *qsets[(i + 1) % 3], ms5)))
+    # configuration 4: rank-16 adapter products at 8192 tokens under Zipf(1.2)-skewed routing (65536 rows)
+    from qwen3_moe_fused.grouped_gemm.fused import grouped_gemm_forward_lora
+    T4, R4, RANK = 8192, 8192 * TOPK, 16
+    bias = (torch.randperm(E, device=dev, generator=g).float() + 1).pow(-1.2).log()
+    _, _, s4 = softmax_topk_raw(torch.randn((T4, E), device=dev, generator=g) + bias, TOPK, True, bf)
+    ms4, _, _ = get_expert_counts_and_idx(s4.view(-1), E)
+    x4, dy4 = rnd(R4, HIDDEN), rnd(R4, INTER)
+    t4, u4 = rnd(R4, RANK), rnd(R4, RANK)
+    la, lb = rnd(E, RANK, HIDDEN, scale=0.01), rnd(E, INTER, RANK, scale=0.01)
+    legs += [
+        (f"gemm_dw_split dA (x 65536x2048, rank 16; largest expert {int(ms4.max().item())} rows)",
+         2.0 * (R4 * HIDDEN + R4 * RANK + E * RANK * HIDDEN), 2.0 * R4 * RANK * HIDDEN,
+         lambda i: grouped_gemm_backward_dw(x4, t4, ms4, bf)),
+        ("gemm_dw_split dB (dy 65536x768, rank 16)", 2.0 * (R4 * INTER + R4 * RANK + E * RANK * INTER),
+         2.0 * R4 * RANK * INTER, lambda i: grouped_gemm_backward_dw(u4, dy4, ms4, bf)),
+        ("gemm_fwd thin output x A^T (65536x2048 -> rank 16)", 2.0 * (R4 * HIDDEN + R4 * RANK + E * RANK * HIDDEN),
+         2.0 * R4 * RANK * HIDDEN, lambda i: grouped_gemm_forward(x4, la, ms4)),
+        ("gemm_dx thin output dy B (65536x768 -> rank 16)", 2.0 * (R4 * INTER + R4 * RANK + E * RANK * INTER),
+         2.0 * R4 * RANK * INTER, lambda i: grouped_gemm_forward_transposed(dy4, lb, ms4)),
+        ("gemm_fwd_lora gate_proj + rank-16 term, 65536 rows",
+         2.0 * (R4 * HIDDEN + E * INTER * HIDDEN + R4 * INTER + R4 * RANK + E * INTER * RANK),
+         2.0 * R4 * INTER * (HIDDEN + RANK), lambda i: grouped_gemm_forward_lora(x4, w_gate, u4, lb, ms4)),
+    ]
     for name, nbytes, flops, fn in legs:
         for i in range(n):
             fn(i)
