@@ -140,3 +140,28 @@ def test_backward_dw_wrapper_takes_the_split_kernel_for_lora_shapes():
     base = torch.ones_like(got)
     acc = grouped_gemm_backward_dw(x, t, ms, torch.bfloat16, out=base.clone(), accumulate=True)
     torch.testing.assert_close(acc.float(), ref + 1.0, rtol=2e-2, atol=unit_scale_atol(ref, 2e-2))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_dw_split_random_shapes(seed):
+    gen = torch.Generator().manual_seed(1000 + seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=gen))  # noqa: E731
+    E = ri(1, 200)
+    R = ri(1, 12000)
+    th = (16, 32)[ri(0, 1)]
+    wide = 256 * ri(1, 4)
+    thin_n = bool(ri(0, 1))
+    N, K = (th, wide) if thin_n else (wide, th)
+    kind = ("uniform", "zipf", "one", "tiny")[ri(0, 3)]
+    ms = _sizes(kind, E, R, gen)
+    if ri(0, 3) == 0:                      # rows at the end that belong to no expert
+        ms[ri(0, E - 1)] = 0
+    ms = ms.to((torch.int32, torch.int64)[ri(0, 1)]).cuda()
+    out_dtype = (torch.bfloat16, torch.float32)[ri(0, 1)]
+    x = torch.randn(R, K, generator=gen).to(torch.bfloat16).cuda()
+    dy = torch.randn(R, N, generator=gen).to(torch.bfloat16).cuda()
+    print(f"dw_split seed {seed}: {kind} E={E} R={R} N={N} K={K} {out_dtype} rows in experts {int(ms.sum())}", flush=True)
+    got = _call(x, dy, ms, out_dtype, 1.0)
+    ref = _closed_form(x, dy, ms, 1.0)
+    assert (got[(ms == 0).nonzero().flatten()] == 0).all()
+    torch.testing.assert_close(got.float(), ref, rtol=1e-2, atol=unit_scale_atol(ref, 1e-2))

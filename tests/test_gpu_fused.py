@@ -350,3 +350,27 @@ def test_lora_term_of_other_element_types_runs_as_two_products():
     ref = (oracle.linear_bwd_input(to_np32(dy), to_np32(w), sel).astype(np.float64)
            + oracle.linear_bwd_input(to_np32(xt), to_np32(wa), sel))
     check_close(dx, ref, rtol=1e-4, atol=1e-4, what="fp32 input gradient with a rank-r term")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_lora_term_random_shapes(seed):
+    g = gen(4000 + seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+    E, R = ri(1, 48), ri(1, 3000)
+    N, K, r = 8 * ri(1, 100), 8 * ri(1, 64), 8 * ri(1, 12)
+    x, xt = randn((R, K), g, 1.0, torch.bfloat16), randn((R, r), g, 1.0, torch.bfloat16)
+    w, wt = randn((E, N, K), g, 0.05, torch.bfloat16), randn((E, N, r), g, 0.2, torch.bfloat16)
+    ms = m_sizes_uniform(R, E, g)
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    print(f"lora term seed {seed}: E={E} R={R} N={N} K={K} r={r}", flush=True)
+    y = grouped_gemm_forward_lora(x.to(DEV), w.to(DEV), xt.to(DEV), wt.to(DEV), ms.to(DEV))
+    ref = (oracle.linear_fwd(to_np32(x), to_np32(w), sel).astype(np.float64)
+           + oracle.linear_fwd(to_np32(xt), to_np32(wt), sel))
+    check_close(y, ref, what="forward with a rank-r term vs oracle")
+    # the input gradient of the same layer: dx (R, K) = dy (R, N) @ w[e] + tt (R, r) @ a[e], a (E, r, K)
+    dy, tt = randn((R, N), g, 1.0, torch.bfloat16), randn((R, r), g, 1.0, torch.bfloat16)
+    a = randn((E, r, K), g, 0.2, torch.bfloat16)
+    dx = grouped_gemm_forward_transposed_lora(dy.to(DEV), w.to(DEV), tt.to(DEV), a.to(DEV), ms.to(DEV))
+    ref = (oracle.linear_bwd_input(to_np32(dy), to_np32(w), sel).astype(np.float64)
+           + oracle.linear_bwd_input(to_np32(tt), to_np32(a), sel))
+    check_close(dx, ref, what="input gradient with a rank-r term vs oracle")
