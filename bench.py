@@ -436,8 +436,21 @@ def main() -> int:
         us = _event_us(mlp_step, 10, 5, stream)
         lora["expert_mlp_lora_fwd_bwd"] = {"us": round(us, 1), "tokens_per_s": round(T4 / us * 1e6),
                                            "tflops": round(6 * flop4 / us / 1e6, 1)}  # 3 forward + 3 dX products
+        # the same step over packed NF4 base weights (QLoRA)
+        q_gate, q_up, q_down = (quantize_nf4(w, 64) for w in (ws[0], ws[1], w_down.contiguous()))
+
+        def qlora_step(i):
+            (ag, bg), (au, bu), (aw, bw) = adapters
+            y = fast_lora(x4, *q_gate, ag, bg, 2.0, *q_up, au, bu, 2.0, *q_down, aw, bw, 2.0, ms4)
+            y.backward(dyh)
+            x4.grad = None
+            for a_, b_ in adapters:
+                a_.grad = b_.grad = None
+        us = _event_us(qlora_step, 10, 5, stream)
+        lora["expert_mlp_qlora_nf4_fwd_bwd"] = {"us": round(us, 1), "tokens_per_s": round(T4 / us * 1e6),
+                                                "tflops": round(6 * flop4 / us / 1e6, 1)}
         extra["lora_rank16_zipf_config4"] = lora
-        del x4, dy4, dyh, adapters
+        del x4, dy4, dyh, adapters, q_gate, q_up, q_down
         # config 5: the whole sparse block (router -> top-k -> sort -> gather -> gate/up -> SiLU-mul -> down ->
         # weighted combine) with NF4 experts, forward only, module calls as a user makes them
         from types import SimpleNamespace

@@ -148,6 +148,20 @@ MFL_API int mfl_gemm_dx_lora(const void *dy, const void *w, const void *dy2, con
                      void *dx, int64_t R, int N, int K, int E, int in_dtype, int out_dtype,
                      void *stream);
 
+/* mfl_gemm_fwd_lora / mfl_gemm_dx_lora over packed NF4 base weights (arguments as in mfl_gemm_fwd_nf4 /
+ * mfl_gemm_dx_nf4; the thin term's operands xt, wt are bf16): the QLoRA forms of the same two products
+ * (qwen3_moe_fused/kernels/fast_lora.py:57-63,65-88,127-131 dequantise, multiply and add).  Return
+ * MFL_ERR_UNSUPPORTED, with nothing enqueued, unless the element type is bf16, K % 64 == 0, N % 8 == 0
+ * (dx: N % 32 == 0), KT % 8 == 0, blocksize >= 8, E <= 512 and the pointers are 16-byte aligned. */
+MFL_API int mfl_gemm_fwd_nf4_lora(const void *x, const uint8_t *wq, const float *code16,
+                          const float *absmax, int blocksize, const void *xt, const void *wt, int KT,
+                          const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K,
+                          int E, int in_dtype, int out_dtype, void *stream);
+MFL_API int mfl_gemm_dx_nf4_lora(const void *dy, const uint8_t *wq, const float *code16,
+                         const float *absmax, int blocksize, const void *xt, const void *wt, int KT,
+                         const void *m_sizes, int m_sizes_dtype, void *dx, int64_t R, int N, int K,
+                         int E, int in_dtype, int out_dtype, void *stream);
+
 /* ---- forward products fused with their neighbours in the sparse MLP block ---------
  * The reference names these fusions as future work (modular_qwen3_moe_fused.py:100-101,105).
  * Each call returns MFL_ERR_UNSUPPORTED, with nothing enqueued, for a request the pipelined

@@ -374,3 +374,46 @@ def test_lora_term_random_shapes(seed):
     ref = (oracle.linear_bwd_input(to_np32(dy), to_np32(w), sel).astype(np.float64)
            + oracle.linear_bwd_input(to_np32(tt), to_np32(a), sel))
     check_close(dx, ref, what="input gradient with a rank-r term vs oracle")
+
+
+from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit  # noqa: E402
+from qwen3_moe_fused.grouped_gemm.fused import (grouped_gemm_forward_4bit_lora,  # noqa: E402
+                                                grouped_gemm_forward_transposed_4bit_lora)
+from qwen3_moe_fused.quantize.nf4 import quantize_nf4  # noqa: E402
+
+
+# R, N, K, E, rank, blocksize: the rank-r term in the reduction of a product over packed NF4 weights
+@pytest.mark.parametrize("R,N,K,E,r,bs", [(4096, 768, 2048, 16, 16, 64), (9000, 512, 256, 4, 32, 64),
+                                          (700, 224, 64, 5, 8, 16), (600, 160, 192, 6, 72, 32),
+                                          (300, 72, 128, 3, 24, 64),      # dx: N % 32 != 0 -> two products
+                                          (40, 64, 128, 20, 16, 64)])     # a row or two per expert
+def test_nf4_products_with_lora_term(R, N, K, E, r, bs):
+    g = gen(R + N + r + 7)
+    w = randn((E, N, K), g, 0.05, torch.bfloat16).to(DEV)
+    packed, state = quantize_nf4(w, bs)
+    x, xt = randn((R, K), g, 1.0, torch.bfloat16).to(DEV), randn((R, r), g, 1.0, torch.bfloat16).to(DEV)
+    wt = randn((E, N, r), g, 0.2, torch.bfloat16).to(DEV)
+    ms = m_sizes_uniform(R, E, g).to(DEV)
+    # forward: against the fused NF4 product followed by the accumulated thin product (two roundings instead of
+    # one: a bf16 ulp of the sum apart at most), and against the oracle on the dequantised weights
+    y = grouped_gemm_forward_4bit_lora(x, packed, state, xt, wt, ms)
+    y2 = grouped_gemm_forward_4bit(x, packed, state, ms)
+    grouped_gemm_forward(xt, wt, ms, out=y2, accumulate=True)
+    sel = oracle.sel_from_m_sizes(ms.cpu().numpy())
+    from qwen3_moe_fused.quantize.nf4 import dequantize_nf4
+    wd = to_np32(dequantize_nf4(packed, state, torch.bfloat16))
+    ref = oracle.linear_fwd(to_np32(x), wd, sel).astype(np.float64) + oracle.linear_fwd(to_np32(xt), to_np32(wt), sel)
+    check_close(y, ref, what="NF4 forward with a rank-r term vs oracle")
+    # (two bf16 roundings against one: up to two ulps of the output apart)
+    check_close(y, to_np32(y2), atol=unit_scale_atol(to_np32(y2), 2e-2), what="NF4 forward with a rank-r term vs two products")
+    # input gradient of the same layer: dx (R, K) = dy (R, N) @ W[e] + tt (R, r) @ a[e]
+    dy, tt = randn((R, N), g, 1.0, torch.bfloat16).to(DEV), randn((R, r), g, 1.0, torch.bfloat16).to(DEV)
+    a = randn((E, r, K), g, 0.2, torch.bfloat16).to(DEV)
+    dx = grouped_gemm_forward_transposed_4bit_lora(dy, packed, state, tt, a, ms)
+    ref = (oracle.linear_bwd_input(to_np32(dy), wd, sel).astype(np.float64)
+           + oracle.linear_bwd_input(to_np32(tt), to_np32(a), sel))
+    check_close(dx, ref, what="NF4 input gradient with a rank-r term vs oracle")
+    dx2 = grouped_gemm_forward_transposed_4bit(dy, packed, state, ms)
+    grouped_gemm_forward_transposed(tt, a, ms, out=dx2, accumulate=True)
+    check_close(dx, to_np32(dx2), atol=unit_scale_atol(to_np32(dx2), 2e-2),
+                what="NF4 input gradient with a rank-r term vs two products")

@@ -194,6 +194,49 @@ int mfl_gemm_dx_lora(const void *dy, const void *w, const void *dy2, const void 
                           (hipStream_t)stream, &fu);
 }
 
+namespace {
+
+int check_nf4_lora(const void *a, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                   const void *xt, const void *wt, int KT, const void *m_sizes, int ms_dtype, const void *c, int64_t R,
+                   int N, int K, int E, int in_dtype, int out_dtype) {
+    if (R < 0 || N <= 0 || K <= 0 || E <= 0 || KT <= 0 || R > 0x7fffffff) return MFL_ERR_SHAPE;
+    if (blocksize < 2 || (blocksize & (blocksize - 1)) != 0) return MFL_ERR_SHAPE;
+    if (((int64_t)E * N * K) % blocksize != 0 || ((int64_t)E * N * K) % 2 != 0) return MFL_ERR_SHAPE;
+    if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || !itype_ok(ms_dtype)) return MFL_ERR_DTYPE;
+    if (!wq || !code16 || !absmax || !m_sizes || (R > 0 && (!a || !c || !xt || !wt))) return MFL_ERR_NULL;
+    return MFL_OK;
+}
+
+}  // namespace
+
+int mfl_gemm_fwd_nf4_lora(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                          const void *xt, const void *wt, int KT, const void *m_sizes, int m_sizes_dtype, void *y,
+                          int64_t R, int N, int K, int E, int in_dtype, int out_dtype, void *stream) {
+    int rc = check_nf4_lora(x, wq, code16, absmax, blocksize, xt, wt, KT, m_sizes, m_sizes_dtype, y, R, N, K, E, in_dtype,
+                            out_dtype);
+    if (rc) return rc;
+    if (R == 0) return MFL_OK;
+    if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    GemmFusion fu = {nullptr, 1, 0, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr};
+    fu.xt = xt, fu.wt = wt, fu.kt = KT;
+    return gemm_nf4_pipe(x, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E, out_dtype,
+                         (hipStream_t)stream, &fu);
+}
+
+int mfl_gemm_dx_nf4_lora(const void *dy, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                         const void *xt, const void *wt, int KT, const void *m_sizes, int m_sizes_dtype, void *dx,
+                         int64_t R, int N, int K, int E, int in_dtype, int out_dtype, void *stream) {
+    int rc = check_nf4_lora(dy, wq, code16, absmax, blocksize, xt, wt, KT, m_sizes, m_sizes_dtype, dx, R, N, K, E,
+                            in_dtype, out_dtype);
+    if (rc) return rc;
+    if (R == 0) return MFL_OK;
+    if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    GemmFusion fu = {nullptr, 1, 0, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr};
+    fu.xt = xt, fu.wt = wt, fu.kt = KT;
+    return gemm_nf4_pipe_dx(dy, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, dx, R, N, K, E,
+                            out_dtype, 1.0f, 0, (hipStream_t)stream, &fu);
+}
+
 /* ---- forward products fused with their neighbours in the sparse MLP block ---- */
 
 namespace {

@@ -87,7 +87,7 @@ int gemm_nf4_pipe(const void *x, const uint8_t *wq, const float *code16, const f
 // into LDS like the forward.  Needs K % 64 == 0, N % 32 == 0.
 int gemm_nf4_pipe_dx(const void *dy, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
                      const void *m_sizes, int ms_i64, void *dx, int64_t R, int N, int K, int E, int out_dtype,
-                     float alpha, int accumulate, hipStream_t stream);
+                     float alpha, int accumulate, hipStream_t stream, const GemmFusion *fusion = nullptr);
 
 // bf16 MFMA forward with NF4 weights decoded in the K loop.
 int gemm_nf4_mfma(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,

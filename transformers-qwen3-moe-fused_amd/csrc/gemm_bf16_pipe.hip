@@ -245,7 +245,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                                                                   float alpha, int accumulate, Nf4Params nf4,
                                                                   FwdFusion fu) {
     constexpr bool GLU = FUSE == 1, THIN = FUSE == 2;
-    static_assert(!THIN || (MODE != MODE_DW && !NF4), "the thin last term belongs to the row-grouped bf16 products");
+    static_assert(!THIN || MODE != MODE_DW, "the thin last term belongs to the row-grouped products");
     static_assert(!NF4 || (MODE != MODE_DW && S == 2 && BK == 64), "NF4 weights: row-grouped products, two stages");
     static_assert(!GLU || (MODE == MODE_FWD && WGN % 2 == 0 && sizeof(TO) == 2 && BK == 64),
                   "GLU: forward product, bf16 output, the waves along N split in a gate half and an up half");
@@ -526,9 +526,11 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 const unsigned char *p = r >= k2 ? (const unsigned char *)&g_zero_chunk : at_tile + ((int64_t)i * k2 + r) * 2;
                 copy_to_lds<0, ASM_COPY>(p, st + load * 1024);
             }
+            // (with NF4 weights the other steps fill the weight stage by decoding; this one copies bf16)
+            constexpr int LBT = SB::kWaveLoads / NW;
 #pragma unroll
-            for (int q = 0; q < LB; ++q) {
-                const int load = wave * LB + q;
+            for (int q = 0; q < LBT; ++q) {
+                const int load = wave * LBT + q;
                 const int row = SB::row_of(load, ln);
                 const int c = SB::swz(row, SB::phys_of(load, ln));
                 const unsigned char *p;
@@ -758,18 +760,19 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             Nf4Regs r0, r1;
             if (tid < 16) lut[tid] = nf4.code16[tid];
             if (GLU && tid >= 16 && tid < 32) lut[tid] = fu.nf4_2.code16[tid - 16];
-            if (KT > 0) nf4_load(0, r0);
-            if (KT > 1) nf4_load(1, r1);
+            // steps from KT_thin on (a thin last term) copy bf16 weights: nothing to load or decode for them
+            if (KT_thin > 0) nf4_load(0, r0);
+            if (KT_thin > 1) nf4_load(1, r1);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();  // the code table is in LDS
-            if (KT > 0) nf4_decode(0, r0);
+            if (KT_thin > 0) nf4_decode(0, r0);
             auto step = [&](int kt, Nf4Regs &r_even, Nf4Regs &r_odd) {
                 // on entry: r_odd holds step kt+1 (in flight or landed), r_even is free
                 wait_vmcnt<0>();
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // decoded weights of step kt are written
                 __builtin_amdgcn_s_barrier();
                 if (kt + 1 < KT) issue(kt + 1);
-                if (kt + 2 < KT) nf4_load(kt + 2, r_even);
+                if (kt + 2 < KT_thin) nf4_load(kt + 2, r_even);
                 const unsigned char *sa = smem + (kt % S) * STAGE_BYTES, *sb = sa + SA::kBytes;
                 // The decode of the next step's weights (vector ALU) is spread over the four
                 // sub-steps, so that it runs under this step's matrix instructions instead of
@@ -778,7 +781,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 // (Forcing a finer interleave with scheduling barriers, or one straight-line
                 // variant of the step per case, made the register allocator spill.)
                 static_assert(KS == 4, "one packed dword per sub-step");
-                const bool dec = nf4_on && kt + 1 < KT;
+                const bool dec = nf4_on && kt + 1 < KT_thin;
                 bf16x8 fa[2][TA], fb[2][TN];
 #pragma unroll
                 for (int bj = 0; bj < TN; ++bj) fb[0][bj] = fo_b.load(sb, bj, 0);
@@ -997,7 +1000,7 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
     const bool glu = fu.b2 != nullptr && fu.a2 == nullptr;
     if ((glu || fu.row_idx) && mode != MODE_FWD) return MFL_ERR_UNSUPPORTED;
     if (fu.a2 != nullptr && (mode != MODE_DX || nf4 != nullptr || fu.b2 == nullptr)) return MFL_ERR_UNSUPPORTED;
-    if (fu.at != nullptr && (mode == MODE_DW || nf4 != nullptr || glu || fu.bt == nullptr)) return MFL_ERR_UNSUPPORTED;
+    if (fu.at != nullptr && (mode == MODE_DW || glu || fu.bt == nullptr)) return MFL_ERR_UNSUPPORTED;
 #define MFL_PIPE(MODE, NF4, GLU)                                                                                \
     {                                                                                                           \
         auto kern = gemm_pipe_kernel<MB, NB, BK, S, WGM, WGN, MODE, NF4, GLU, TO>;                              \
@@ -1026,8 +1029,18 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
     } else if (fu.at != nullptr) {
         // MODES bit 4: the configuration is also built with the thin last term
         if constexpr ((MODES & 16) != 0 && (MODES & 3) == 3) {
-            if (mode == MODE_FWD) MFL_PIPE(MODE_FWD, false, 2)
-            else MFL_PIPE(MODE_DX, false, 2)
+            if (nf4 != nullptr) {
+                if constexpr (S == 2 && BK == 64 && NB * 64 <= NT) {
+                    if (mode == MODE_FWD) MFL_PIPE(MODE_FWD, true, 2)
+                    else MFL_PIPE(MODE_DX, true, 2)
+                } else {
+                    return MFL_ERR_UNSUPPORTED;
+                }
+            } else if (mode == MODE_FWD) {
+                MFL_PIPE(MODE_FWD, false, 2)
+            } else {
+                MFL_PIPE(MODE_DX, false, 2)
+            }
         } else {
             return MFL_ERR_UNSUPPORTED;
         }
@@ -1137,7 +1150,7 @@ int make_fusion(const GemmFusion *f, int K, bool nf4, FwdFusion *out) {
         out->idx_div = f->idx_div;
     }
     if (f->xt != nullptr) {
-        if (nf4 || f->wt == nullptr || f->kt < 8 || f->kt % 8 != 0 || !aligned(f->xt, 16) || !aligned(f->wt, 16) ||
+        if (f->wt == nullptr || f->kt < 8 || f->kt % 8 != 0 || !aligned(f->xt, 16) || !aligned(f->wt, 16) ||
             f->row_idx != nullptr || (f->w2 != nullptr && f->x2 == nullptr))
             return MFL_ERR_UNSUPPORTED;
         out->at = f->xt;
@@ -1221,7 +1234,7 @@ int gemm_nf4_pipe(const void *x, const uint8_t *wq, const float *code16, const f
 
 int gemm_nf4_pipe_dx(const void *dy, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
                      const void *m_sizes, int ms_i64, void *dx, int64_t R, int N, int K, int E, int out_dtype,
-                     float alpha, int accumulate, hipStream_t stream) {
+                     float alpha, int accumulate, hipStream_t stream, const GemmFusion *fusion) {
     if (g_pipe_config < 0 || E > kMaxTableExperts) return MFL_ERR_UNSUPPORTED;
     int shift = 0;
     while ((1 << shift) < blocksize) ++shift;
@@ -1229,10 +1242,19 @@ int gemm_nf4_pipe_dx(const void *dy, const uint8_t *wq, const float *code16, con
     if (K % 64 != 0 || N % 32 != 0 || N < 32 || blocksize < 8) return MFL_ERR_UNSUPPORTED;
     if (!aligned(dy, 16) || !aligned(wq, 16) || !aligned(dx, 16)) return MFL_ERR_UNSUPPORTED;
     if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
+    FwdFusion fu;
+    if (fusion != nullptr) {
+        // only the thin last term
+        if (fusion->xt == nullptr || fusion->x2 != nullptr || fusion->w2 != nullptr || fusion->row_idx != nullptr ||
+            accumulate || alpha != 1.0f)
+            return MFL_ERR_UNSUPPORTED;
+        const int rc = make_fusion(fusion, K, true, &fu);
+        if (rc) return rc;
+    }
     if (R <= 0) return MFL_OK;
     const Nf4Params nf4 = {code16, absmax, shift};
-    return dispatch_pipe(MODE_DX, dy, wq, m_sizes, ms_i64, dx, R, N, K, E, out_dtype, alpha, accumulate, &nf4, nullptr,
-                         stream);
+    return dispatch_pipe(MODE_DX, dy, wq, m_sizes, ms_i64, dx, R, N, K, E, out_dtype, alpha, accumulate, &nf4,
+                         fusion ? &fu : nullptr, stream);
 }
 
 }  // namespace mfl

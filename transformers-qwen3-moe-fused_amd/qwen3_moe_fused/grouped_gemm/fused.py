@@ -239,3 +239,58 @@ def grouped_gemm_forward_transposed_lora(dy: torch.Tensor, w: torch.Tensor, xt: 
         return grouped_gemm_forward_transposed(xt, wt, m_sizes, dtype, out=dx, accumulate=True)
     _lib.check(rc, "mfl_gemm_dx_lora")
     return dx
+
+
+def grouped_gemm_forward_4bit_lora(x: torch.Tensor, w_quant: torch.Tensor, w_quant_state, xt: torch.Tensor,
+                                   wt: torch.Tensor, m_sizes: torch.Tensor,
+                                   dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``grouped_gemm_forward_lora`` over NF4 base weights: ``x W^T + xt wt^T`` with ``W`` decoded inside the
+    kernel (the QLoRA forward product; the reference dequantises, multiplies and adds:
+    qwen3_moe_fused/kernels/fast_lora.py:57-63,65-88)."""
+    assert x.is_cuda and x.ndim == 2 and x.is_contiguous() and m_sizes.is_contiguous() and is_int_tensor(m_sizes)
+    rows, k = x.shape
+    code, absmax, blocksize, experts, n = _nf4_args(w_quant, w_quant_state, x, k)
+    r = xt.shape[1]
+    assert m_sizes.numel() == experts and xt.shape == (rows, r) and wt.shape == (experts, n, r)
+    assert xt.is_contiguous() and wt.is_contiguous() and xt.dtype == x.dtype and wt.dtype == x.dtype
+    y = torch.empty((rows, n), device=x.device, dtype=x.dtype if dtype is None else dtype)
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_gemm_fwd_nf4_lora(_lib.ptr(x), _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), blocksize,
+                                          _lib.ptr(xt), _lib.ptr(wt), r, _lib.ptr(ms), _lib.itype_code(ms.dtype),
+                                          _lib.ptr(y), rows, n, k, experts, _lib.dtype_code(x.dtype),
+                                          _lib.dtype_code(y.dtype), _lib.stream())
+    if rc == UNSUPPORTED:
+        y = grouped_gemm_forward_4bit(x, w_quant, w_quant_state, m_sizes, dtype)
+        return grouped_gemm_forward(xt, wt, m_sizes, dtype, out=y, accumulate=True)
+    _lib.check(rc, "mfl_gemm_fwd_nf4_lora")
+    return y
+
+
+def grouped_gemm_forward_transposed_4bit_lora(dy: torch.Tensor, w_quant: torch.Tensor, w_quant_state, xt: torch.Tensor,
+                                              wt: torch.Tensor, m_sizes: torch.Tensor,
+                                              dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``grouped_gemm_forward_transposed_lora`` over NF4 base weights of shape (E, out, in) =
+    ``w_quant_state.shape``: dx (rows, in) = dy (rows, out) @ W[e] + xt (rows, r) @ wt[e], wt (E, r, in)
+    (qwen3_moe_fused/kernels/fast_lora.py:57-63,127-131)."""
+    from .forward_4bit import grouped_gemm_forward_transposed_4bit
+    from .forward_transposed import grouped_gemm_forward_transposed
+
+    assert dy.is_cuda and dy.ndim == 2 and dy.is_contiguous() and m_sizes.is_contiguous() and is_int_tensor(m_sizes)
+    assert w_quant_state.quant_type in ("nf4", "fp4") and is_int_tensor(w_quant) and w_quant.is_contiguous()
+    blocksize = int(w_quant_state.blocksize)
+    code, absmax = w_quant_state.code, resolve_absmax(w_quant_state)
+    experts, k, n = w_quant_state.shape
+    rows, r = dy.shape[0], xt.shape[1]
+    assert dy.shape[1] == k and m_sizes.numel() == experts and xt.shape == (rows, r) and wt.shape == (experts, r, n)
+    assert xt.is_contiguous() and wt.is_contiguous() and xt.dtype == dy.dtype and wt.dtype == dy.dtype
+    dx = torch.empty((rows, n), device=dy.device, dtype=dy.dtype if dtype is None else dtype)
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_gemm_dx_nf4_lora(_lib.ptr(dy), _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), blocksize,
+                                         _lib.ptr(xt), _lib.ptr(wt), r, _lib.ptr(ms), _lib.itype_code(ms.dtype),
+                                         _lib.ptr(dx), rows, n, k, experts, _lib.dtype_code(dy.dtype),
+                                         _lib.dtype_code(dx.dtype), _lib.stream())
+    if rc == UNSUPPORTED:
+        grouped_gemm_forward_transposed_4bit(dy, w_quant, w_quant_state, m_sizes, dtype, out=dx)
+        return grouped_gemm_forward_transposed(xt, wt, m_sizes, dtype, out=dx, accumulate=True)
+    _lib.check(rc, "mfl_gemm_dx_nf4_lora")
+    return dx

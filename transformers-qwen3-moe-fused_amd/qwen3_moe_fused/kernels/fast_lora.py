@@ -23,7 +23,9 @@ from ..grouped_gemm.forward import grouped_gemm_forward as _fwd
 from ..grouped_gemm.forward_4bit import grouped_gemm_forward_4bit as _fwd4
 from ..grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit as _dx4
 from ..grouped_gemm.forward_transposed import grouped_gemm_forward_transposed as _dx
+from ..grouped_gemm.fused import grouped_gemm_forward_4bit_lora as _fwd4_lora
 from ..grouped_gemm.fused import grouped_gemm_forward_lora as _fwd_lora
+from ..grouped_gemm.fused import grouped_gemm_forward_transposed_4bit_lora as _dx4_lora
 from ..grouped_gemm.fused import grouped_gemm_forward_transposed_lora as _dx_lora
 from ..quantize.nf4 import dequantize_nf4
 from .silu_mul import silu_mul_backward_inplace, silu_mul_forward
@@ -47,6 +49,8 @@ def _proj_fwd(x, wq, wqs, a, b, s, m_sizes):
     if wqs is None and x.dtype == torch.bfloat16:
         # bf16 weights: the rank-r term rides in the reduction of the base product (no second pass over y)
         return _fwd_lora(x, wq.to(x.dtype), us, b, m_sizes), us
+    if wqs is not None and x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and int(wqs.blocksize) >= 8:
+        return _fwd4_lora(x, wq, wqs, us, b, m_sizes), us   # the same over packed NF4 weights
     y = _base_fwd(x, wq, wqs, m_sizes)
     _fwd(us, b, m_sizes, out=y, accumulate=True)             # y += us b^T
     return y, us
@@ -56,6 +60,8 @@ def _proj_bwd_input(dout, ts, wq, wqs, a, m_sizes, out=None):
     """dIn (+)= dOut W + ts A with ts = s dOut B (rows x r)."""
     if wqs is None and dout.dtype == torch.bfloat16 and out is None:
         return _dx_lora(dout, wq.to(dout.dtype), ts, a, m_sizes)
+    if wqs is not None and dout.dtype == torch.bfloat16 and out is None:
+        return _dx4_lora(dout, wq, wqs, ts, a, m_sizes)
     if wqs is not None and dout.dtype == torch.bfloat16:
         out = _dx4(dout, wq, wqs, m_sizes, out=out, accumulate=out is not None)
     else:
@@ -110,8 +116,12 @@ class FastLora(torch.autograd.Function):
                 # both base terms and both rank-r terms (side by side as one term of rank 2 r) in one reduction
                 dx = _dx_lora(de, Gq, torch.cat((tg, tu), dim=1), torch.cat((Ag, Au), dim=1), m_sizes, dy2=dg, w2=Uq)
             else:
-                dx = _proj_bwd_input(de, tg, Gq, Gqs, Ag, m_sizes)
-                dx = _proj_bwd_input(dg, tu, Uq, Uqs, Au, m_sizes, out=dx)
+                # both rank-r terms with the first base product, the second base product accumulates
+                dx = _proj_bwd_input(de, torch.cat((tg, tu), dim=1), Gq, Gqs, torch.cat((Ag, Au), dim=1), m_sizes)
+                if Uqs is not None and dt == torch.bfloat16:
+                    _dx4(dg, Uq, Uqs, m_sizes, out=dx, accumulate=True)
+                else:
+                    _dx(dg, _dense(Uq, Uqs, dt), m_sizes, out=dx, accumulate=True)
 
         return (dx, None, None, dAg, dBg, None, None, None, dAu, dBu, None, None, None, dAw, dBw, None, None)
 
