@@ -43,9 +43,10 @@ def _dense(wq, wqs, dtype):
     return wq.to(dtype) if wqs is None else dequantize_nf4(wq, wqs, dtype)
 
 
-def _proj_fwd(x, wq, wqs, a, b, s, m_sizes):
+def _proj_fwd(x, wq, wqs, a, b, s, m_sizes, us=None):
     """y = x W^T + (s x A^T) B^T; returns y and the scaled rank-r activation s x A^T (rows x r)."""
-    us = _fwd(x, a, m_sizes, alpha=s)
+    if us is None:
+        us = _fwd(x, a, m_sizes, alpha=s)
     if wqs is None and x.dtype == torch.bfloat16:
         # bf16 weights: the rank-r term rides in the reduction of the base product (no second pass over y)
         return _fwd_lora(x, wq.to(x.dtype), us, b, m_sizes), us
@@ -69,14 +70,24 @@ def _proj_bwd_input(dout, ts, wq, wqs, a, m_sizes, out=None):
     return _dx(ts, a, m_sizes, out=out, accumulate=True)
 
 
+# from this many rows on, two thin products that stream the same wide operand are run as one of twice the rank
+_WIDE_ROWS = 4096
+
+
 class FastLora(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, Gq, Gqs, Ag, Bg, Sg, Uq, Uqs, Au, Bu, Su, Wq, Wqs, Aw, Bw, Sw, m_sizes):
         dt = x.dtype
         x = x.contiguous()
         Ag, Bg, Au, Bu, Aw, Bw = (p.to(dt).contiguous() for p in (Ag, Bg, Au, Bu, Aw, Bw))
-        e, ug = _proj_fwd(x, Gq, Gqs, Ag, Bg, Sg, m_sizes)
-        g, uu = _proj_fwd(x, Uq, Uqs, Au, Bu, Su, m_sizes)
+        ug = uu = None
+        if Sg == Su and Ag.shape == Au.shape and x.shape[0] >= _WIDE_ROWS:
+            # one pass over x for both adapters' rank-r activations
+            r = Ag.shape[1]
+            ucat = _fwd(x, torch.cat((Ag, Au), dim=1), m_sizes, alpha=Sg)
+            ug, uu = ucat[:, :r].contiguous(), ucat[:, r:].contiguous()
+        e, ug = _proj_fwd(x, Gq, Gqs, Ag, Bg, Sg, m_sizes, ug)
+        g, uu = _proj_fwd(x, Uq, Uqs, Au, Bu, Su, m_sizes, uu)
         h = silu_mul_forward(e, g)
         y, _ = _proj_fwd(h, Wq, Wqs, Aw, Bw, Sw, m_sizes)
         ctx.frozen = (Gq, Gqs, Sg, Uq, Uqs, Su, Wq, Wqs, Sw, m_sizes)
@@ -100,24 +111,29 @@ class FastLora(torch.autograd.Function):
         dAw = _dw(h, tw, m_sizes, dt)                                  # (E, r, M)
         dBw = _dw(_fwd(h, Aw, m_sizes, alpha=Sw), dy, m_sizes, dt)     # (E, H, r)
 
-        # up projection
+        # up and gate projections
         tu = _dx(dg, Bu, m_sizes, alpha=Su)
-        dAu = _dw(x, tu, m_sizes, dt)                                  # (E, r, H)
-        dBu = _dw(uu, dg, m_sizes, dt)                                 # (E, M, r)
-
-        # gate projection
         tg = _dx(de, Bg, m_sizes, alpha=Sg)
-        dAg = _dw(x, tg, m_sizes, dt)
+        tcat = torch.cat((tg, tu), dim=1)
+        if tg.shape == tu.shape and x.shape[0] >= _WIDE_ROWS:
+            # one pass over x for both: (E, 2 r, H)
+            r = tg.shape[1]
+            dAcat = _dw(x, tcat, m_sizes, dt)
+            dAg, dAu = dAcat[:, :r], dAcat[:, r:]
+        else:
+            dAu = _dw(x, tu, m_sizes, dt)                              # (E, r, H)
+            dAg = _dw(x, tg, m_sizes, dt)
+        dBu = _dw(uu, dg, m_sizes, dt)                                 # (E, M, r)
         dBg = _dw(ug, de, m_sizes, dt)
 
         dx = None
         if ctx.needs_input_grad[0]:
             if Gqs is None and Uqs is None and dt == torch.bfloat16 and Gq.dtype == dt and Uq.dtype == dt:
                 # both base terms and both rank-r terms (side by side as one term of rank 2 r) in one reduction
-                dx = _dx_lora(de, Gq, torch.cat((tg, tu), dim=1), torch.cat((Ag, Au), dim=1), m_sizes, dy2=dg, w2=Uq)
+                dx = _dx_lora(de, Gq, tcat, torch.cat((Ag, Au), dim=1), m_sizes, dy2=dg, w2=Uq)
             else:
                 # both rank-r terms with the first base product, the second base product accumulates
-                dx = _proj_bwd_input(de, torch.cat((tg, tu), dim=1), Gq, Gqs, torch.cat((Ag, Au), dim=1), m_sizes)
+                dx = _proj_bwd_input(de, tcat, Gq, Gqs, torch.cat((Ag, Au), dim=1), m_sizes)
                 if Uqs is not None and dt == torch.bfloat16:
                     _dx4(dg, Uq, Uqs, m_sizes, out=dx, accumulate=True)
                 else:
