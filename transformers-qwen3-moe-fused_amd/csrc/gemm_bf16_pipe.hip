@@ -490,8 +490,50 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
         if (active > TM) active = TM;
     };
 
+    // ---- dW, two stages, whole tiles: the tiles of a workgroup form ONE stream of reduction steps.  A tile of dW
+    // has only a handful of steps (rows of the expert / BK), so a pipeline that drains at every tile end and
+    // fills again after the epilogue spends a third of its time doing one or the other.  Here the first step of
+    // the NEXT tile is requested where a step of the current tile would be, at the top of its last step, into the
+    // stage that step frees; the epilogue stages its output in the other stage, the one the last step was read
+    // from.  Only scalars change from tile to tile when every tile is whole (N % BM == 0, K % BN == 0): the
+    // per-lane source offsets of the copies are computed once, which is what keeps the accumulators out of
+    // scratch memory (a second call of the whole set-up with live accumulators spilled 500-760 bytes per lane).
+    constexpr bool XT = MODE == MODE_DW && S == 2 && !NF4 && NW * 32 * ((NB / WGN) * 64 + 16) <= STAGE_BYTES;
+    const bool xt = XT && N % BM == 0 && K % BN == 0 && !(accumulate && sizeof(TO) == 2);
+    int xt_g = 0;             // stage of the current tile's step 0
+    bool xt_fetched = false;  // the current tile's step 0 has been requested already
+    int n_i0 = 0, n_j0 = 0, n_red = 0;
+    const unsigned char *n_a = nullptr, *n_b = nullptr;
+    TO *n_c = nullptr;
+    auto dw_next = [&](int L) {  // coordinates of dW tile L: scalars only
+        const int e = L / per_expert, local = L % per_expert;
+        n_i0 = (local / tiles_n) * BM;
+        n_j0 = (local % tiles_n) * BN;
+        int rb = __builtin_amdgcn_readfirstlane(tab_rows[e]);
+        int re = __builtin_amdgcn_readfirstlane(tab_rows[e + 1]);
+        if ((int64_t)re > R) re = (int)R;
+        if (rb > re) rb = re;
+        n_a = (const unsigned char *)(a + (int64_t)rb * N + n_i0);
+        n_b = (const unsigned char *)(b + (int64_t)rb * K + n_j0);
+        n_c = c + (int64_t)e * N * K;
+        n_red = re - rb;
+    };
+
     for (int L = L_begin + blockIdx.x / kXcd; L < L_end; L += per_xcd) {
-        setup_tile(L);
+        if (XT && xt_fetched) {
+            // set-up of a tile whose first step is on its way: what dw_next computed
+            i0 = n_i0, j0 = n_j0, a_tile = n_a, b_tile = n_b, c_base = n_c, red = n_red;
+            r_begin = 0, r_end = n_red;
+            KT1 = KT = ceil_div(red, BK);
+        } else {
+            setup_tile(L);
+        }
+        // the tile after this one, if its first step is to be requested under this one's last step
+        bool xt_next = false;
+        if (XT && xt && KT > 0 && L + per_xcd < L_end) {
+            dw_next(L + per_xcd);
+            xt_next = n_red > 0;
+        }
 
         // Cache policy of the weight copies in the row-grouped products: a weight is read by exactly
         // one workgroup, so it is fetched non-temporal (bit 1 of the instruction's cache-policy
@@ -548,8 +590,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 copy_to_lds<0, ASM_COPY>(p, st + SA::kBytes + load * 1024);
             }
         };
-        auto issue = [&](int kt) {
-            unsigned char *st = smem + (kt % S) * STAGE_BYTES;
+        // next_tile (XT only): step 0 of the tile after this one, into the stage after this tile's last
+        auto issue = [&](int kt, bool next_tile = false) {
+            unsigned char *st = smem + ((XT ? xt_g + kt : kt) % S) * STAGE_BYTES;
             if constexpr (THIN) {
                 if (kt >= KT_thin) {
                     issue_second(kt - KT_thin, st);
@@ -559,6 +602,13 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             // step of the term that is being reduced (two-term DX: the second term follows the first)
             int ks = kt;
             const unsigned char *a_term = a_tile, *b_term = b_tile;
+            int red = r_end - r_begin;  // shadows the tile's: the reduction length the tail handling goes by
+            if (XT && next_tile) {
+                ks = 0;
+                a_term = n_a;
+                b_term = n_b;
+                red = n_red;
+            }
             if (MODE == MODE_DX && kt >= KT1) {
                 ks = kt - KT1;
                 a_term = a2_tile;
@@ -637,14 +687,16 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[t][bj][r] = 0.f;
 
-        // every store of the previous tile has left, every wave is done with the stages
-        wait_vmcnt<0>();
-        __builtin_amdgcn_s_barrier();
+        if (!(XT && xt_fetched)) {
+            // every store of the previous tile has left, every wave is done with the stages
+            wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();
 
-        // ---- prologue: S-1 steps in flight
+            // ---- prologue: S-1 steps in flight
 #pragma unroll
-        for (int s = 0; s < S - 1; ++s)
-            if (s < KT) issue(s);
+            for (int s = 0; s < S - 1; ++s)
+                if (s < KT) issue(s);
+        }
 
         // ---- reduction loop, instantiated per number of row blocks that are multiplied.  The
         // MFMA operands are swapped (B first): the accumulator of a lane then holds, for output
@@ -657,14 +709,24 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 // step kt has landed for this wave's copies; the barrier extends that to all
                 // waves and tells us everybody finished reading step kt-1, whose stage is
                 // refilled next
-                if (kt + S - 2 < KT)
+                // A tile whose first step was requested under the previous tile: that tile's output stores were
+                // issued after those copies, the memory counter counts down in order of issue, so "at most as
+                // many outstanding as there were stores" means the copies have landed, and the stores' way to
+                // memory is not waited for.
+                constexpr int XT_STORES = TM * (WTN / 16);  // per wave, bf16 output staged through LDS, whole tiles
+                if (XT && XT_STORES < 64 && sizeof(TO) == 2 && !accumulate && xt_fetched && kt == 0)
+                    wait_vmcnt<(XT_STORES < 64 ? XT_STORES : 0)>();
+                else if (kt + S - 2 < KT)
                     wait_vmcnt<(S - 2) * LPW>();
                 else
                     wait_vmcnt<0>();
                 __builtin_amdgcn_s_barrier();
-                if (kt + S - 1 < KT) issue(kt + S - 1);
+                if (kt + S - 1 < KT)
+                    issue(kt + S - 1);
+                else if (XT && xt_next)
+                    issue(KT, true);
 
-                unsigned char *st = smem + (kt % S) * STAGE_BYTES;
+                unsigned char *st = smem + ((XT ? xt_g + kt : kt) % S) * STAGE_BYTES;
                 const unsigned char *sa = st, *sb = st + SA::kBytes;
                 const int ks_lim = MODE == MODE_DW && kt == KT - 1 ? ks_last : KS;
                 // fragments of sub-step ks+1 are fetched while sub-step ks is multiplied
@@ -827,6 +889,13 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
 
         // ---- epilogue
         const int h = lane >> 5, rl = lane & 31;
+        // where the output is staged: the stages are idle, except (XT) the one that receives the next tile's
+        // first step; the other one is the stage the last step was read from
+        unsigned char *const ep_base = smem + (XT && xt_next ? ((xt_g + KT + 1) & 1) * STAGE_BYTES : 0);
+        if (XT) {
+            xt_g = (xt_g + KT) & 1;
+            xt_fetched = xt_next;
+        }
         if constexpr (GLU) {
             // Each wave stages its 32-row block of one product in LDS as bf16; the wave that holds
             // the other product of the same rows and columns does the same; then each of the two
@@ -884,7 +953,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             __builtin_amdgcn_s_barrier();  // all waves are done reading the last stage
             constexpr int ROWB = WTN * 2 + 16;  // padded row, bytes
             constexpr int CPR = WTN / 8;        // 16-byte chunks per row
-            unsigned char *ep = smem + wave * (32 * ROWB);
+            unsigned char *ep = ep_base + wave * (32 * ROWB);
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
                 if (t >= active) continue;
@@ -920,7 +989,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
             constexpr int ROWF = WTN * 4 + 16;  // padded row of floats, bytes
             constexpr int CPR = WTN / 8;        // 16-byte output chunks per row
             static_assert(NW * 32 * ROWF <= S * STAGE_BYTES, "fp32 output staging must fit in the stages");
-            unsigned char *ep = smem + wave * (32 * ROWF);
+            unsigned char *ep = ep_base + wave * (32 * ROWF);
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
                 if (t >= active) continue;
