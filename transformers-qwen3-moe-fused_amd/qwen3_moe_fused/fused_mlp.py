@@ -14,7 +14,7 @@ import torch
 from .grouped_gemm.backward_dw import grouped_gemm_backward_dw
 from .grouped_gemm.fused import (grouped_gemm_forward_transposed_dual, grouped_glu_forward,
                                  grouped_glu_forward_4bit)
-from .kernels.routing import _combine, _gather
+from .kernels.routing import _combine, _gather, _scatter
 from .kernels.silu_mul import silu_mul_backward
 from .grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit
 
@@ -42,7 +42,9 @@ class _GluGathered(torch.autograd.Function):
             dx = grouped_gemm_forward_transposed_dual(de, w_gate, dg, w_up, m_sizes, tokens.dtype)
             d_tokens = _combine(dx, inv_sort_idx, None, tokens.shape[0], ctx.k)
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            xg = _gather(tokens, sort_idx, ctx.k, None)
+            # the replicated, sorted rows again (the forward pass never wrote them), from the source's side: every
+            # token row is read once and written k times
+            xg = _scatter(tokens, inv_sort_idx, ctx.k, None) if ctx.k > 1 else _gather(tokens, sort_idx, ctx.k, None)
             if ctx.needs_input_grad[1]:
                 d_gate = grouped_gemm_backward_dw(xg, de, m_sizes, w_gate.dtype)
             if ctx.needs_input_grad[2]:
