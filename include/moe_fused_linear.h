@@ -233,6 +233,16 @@ MFL_API int mfl_route_softmax_topk(const void *logits, int logits_dtype, int64_t
                            int renorm, float *weights_f32, void *weights_cast, int cast_dtype,
                            int64_t *idx, void *stream);
 
+/* Gradient of mfl_route_softmax_topk's weights with respect to the logits: dlogits (T,E), in the
+ * logits' type, from dweights (T,k) of dweights_dtype, the selections idx and the fp32 weights
+ * that the forward call wrote; the softmax is recomputed.  E <= 1024.  It is the derivative that
+ * autograd forms for qwen3_moe_fused/modular_qwen3_moe_fused.py:87-93 (softmax, topk, the
+ * optional renormalisation) from separate tensor operations. */
+MFL_API int mfl_route_softmax_topk_bwd(const void *logits, int logits_dtype, int64_t T, int E, int k,
+                               int renorm, const int64_t *idx, const float *weights_f32,
+                               const void *dweights, int dweights_dtype, void *dlogits,
+                               void *stream);
+
 /* mfl_route_softmax_topk followed by mfl_expert_sort of its T * k selections, as ONE launch
  * for decode-sized batches (the three launches of the separate calls cost more than their
  * work there).  Same outputs, bit for bit: weights_f32 / weights_cast / idx as in

@@ -269,3 +269,44 @@ def test_one_launch_entry_point_up_to_its_own_limit(T, E, k):
                                          _lib.ptr(inv), _lib.stream())
     _lib.check(rc, "mfl_route_sort_small")
     _check_route_outputs(logits, k, E, w, sel, m_sizes, sort_idx, inv)
+
+
+@pytest.mark.parametrize("dw_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("renorm", [True, False])
+@pytest.mark.parametrize("T,E,k", [(37, 8, 2), (4096, 128, 8), (5, 1000, 64), (64, 130, 3), (1, 64, 1)])
+def test_routing_weight_gradient_matches_autograd_in_fp64(T, E, k, renorm, dw_dtype):
+    """d logits of the routing weights (one kernel) against autograd of the textbook composition
+    softmax -> topk -> renormalise (modular_qwen3_moe_fused.py:87-93) in fp64."""
+    g = gen(T + E + k)
+    logits = randn((T, E), g)
+    dw = randn((T, k), g).to(dw_dtype)
+    ld = logits.to(DEV).requires_grad_()
+    w, idx = softmax_topk(ld, k, renorm, torch.float32)
+    (w * dw.to(DEV).float()).sum().backward()
+    l64 = logits.double().requires_grad_()
+    p = torch.softmax(l64, dim=-1)
+    w64 = p.gather(1, idx.cpu())              # the same selections: the gradient of the weights, not of the choice
+    if renorm:
+        w64 = w64 / w64.sum(dim=-1, keepdim=True)
+    (w64 * dw.double()).sum().backward()
+    ref = l64.grad.numpy()
+    check_close(ld.grad, ref, rtol=1e-4, atol=1e-6 * max(1.0, float(np.abs(ref).max())), what="d logits")
+    assert ld.grad.dtype == torch.float32
+
+
+def test_routing_weight_gradient_bf16_logits_through_route_and_sort():
+    from qwen3_moe_fused.kernels.routing import route_and_sort
+    g = gen(91)
+    T, E, k = 300, 128, 8
+    logits = randn((T, E), g).bfloat16()
+    dw = randn((T, k), g).bfloat16()
+    ld = logits.to(DEV).requires_grad_()
+    w, idx, *_ = route_and_sort(ld, k, True, torch.bfloat16, E)
+    (w.float() * dw.to(DEV).float()).sum().backward()
+    l64 = logits.double().requires_grad_()
+    p = torch.softmax(l64, dim=-1)
+    w64 = p.gather(1, idx.cpu())
+    w64 = w64 / w64.sum(dim=-1, keepdim=True)
+    (w64 * dw.double()).sum().backward()
+    assert ld.grad.dtype == torch.bfloat16
+    check_close(ld.grad, l64.grad.numpy(), rtol=1e-2, atol=1e-2 * float(l64.grad.abs().max()), what="d logits (bf16)")

@@ -355,6 +355,16 @@ int mfl_route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int 
                               weights_cast ? cast_dtype : MFL_F32, idx, (hipStream_t)stream);
 }
 
+int mfl_route_softmax_topk_bwd(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm,
+                               const int64_t *idx, const float *weights_f32, const void *dweights, int dweights_dtype,
+                               void *dlogits, void *stream) {
+    if (T < 0 || E <= 0 || k <= 0 || k > E || k > 64) return MFL_ERR_SHAPE;
+    if (!dtype_ok(logits_dtype) || !dtype_ok(dweights_dtype)) return MFL_ERR_DTYPE;
+    if (T > 0 && (!logits || !idx || !weights_f32 || !dweights || !dlogits)) return MFL_ERR_NULL;
+    return route_softmax_topk_bwd(logits, logits_dtype, T, E, k, renorm, idx, weights_f32, dweights, dweights_dtype,
+                                  dlogits, (hipStream_t)stream);
+}
+
 int mfl_route_sort_small(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, float *weights_f32,
                          void *weights_cast, int cast_dtype, int64_t *idx, int32_t *counts, int32_t *sort_idx,
                          int32_t *inv_sort_idx, void *stream) {

@@ -24,6 +24,9 @@ int nf4_quant(const void *w, int w_dtype, int64_t n, int blocksize, const float 
 
 int route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, float *w_f32,
                        void *w_cast, int cast_dtype, int64_t *idx, hipStream_t stream);
+// d logits of the routing weights (recomputes the softmax; idx and w_f32 as route_softmax_topk wrote them)
+int route_softmax_topk_bwd(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, const int64_t *idx,
+                           const float *w_f32, const void *dw, int dw_dtype, void *dlogits, hipStream_t stream);
 int route_sort_small(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, float *w_f32,
                      void *w_cast, int cast_dtype, int64_t *idx, int32_t *counts, int32_t *sort_idx,
                      int32_t *inv_sort_idx, hipStream_t stream);

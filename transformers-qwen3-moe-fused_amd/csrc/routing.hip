@@ -147,6 +147,107 @@ int launch_topk(const void *logits, int64_t T, int E, int k, int renorm, float *
     return launch_status();
 }
 
+// Gradient of the routing weights with respect to the logits: a wave per token recomputes the softmax, spreads the
+// k incoming gradients over the selected experts and applies the softmax Jacobian:
+//   renorm:  w_j = p_sel_j / s, s = sum_j p_sel_j   ->   dp_sel_j = (dw_j - sum_i dw_i w_i) / s
+//   dlogits_e = p_e (dp_e - sum_j dp_sel_j p_sel_j),  dp_e = dp_sel_j where e is the j-th selection, else 0
+// (the derivative of modular_qwen3_moe_fused.py:87-93 that autograd forms there from five tensor operations).
+template <typename TI, typename TG, int VPL>
+__global__ __launch_bounds__(256) void softmax_topk_bwd_kernel(const TI *__restrict__ logits, int64_t T, int E, int k,
+                                                               int renorm, const int64_t *__restrict__ idx,
+                                                               const float *__restrict__ w_f32,
+                                                               const TG *__restrict__ dw, TI *__restrict__ dlogits) {
+    const int lane = threadIdx.x & 63;
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= T) return;
+    const TI *row = logits + t * E;
+    float p[VPL];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+        const int e = lane + 64 * v;
+        p[v] = e < E ? to_f32(row[e]) : -INFINITY;
+        mx = fmaxf(mx, p[v]);
+    }
+    mx = wave_max_f32(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+        const int e = lane + 64 * v;
+        p[v] = e < E ? expf(p[v] - mx) : 0.f;
+        sum += p[v];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) p[v] = p[v] / sum;
+
+    // lane j < k: the j-th selection, its probability, weight and incoming gradient
+    const int my_i = lane < k ? (int)idx[t * k + lane] : 0;
+    const float my_w = lane < k ? w_f32[t * k + lane] : 0.f;
+    float my_g = lane < k ? to_f32(dw[t * k + lane]) : 0.f;
+    float my_p = 0.f, s = 0.f;
+    for (int j = 0; j < k; ++j) {
+        const int ij = __builtin_amdgcn_readlane(my_i, j);
+        float pv = 0.f;
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            if ((ij >> 6) == v) pv = p[v];
+        const float pj = __shfl(pv, ij & 63);
+        if (lane == j) my_p = pj;
+        s += pj;
+    }
+    if (renorm) {
+        float c = my_g * my_w;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
+        my_g = (my_g - c) / s;
+    }
+    float tsum = lane < k ? my_g * my_p : 0.f;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) tsum += __shfl_xor(tsum, off);
+    float dp[VPL];
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) dp[v] = 0.f;
+    for (int j = 0; j < k; ++j) {
+        const int ij = __builtin_amdgcn_readlane(my_i, j);
+        const float gj = __shfl(my_g, j);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            if (ij == lane + 64 * v) dp[v] += gj;
+    }
+    TI *out = dlogits + t * E;
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+        const int e = lane + 64 * v;
+        if (e < E) out[e] = from_f32<TI>(p[v] * (dp[v] - tsum));
+    }
+}
+
+template <typename TI, typename TG>
+int launch_topk_bwd(const void *logits, int64_t T, int E, int k, int renorm, const int64_t *idx, const float *w_f32,
+                    const void *dw, void *dlogits, hipStream_t stream) {
+    const unsigned grid = (unsigned)((T + 3) / 4);
+    const int vpl = ceil_div(E, 64);
+#define MFL_TOPKB(V)                                                                                          \
+    softmax_topk_bwd_kernel<TI, TG, V><<<grid, 256, 0, stream>>>((const TI *)logits, T, E, k, renorm, idx, w_f32, \
+                                                                 (const TG *)dw, (TI *)dlogits)
+    if (vpl <= 1)
+        MFL_TOPKB(1);
+    else if (vpl <= 2)
+        MFL_TOPKB(2);
+    else if (vpl <= 4)
+        MFL_TOPKB(4);
+    else if (vpl <= 8)
+        MFL_TOPKB(8);
+    else if (vpl <= 16)
+        MFL_TOPKB(16);
+    else
+        return MFL_ERR_UNSUPPORTED;
+#undef MFL_TOPKB
+    return launch_status();
+}
+
 // ---------------------------------------------------------------- stable counting sort
 
 constexpr int kSortMaxE = 4096;
@@ -731,6 +832,15 @@ int route_softmax_topk(const void *logits, int logits_dtype, int64_t T, int E, i
     int rc = MFL_ERR_DTYPE;
     MFL_DISPATCH_FLOAT(logits_dtype, TI, MFL_DISPATCH_FLOAT(cast_dtype, TC, rc = (launch_topk<TI, TC>(
         logits, T, E, k, renorm, w_f32, w_cast, idx, stream))));
+    return rc;
+}
+
+int route_softmax_topk_bwd(const void *logits, int logits_dtype, int64_t T, int E, int k, int renorm, const int64_t *idx,
+                           const float *w_f32, const void *dw, int dw_dtype, void *dlogits, hipStream_t stream) {
+    if (T == 0) return MFL_OK;
+    int rc = MFL_ERR_DTYPE;
+    MFL_DISPATCH_FLOAT(logits_dtype, TI, MFL_DISPATCH_FLOAT(dw_dtype, TG, rc = (launch_topk_bwd<TI, TG>(
+        logits, T, E, k, renorm, idx, w_f32, dw, dlogits, stream))));
     return rc;
 }
 

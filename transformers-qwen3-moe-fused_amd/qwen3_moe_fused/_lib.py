@@ -50,6 +50,7 @@ _SIGNATURES = {
     "mfl_dequant_blockwise_u8": (_i, [_vp, _vp, _vp, _i, _f, _vp, _i64, _vp]),
     "mfl_nf4_quant": (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _vp]),
     "mfl_route_softmax_topk": (_i, [_vp, _i, _i64, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
+    "mfl_route_softmax_topk_bwd": (_i, [_vp, _i, _i64, _i, _i, _i, _vp, _vp, _vp, _i, _vp, _vp]),
     "mfl_route_sort_small": (_i, [_vp, _i, _i64, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "mfl_route_sort_workspace": (_sz, [_i64, _i, _i]),
     "mfl_route_sort": (_i, [_vp, _i, _i64, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),

@@ -51,6 +51,17 @@ class _SoftmaxTopk(torch.autograd.Function):
 
 
 def _softmax_topk_backward(logits, idx, w32, renorm, dw):
+    T, E = logits.shape
+    k = idx.shape[1]
+    if logits.is_cuda and E <= 1024 and k <= 64 and dw.dtype in (torch.float32, torch.bfloat16, torch.float16):
+        # one kernel: a wave per token recomputes the softmax and applies both Jacobians
+        dw = dw.contiguous()
+        dlogits = torch.empty_like(logits)
+        rc = _lib.lib().mfl_route_softmax_topk_bwd(_lib.ptr(logits), _lib.dtype_code(logits.dtype), T, E, k,
+                                                   int(bool(renorm)), _lib.ptr(idx), _lib.ptr(w32), _lib.ptr(dw),
+                                                   _lib.dtype_code(dw.dtype), _lib.ptr(dlogits), _lib.stream())
+        _lib.check(rc, "mfl_route_softmax_topk_bwd")
+        return dlogits
     dw = dw.float()
     p = torch.softmax(logits.float(), dim=-1)
     if renorm:
