@@ -3,7 +3,7 @@
 //   dw[e, n, k] = alpha * sum_{m in expert e} dy[m, n] * x[m, k]
 //   (qwen3_moe_fused/grouped_gemm/backward_dw.py:64-89)
 //
-// with N or K equal to 16 or 32 -- the rank of a LoRA adapter (qwen3_moe_fused/lora.py:71-72), i.e. the
+// with N or K equal to 16, 32 or 64 -- the rank of a LoRA adapter (qwen3_moe_fused/lora.py:71-72), i.e. the
 // products dA and dB of qwen3_moe_fused/kernels/fast_lora.py:121-125,139-149 -- and the other side a multiple
 // of 256.  Such a product does nothing but stream its wide operand once, and a tile per (expert, slice) as in
 // the general kernel makes the expert with the most rows the last to finish, however the tiles are dealt:
@@ -22,8 +22,8 @@
 //     step of the expert before it (chunk 0 for experts with no rows before them).
 // Both operands have the reduction index as their slow one, so both go to LDS as they lie in memory (copies
 // that bypass the registers, a ring of stages) and are read with transposing reads (ds_read_b64_tr_b16) into
-// v_mfma_f32_32x32x16_bf16 fragments: the thin operand is the first MFMA operand (its 16 or 32 values index the
-// accumulator registers), the 32 columns of a block of the wide operand the second (they index the lanes).
+// v_mfma_f32_32x32x16_bf16 fragments: the thin operand is the first MFMA operand (16 or 32 of its values index the
+// accumulator registers of a block; rank 64 is two blocks), the 32 columns of a block of the wide operand the second (they index the lanes).
 // Rows of a step past the end of the expert are copied from a block of zeros.
 #include <type_traits>
 
@@ -53,7 +53,9 @@ constexpr int kSplitMaxExperts = 512;
 constexpr int kMinStepsPerChunk = 8;
 
 constexpr int split_stage_bytes(int th) { return kWideStageBytes + kStepRows * th * 2; }
-constexpr int split_lds_bytes(int th) { return kSplitStages * split_stage_bytes(th) + 2 * (kSplitMaxExperts + 1) * 4; }
+// rank 64: three stages, so that two workgroups still fit in a compute unit's LDS
+constexpr int split_stages(int th) { return th == 64 ? 3 : kSplitStages; }
+constexpr int split_lds_bytes(int th) { return split_stages(th) * split_stage_bytes(th) + 2 * (kSplitMaxExperts + 1) * 4; }
 
 __device__ uint4_t g_split_zeros = {0u, 0u, 0u, 0u};
 
@@ -95,11 +97,14 @@ __global__ __launch_bounds__(kSplitThreads) void dw_split_kernel(const bf16_t *_
                                                                  TO *__restrict__ out, float *__restrict__ partial,
                                                                  int4 *__restrict__ plan, int64_t R, int WIDE, int E,
                                                                  int chunks, float alpha) {
-    static_assert(TH == 16 || TH == 32, "one MFMA block of thin values");
+    static_assert(TH == 16 || TH == 32 || TH == 64, "one or two MFMA blocks of thin values");
+    constexpr int TB = TH == 64 ? 2 : 1;  // thin blocks of 32
+    constexpr int THB = TH / TB;          // thin values per block
     constexpr int STAGE = split_stage_bytes(TH);
+    constexpr int STAGES = split_stages(TH);
     constexpr int THIN_ROW = TH * 2;
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    int *tab_rows = (int *)(smem + kSplitStages * STAGE);
+    int *tab_rows = (int *)(smem + STAGES * STAGE);
     int *tab_steps = tab_rows + (kSplitMaxExperts + 1);
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -238,7 +243,7 @@ __global__ __launch_bounds__(kSplitThreads) void dw_split_kernel(const bf16_t *_
     // ---- per-lane offsets of the fragment reads
     const int g = lane >> 4, il = lane & 15;
     const int fr = 8 * (g >> 1) + (il >> 2);
-    const int thin_off = fr * THIN_ROW + ((16 * (g & 1) + 4 * (il & 3)) % TH) * 2;
+    const int thin_off = fr * THIN_ROW + ((16 * (g & 1) + 4 * (il & 3)) % THB) * 2;  // block tb: + 64 bytes
     int wide_off[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -246,11 +251,13 @@ __global__ __launch_bounds__(kSplitThreads) void dw_split_kernel(const bf16_t *_
         wide_off[t] = fr * kWideRowBytes + (((i >> 3) ^ ((fr & 3) << 2)) * 16) + (i & 7) * 2;
     }
 
-    floatx16 acc[2];
+    floatx16 acc[2][TB];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+        for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][tb][r] = 0.f;
 
     const int h = lane >> 5;
     auto store_block = [&](auto *dst, float scale) {
@@ -259,21 +266,25 @@ __global__ __launch_bounds__(kSplitThreads) void dw_split_kernel(const bf16_t *_
         for (int t = 0; t < 2; ++t) {
             const int j = col0 + (2 * wave + t) * 32 + (lane & 31);
 #pragma unroll
-            for (int gg = 0; gg < TH / 8; ++gg) {
-                const int i0 = 8 * gg + 4 * h;
-                if (THIN_N) {
+            for (int tb = 0; tb < TB; ++tb) {
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) dst[(int64_t)(i0 + u) * WIDE + j] = (T)(acc[t][4 * gg + u] * scale);
-                } else {
-                    typedef T vec4 __attribute__((ext_vector_type(4)));
-                    vec4 v;
+                for (int gg = 0; gg < THB / 8; ++gg) {
+                    const int i0 = 32 * tb + 8 * gg + 4 * h;
+                    if (THIN_N) {
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) v[u] = (T)(acc[t][4 * gg + u] * scale);
-                    *(vec4 *)(dst + (int64_t)j * TH + i0) = v;
+                        for (int u = 0; u < 4; ++u)
+                            dst[(int64_t)(i0 + u) * WIDE + j] = (T)(acc[t][tb][4 * gg + u] * scale);
+                    } else {
+                        typedef T vec4 __attribute__((ext_vector_type(4)));
+                        vec4 v;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) v[u] = (T)(acc[t][tb][4 * gg + u] * scale);
+                        *(vec4 *)(dst + (int64_t)j * TH + i0) = v;
+                    }
                 }
-            }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+                for (int r = 0; r < 16; ++r) acc[t][tb][r] = 0.f;
+            }
         }
     };
     auto flush = [&](int e) {
@@ -285,9 +296,9 @@ __global__ __launch_bounds__(kSplitThreads) void dw_split_kernel(const bf16_t *_
             store_block(partial + (int64_t)split_slot(chunk, spc, sb) * mat, 1.0f);
     };
 
-    // ---- ring of stages: kSplitStages - 1 steps in flight
+    // ---- ring of stages: STAGES - 1 steps in flight
 #pragma unroll
-    for (int s = 0; s < kSplitStages - 1; ++s)
+    for (int s = 0; s < STAGES - 1; ++s)
         if (s < KT) {
             issue(ci, s);
             advance(ci);
@@ -295,23 +306,27 @@ __global__ __launch_bounds__(kSplitThreads) void dw_split_kernel(const bf16_t *_
     for (int kt = 0; kt < KT; ++kt) {
         // this wave's copies of step kt have landed; the barrier extends that to all waves and says that
         // everybody is done with step kt - 1, whose stage is filled next
-        if (kt + kSplitStages - 2 < KT)
-            split_wait_vmcnt<(kSplitStages - 2) * kCopiesPerWave>();
+        if (kt + STAGES - 2 < KT)
+            split_wait_vmcnt<(STAGES - 2) * kCopiesPerWave>();
         else
             split_wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
-        if (kt + kSplitStages - 1 < KT) {
-            issue(ci, (kt + kSplitStages - 1) % kSplitStages);
+        if (kt + STAGES - 1 < KT) {
+            issue(ci, (kt + STAGES - 1) % STAGES);
             advance(ci);
         }
-        const unsigned char *sw = smem + (kt % kSplitStages) * STAGE, *stn = sw + kWideStageBytes;
+        const unsigned char *sw = smem + (kt % STAGES) * STAGE, *stn = sw + kWideStageBytes;
 #pragma unroll
         for (int ks = 0; ks < kStepRows / 16; ++ks) {
-            const bf16x8 tf = split_tr_fragment(stn + thin_off + ks * 16 * THIN_ROW, THIN_ROW);
+            bf16x8 tf[TB];
+#pragma unroll
+            for (int tb = 0; tb < TB; ++tb) tf[tb] = split_tr_fragment(stn + thin_off + tb * 64 + ks * 16 * THIN_ROW, THIN_ROW);
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 const bf16x8 wf = split_tr_fragment(sw + wide_off[t] + ks * 16 * kWideRowBytes, kWideRowBytes);
-                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf, wf, acc[t], 0, 0, 0);
+#pragma unroll
+                for (int tb = 0; tb < TB; ++tb)
+                    acc[t][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf[tb], wf, acc[t][tb], 0, 0, 0);
             }
         }
         if (cc.b + 1 == cc.nb || kt == KT - 1) flush(cc.e);
@@ -357,8 +372,8 @@ int split_chunks(int64_t R, int wide) {
 
 bool split_shape_ok(int64_t R, int N, int K, int E) {
     if (R <= 0 || R > 0x7fffffff || E <= 0 || E > kSplitMaxExperts) return false;
-    const bool thin_n = N == 16 || N == 32;
-    const bool thin_k = K == 16 || K == 32;
+    const bool thin_n = N == 16 || N == 32 || N == 64;
+    const bool thin_k = K == 16 || K == 32 || K == 64;
     if (thin_n == thin_k) return false;
     const int wide = thin_n ? K : N;
     return wide % kSliceCols == 0 && wide / kSliceCols <= 256;
@@ -389,7 +404,7 @@ int launch_split(const bf16_t *thin, const bf16_t *wide_p, const void *m_sizes, 
 
 size_t gemm_dw_split_workspace(int64_t R, int N, int K, int E) {
     if (!split_shape_ok(R, N, K, E)) return 0;
-    const bool thin_n = N == 16 || N == 32;
+    const bool thin_n = N == 16 || N == 32 || N == 64;
     const int wide = thin_n ? K : N, th = thin_n ? N : K;
     // two partial sums and one border entry per chunk
     return (size_t)split_chunks(R, wide) * (2 * (size_t)th * wide * sizeof(float) + sizeof(int4));
@@ -401,7 +416,7 @@ int gemm_dw_split(const void *dy, const void *x, const void *m_sizes, int ms_i64
     if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
     if (!aligned(dy, 16) || !aligned(x, 16) || !aligned(dw, 16) || !aligned(workspace, 16)) return MFL_ERR_ALIGN;
     if (!workspace || ws_bytes < gemm_dw_split_workspace(R, N, K, E)) return MFL_ERR_WORKSPACE;
-    const bool thin_n = N == 16 || N == 32;
+    const bool thin_n = N == 16 || N == 32 || N == 64;
     const int wide = thin_n ? K : N, th = thin_n ? N : K;
     const bf16_t *thin_p = (const bf16_t *)(thin_n ? dy : x), *wide_p = (const bf16_t *)(thin_n ? x : dy);
     const int chunks = split_chunks(R, wide);
@@ -411,8 +426,8 @@ int gemm_dw_split(const void *dy, const void *x, const void *m_sizes, int ms_i64
                                                            wide, E, chunks, alpha, stream)                            \
                            : launch_split<TH_, TN_, float>(thin_p, wide_p, m_sizes, ms_i64, (float *)dw, partial, R,   \
                                                           wide, E, chunks, alpha, stream))
-    if (thin_n) return th == 16 ? MFL_SPLIT(16, true) : MFL_SPLIT(32, true);
-    return th == 16 ? MFL_SPLIT(16, false) : MFL_SPLIT(32, false);
+    if (thin_n) return th == 16 ? MFL_SPLIT(16, true) : th == 32 ? MFL_SPLIT(32, true) : MFL_SPLIT(64, true);
+    return th == 16 ? MFL_SPLIT(16, false) : th == 32 ? MFL_SPLIT(32, false) : MFL_SPLIT(64, false);
 #undef MFL_SPLIT
 }
 

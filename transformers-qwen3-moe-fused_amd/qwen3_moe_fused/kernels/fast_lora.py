@@ -115,7 +115,7 @@ class FastLora(torch.autograd.Function):
         tu = _dx(dg, Bu, m_sizes, alpha=Su)
         tg = _dx(de, Bg, m_sizes, alpha=Sg)
         tcat = torch.cat((tg, tu), dim=1)
-        if tg.shape == tu.shape and x.shape[0] >= _WIDE_ROWS:
+        if tg.shape == tu.shape and x.shape[0] >= _WIDE_ROWS and 2 * tg.shape[1] <= 64:
             # one pass over x for both: (E, 2 r, H)
             r = tg.shape[1]
             dAcat = _dw(x, tcat, m_sizes, dt)
