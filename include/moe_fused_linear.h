@@ -85,7 +85,7 @@ MFL_API int mfl_gemm_dw(const void *x, const void *dy, const void *m_sizes, int 
                 int64_t R, int N, int K, int E, int in_dtype, int out_dtype, float alpha,
                 int accumulate, void *stream);
 
-/* mfl_gemm_dw for a product with one thin side -- N or K equal to 16, 32 or 64 (the rank of a LoRA adapter,
+/* mfl_gemm_dw for a product with one thin side -- N or K equal to 8, 16, 32 or 64 (the rank of a LoRA adapter,
  * qwen3_moe_fused/lora.py:71-72: the products dA and dB of qwen3_moe_fused/kernels/fast_lora.py:121-125,
  * 139-149), the other side a multiple of 256, bf16 operands, bf16 or fp32 result, at most 512 experts.
  * The rows are dealt out evenly over the workgroups whatever the sizes of the experts; an expert cut by

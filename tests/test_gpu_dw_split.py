@@ -70,6 +70,8 @@ CASES = [
     ("uniform", 512, 30000, 16, 768, torch.int32, torch.bfloat16, 1.0),    # the most experts the entry takes
     ("zipf", 48, 15000, 64, 1024, torch.int32, torch.bfloat16, 1.0),       # rank 64: two blocks of thin values
     ("tiny", 70, 6000, 512, 64, torch.int64, torch.float32, 0.25),
+    ("zipf", 20, 7000, 8, 512, torch.int32, torch.bfloat16, 1.0),          # rank 8
+    ("uniform", 9, 5000, 256, 8, torch.int32, torch.bfloat16, 2.0),
 ]
 
 
@@ -150,7 +152,7 @@ def test_dw_split_random_shapes(seed):
     ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=gen))  # noqa: E731
     E = ri(1, 200)
     R = ri(1, 12000)
-    th = (16, 32, 64)[ri(0, 2)]
+    th = (8, 16, 32, 64)[ri(0, 3)]
     wide = 256 * ri(1, 4)
     thin_n = bool(ri(0, 1))
     N, K = (th, wide) if thin_n else (wide, th)

@@ -42,7 +42,7 @@ int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, 
                    int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream,
                    const GemmFusion *fusion = nullptr);
 
-// The weight-gradient product with one thin side (N or K equal to 16, 32 or 64, the other a multiple of 256; bf16 in,
+// The weight-gradient product with one thin side (N or K equal to 8, 16, 32 or 64, the other a multiple of 256; bf16 in,
 // bf16 or fp32 out): steps of 32 rows dealt out evenly over the workgroups, experts cut by a border finished by
 // a second kernel from fp32 partial sums in the workspace.  Takes (a = dy, b = x) like the other kernels.
 // gemm_dw_split_workspace returns 0 for a shape the kernel does not take (gemm_dw_split then returns

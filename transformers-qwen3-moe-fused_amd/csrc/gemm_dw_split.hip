@@ -3,7 +3,7 @@
 //   dw[e, n, k] = alpha * sum_{m in expert e} dy[m, n] * x[m, k]
 //   (qwen3_moe_fused/grouped_gemm/backward_dw.py:64-89)
 //
-// with N or K equal to 16, 32 or 64 -- the rank of a LoRA adapter (qwen3_moe_fused/lora.py:71-72), i.e. the
+// with N or K equal to 8, 16, 32 or 64 -- the rank of a LoRA adapter (qwen3_moe_fused/lora.py:71-72), i.e. the
 // products dA and dB of qwen3_moe_fused/kernels/fast_lora.py:121-125,139-149 -- and the other side a multiple
 // of 256.  Such a product does nothing but stream its wide operand once, and a tile per (expert, slice) as in
 // the general kernel makes the expert with the most rows the last to finish, however the tiles are dealt:
@@ -22,7 +22,7 @@
 //     step of the expert before it (chunk 0 for experts with no rows before them).
 // Both operands have the reduction index as their slow one, so both go to LDS as they lie in memory (copies
 // that bypass the registers, a ring of stages) and are read with transposing reads (ds_read_b64_tr_b16) into
-// v_mfma_f32_32x32x16_bf16 fragments: the thin operand is the first MFMA operand (16 or 32 of its values index the
+// v_mfma_f32_32x32x16_bf16 fragments: the thin operand is the first MFMA operand (8, 16 or 32 of its values index the
 // accumulator registers of a block; rank 64 is two blocks), the 32 columns of a block of the wide operand the second (they index the lanes).
 // Rows of a step past the end of the expert are copied from a block of zeros.
 #include <type_traits>
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kSplitThreads) void dw_split_kernel(const bf16_t *_
                                                                  TO *__restrict__ out, float *__restrict__ partial,
                                                                  int4 *__restrict__ plan, int64_t R, int WIDE, int E,
                                                                  int chunks, float alpha) {
-    static_assert(TH == 16 || TH == 32 || TH == 64, "one or two MFMA blocks of thin values");
+    static_assert(TH == 8 || TH == 16 || TH == 32 || TH == 64, "one or two MFMA blocks of thin values");
     constexpr int TB = TH == 64 ? 2 : 1;  // thin blocks of 32
     constexpr int THB = TH / TB;          // thin values per block
     constexpr int STAGE = split_stage_bytes(TH);
@@ -370,10 +370,12 @@ int split_chunks(int64_t R, int wide) {
     return chunks < 1 ? 1 : chunks;
 }
 
+bool split_thin(int n) { return n == 8 || n == 16 || n == 32 || n == 64; }
+
 bool split_shape_ok(int64_t R, int N, int K, int E) {
     if (R <= 0 || R > 0x7fffffff || E <= 0 || E > kSplitMaxExperts) return false;
-    const bool thin_n = N == 16 || N == 32 || N == 64;
-    const bool thin_k = K == 16 || K == 32 || K == 64;
+    const bool thin_n = split_thin(N);
+    const bool thin_k = split_thin(K);
     if (thin_n == thin_k) return false;
     const int wide = thin_n ? K : N;
     return wide % kSliceCols == 0 && wide / kSliceCols <= 256;
@@ -404,7 +406,7 @@ int launch_split(const bf16_t *thin, const bf16_t *wide_p, const void *m_sizes, 
 
 size_t gemm_dw_split_workspace(int64_t R, int N, int K, int E) {
     if (!split_shape_ok(R, N, K, E)) return 0;
-    const bool thin_n = N == 16 || N == 32 || N == 64;
+    const bool thin_n = split_thin(N);
     const int wide = thin_n ? K : N, th = thin_n ? N : K;
     // two partial sums and one border entry per chunk
     return (size_t)split_chunks(R, wide) * (2 * (size_t)th * wide * sizeof(float) + sizeof(int4));
@@ -416,7 +418,7 @@ int gemm_dw_split(const void *dy, const void *x, const void *m_sizes, int ms_i64
     if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
     if (!aligned(dy, 16) || !aligned(x, 16) || !aligned(dw, 16) || !aligned(workspace, 16)) return MFL_ERR_ALIGN;
     if (!workspace || ws_bytes < gemm_dw_split_workspace(R, N, K, E)) return MFL_ERR_WORKSPACE;
-    const bool thin_n = N == 16 || N == 32 || N == 64;
+    const bool thin_n = split_thin(N);
     const int wide = thin_n ? K : N, th = thin_n ? N : K;
     const bf16_t *thin_p = (const bf16_t *)(thin_n ? dy : x), *wide_p = (const bf16_t *)(thin_n ? x : dy);
     const int chunks = split_chunks(R, wide);
@@ -426,8 +428,9 @@ int gemm_dw_split(const void *dy, const void *x, const void *m_sizes, int ms_i64
                                                            wide, E, chunks, alpha, stream)                            \
                            : launch_split<TH_, TN_, float>(thin_p, wide_p, m_sizes, ms_i64, (float *)dw, partial, R,   \
                                                           wide, E, chunks, alpha, stream))
-    if (thin_n) return th == 16 ? MFL_SPLIT(16, true) : th == 32 ? MFL_SPLIT(32, true) : MFL_SPLIT(64, true);
-    return th == 16 ? MFL_SPLIT(16, false) : th == 32 ? MFL_SPLIT(32, false) : MFL_SPLIT(64, false);
+    if (thin_n)
+        return th == 8 ? MFL_SPLIT(8, true) : th == 16 ? MFL_SPLIT(16, true) : th == 32 ? MFL_SPLIT(32, true) : MFL_SPLIT(64, true);
+    return th == 8 ? MFL_SPLIT(8, false) : th == 16 ? MFL_SPLIT(16, false) : th == 32 ? MFL_SPLIT(32, false) : MFL_SPLIT(64, false);
 #undef MFL_SPLIT
 }
 
