@@ -461,3 +461,44 @@ def test_block_forward_replays_from_a_hip_graph(four_bit):
             graph.replay()
             torch.cuda.synchronize()
             assert torch.equal(static_out, eager_out) and torch.equal(static_logits, eager_logits), seed
+
+
+def test_lora_mlp_step_replays_from_a_hip_graph():
+    """Forward and backward of the LoRA expert MLP (the products with the rank-r term in their reduction, the
+    split-row dA/dB kernels with their workspace, the shared passes over x) captured once and replayed: every replay
+    must equal the eager result for the inputs that are in the static buffers at that time."""
+    R, E, H, M, r = 4608, 6, 256, 256, 16
+    g = gen(5)
+    mk = lambda *shape, scale: randn(shape, g, scale, torch.bfloat16).to(DEV)  # noqa: E731
+    G, U, W = mk(E, M, H, scale=0.05), mk(E, M, H, scale=0.05), mk(E, H, M, scale=0.05)
+    lora = [mk(*s, scale=0.05).requires_grad_() for s in ((E, r, H), (E, M, r), (E, r, H), (E, M, r), (E, r, M), (E, H, r))]
+    ms = torch.bincount(torch.randint(0, E, (R,), generator=g), minlength=E).int().to(DEV)
+    static_x = mk(R, H, scale=1.0).requires_grad_()
+    static_dy = mk(R, H, scale=1.0)
+
+    def step(x, dy):
+        y = fast_lora(x, G, None, lora[0], lora[1], 2.0, U, None, lora[2], lora[3], 2.0, W, None, lora[4], lora[5], 1.5, ms)
+        grads = torch.autograd.grad(y, [x] + lora, dy)
+        return (y,) + grads
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step(static_x, static_dy)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = step(static_x, static_dy)
+    for seed in (1, 2, 3):
+        gs = gen(100 + seed)
+        x = randn((R, H), gs, 1.0, torch.bfloat16).to(DEV).requires_grad_()
+        dy = randn((R, H), gs, 1.0, torch.bfloat16).to(DEV)
+        eager = step(x, dy)                                   # eager work between the replays
+        with torch.no_grad():
+            static_x.copy_(x)
+            static_dy.copy_(dy)
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(static_out, eager):
+            assert torch.equal(a, b), seed
