@@ -119,7 +119,7 @@ class FastLora(torch.autograd.Function):
             # one pass over x for both: (E, 2 r, H)
             r = tg.shape[1]
             dAcat = _dw(x, tcat, m_sizes, dt)
-            dAg, dAu = dAcat[:, :r], dAcat[:, r:]
+            dAg, dAu = dAcat[:, :r].contiguous(), dAcat[:, r:].contiguous()  # gradients of their own, not views
         else:
             dAu = _dw(x, tu, m_sizes, dt)                              # (E, r, H)
             dAg = _dw(x, tg, m_sizes, dt)
