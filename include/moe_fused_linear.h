@@ -196,6 +196,17 @@ MFL_API int mfl_glu_fwd(const void *x, int64_t src_rows, const int32_t *row_idx,
                 void *h, void *e_out, void *g_out, int64_t R, int N, int K, int E, int dtype,
                 void *stream);
 
+/* mfl_glu_fwd with the rank-r terms of the gate and up adapters in the two reductions:
+ * h = silu(x w_gate^T + xt wt_gate^T) * (x w_up^T + xt wt_up^T), the products themselves to e_out / g_out
+ * where not NULL.  xt (R,KT) holds both adapters' scaled activations side by side ([s_g x A_g^T | s_u x A_u^T],
+ * KT = the two ranks together); wt_gate and wt_up (E,N,KT) hold each adapter's B over its own columns of xt
+ * and zeros over the other's.  The gate and up projections of the LoRA MLP with their SiLU-mul in one launch
+ * (qwen3_moe_fused/kernels/fast_lora.py:68-95).  bf16 only; MFL_ERR_UNSUPPORTED as for mfl_glu_fwd. */
+MFL_API int mfl_glu_fwd_lora(const void *x, const void *w_gate, const void *w_up, const void *xt,
+                     const void *wt_gate, const void *wt_up, int KT, const void *m_sizes,
+                     int m_sizes_dtype, void *h, void *e_out, void *g_out, int64_t R, int N, int K,
+                     int E, int dtype, void *stream);
+
 /* The same with NF4 weights, each matrix with its own quantisation state. */
 MFL_API int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div,
                     const uint8_t *wq_gate, const float *code16_gate, const float *absmax_gate,

@@ -417,3 +417,37 @@ def test_nf4_products_with_lora_term(R, N, K, E, r, bs):
     grouped_gemm_forward_transposed(tt, a, ms, out=dx2, accumulate=True)
     check_close(dx, to_np32(dx2), atol=unit_scale_atol(to_np32(dx2), 2e-2),
                 what="NF4 input gradient with a rank-r term vs two products")
+
+
+from qwen3_moe_fused.grouped_gemm.fused import grouped_glu_forward_lora  # noqa: E402
+
+
+@pytest.mark.parametrize("R,N,K,E,r", [(4096, 768, 2048, 16, 16), (9000, 512, 256, 4, 32), (700, 208, 64, 5, 8),
+                                       (33, 64, 192, 40, 16), (300, 72, 128, 3, 24)])
+def test_glu_with_lora_terms_equals_the_separate_products(R, N, K, E, r):
+    """Gate and up projections with their adapters' rank-r terms and the SiLU-mul in one launch: the two
+    products bit for bit those of the product with one thin term (the other adapter's columns meet zeros), h
+    the SiLU-mul kernel's on them."""
+    g = gen(R + N + r + 3)
+    x = randn((R, K), g, 1.0, torch.bfloat16).to(DEV)
+    wg, wu = randn((E, N, K), g, 0.05, torch.bfloat16).to(DEV), randn((E, N, K), g, 0.05, torch.bfloat16).to(DEV)
+    ug, uu = randn((R, r), g, 1.0, torch.bfloat16).to(DEV), randn((R, r), g, 1.0, torch.bfloat16).to(DEV)
+    bg, bu = randn((E, N, r), g, 0.2, torch.bfloat16).to(DEV), randn((E, N, r), g, 0.2, torch.bfloat16).to(DEV)
+    ms = m_sizes_uniform(R, E, g).to(DEV)
+    xt = torch.cat([ug, uu], 1).contiguous()
+    zeros = torch.zeros_like(bg)
+    wt_g, wt_u = torch.cat([bg, zeros], 2).contiguous(), torch.cat([zeros, bu], 2).contiguous()
+    h, e, gg = grouped_glu_forward_lora(x, wg, wu, xt, wt_g, wt_u, ms)
+    e_ref = grouped_gemm_forward_lora(x, wg, ug, bg, ms)
+    g_ref = grouped_gemm_forward_lora(x, wu, uu, bu, ms)
+    sel = oracle.sel_from_m_sizes(ms.cpu().numpy())
+    ref = (oracle.linear_fwd(to_np32(x), to_np32(wg), sel).astype(np.float64)
+           + oracle.linear_fwd(to_np32(ug), to_np32(bg), sel))
+    check_close(e, ref, what="gate product with its rank-r term vs oracle")
+    if K % 64 == 0:
+        assert torch.equal(e, e_ref) and torch.equal(gg, g_ref), "the same reductions in the same order"
+        assert torch.equal(h, silu_mul_forward(e_ref, g_ref))
+    else:
+        check_close(e, to_np32(e_ref), what="gate product")
+        check_close(gg, to_np32(g_ref), what="up product")
+        assert torch.equal(h, silu_mul_forward(e, gg))

@@ -298,6 +298,21 @@ int mfl_glu_fwd(const void *x, int64_t src_rows, const int32_t *row_idx, int idx
                           (hipStream_t)stream, &fu);
 }
 
+int mfl_glu_fwd_lora(const void *x, const void *w_gate, const void *w_up, const void *xt, const void *wt_gate,
+                     const void *wt_up, int KT, const void *m_sizes, int m_sizes_dtype, void *h, void *e_out, void *g_out,
+                     int64_t R, int N, int K, int E, int dtype, void *stream) {
+    int rc = check_fused(0, nullptr, 1, m_sizes, m_sizes_dtype, R, N, K, E, dtype, dtype);
+    if (rc) return rc;
+    if (KT <= 0) return MFL_ERR_SHAPE;
+    if (R > 0 && (!x || !w_gate || !w_up || !h || !xt || !wt_gate || !wt_up)) return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    GemmFusion fu = {nullptr, 1, 0, w_up, nullptr, nullptr, 0, e_out, g_out, nullptr};
+    fu.xt = xt, fu.wt = wt_gate, fu.kt = KT, fu.wt2 = wt_up;
+    return gemm_bf16_pipe(MODE_FWD, x, w_gate, m_sizes, m_sizes_dtype == MFL_I64, h, R, N, K, E, MFL_BF16, 1.0f, 0,
+                          (hipStream_t)stream, &fu);
+}
+
 int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div, const uint8_t *wq_gate,
                     const float *code16_gate, const float *absmax_gate, int blocksize_gate, const uint8_t *wq_up,
                     const float *code16_up, const float *absmax_up, int blocksize_up, const void *m_sizes,

@@ -34,6 +34,8 @@ struct GemmFusion {
     // wt (E, N, kt) in FWD, (E, kt, N) in DX; kt a multiple of 8.  The rank-r term of a LoRA adapter.
     const void *xt, *wt;
     int kt;
+    // the same with the gated unit (w2 given, x2 not): thin weights of the second matrix; xt is shared
+    const void *wt2;
 };
 
 // Pipelined bf16 MFMA kernels (direct global->LDS copies, multi-stage) for aligned shapes.

@@ -233,10 +233,14 @@ struct FwdFusion {
     // in DX.
     const void *at, *bt;
     int kthin;
+    // with the GLU epilogue: the thin weights of the second (up) matrix; at is shared (its columns are the two
+    // adapters' activations side by side, and each matrix's thin weights are zero over the other's columns)
+    const void *bt2;
 };
 
 // FUSE: 0 plain, 1 two weight matrices and the silu(gate) * up epilogue, 2 a thin last term in the reduction (built
-// as a kernel of its own: the test for it in every step cost the plain products 3-5 %).
+// as a kernel of its own: the test for it in every step cost the plain products 3-5 %), 3 both: each of the two
+// matrices with thin weights of its own, against one thin left operand.
 template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODE, bool NF4, int FUSE, typename TO>
 __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *__restrict__ a,
                                                                   const bf16_t *__restrict__ b,
@@ -244,7 +248,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                                                                   TO *__restrict__ c, int64_t R, int N, int K, int E,
                                                                   float alpha, int accumulate, Nf4Params nf4,
                                                                   FwdFusion fu) {
-    constexpr bool GLU = FUSE == 1, THIN = FUSE == 2;
+    constexpr bool GLU = FUSE == 1 || FUSE == 3, THIN = FUSE >= 2;
     static_assert(!THIN || MODE != MODE_DW, "the thin last term belongs to the row-grouped products");
     static_assert(!NF4 || (MODE != MODE_DW && S == 2 && BK == 64), "NF4 weights: row-grouped products, two stages");
     static_assert(!GLU || (MODE == MODE_FWD && WGN % 2 == 0 && sizeof(TO) == 2 && BK == 64),
@@ -369,7 +373,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
     const unsigned char *a_tile = nullptr, *b_tile = nullptr;
     const unsigned char *b2_tile = nullptr;
     const unsigned char *a2_tile = nullptr;  // two-term DX: second pair of operands
-    const unsigned char *at_tile = nullptr, *bt_tile = nullptr;  // the thin last term
+    const unsigned char *at_tile = nullptr, *bt_tile = nullptr, *bt2_tile = nullptr;  // the thin last term
     int KT_thin = 0;
     int lda = 0, ldb = 0;
     int64_t ldc = 0, nf4_base = 0;
@@ -447,6 +451,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 at_tile = (const unsigned char *)((const bf16_t *)fu.at + (int64_t)i0 * fu.kthin);
                 bt_tile = (const unsigned char *)((const bf16_t *)fu.bt + (B_RC ? ((int64_t)expert * N + j0) * fu.kthin
                                                                                : (int64_t)expert * N * fu.kthin + j0));
+                if constexpr (GLU)
+                    bt2_tile = (const unsigned char *)((const bf16_t *)fu.bt2 + ((int64_t)expert * N + j0) * fu.kthin);
             }
             c_base = c;
         }
@@ -586,9 +592,12 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                 const int c = SB::swz(row, SB::phys_of(load, ln));
                 const unsigned char *p;
                 if (B_RC) {
-                    const int j = row < j_lim ? row : j_lim - 1;
+                    // GLU: the stage row belongs to the gate or to the up matrix, each with its own thin weights
+                    const int col = GLU ? glu_col(row) : row;
+                    const unsigned char *bt_m = GLU && glu_up(row) ? bt2_tile : bt_tile;
+                    const int j = col < j_lim ? col : j_lim - 1;
                     const int r = ks * BK + c * 8;
-                    p = r >= k2 ? (const unsigned char *)&g_zero_chunk : bt_tile + ((int64_t)j * k2 + r) * 2;
+                    p = r >= k2 ? (const unsigned char *)&g_zero_chunk : bt_m + ((int64_t)j * k2 + r) * 2;
                 } else {
                     int r = ks * BK + row;
                     if (r >= k2) r = k2 - 1;
@@ -1073,12 +1082,12 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
     constexpr int PER_CU = LDS_BYTES <= 80 * 1024 ? 2 : 1;
     const int grid = device_info().cu_count / kXcd * kXcd * PER_CU;
     const Nf4Params none = {nullptr, nullptr, 0};
-    const FwdFusion no_fusion = {nullptr, 1, nullptr, none, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+    const FwdFusion no_fusion = {nullptr, 1, nullptr, none, nullptr, nullptr, nullptr, nullptr, nullptr, 0, nullptr};
     const FwdFusion fu = fusion ? *fusion : no_fusion;
     const bool glu = fu.b2 != nullptr && fu.a2 == nullptr;
     if ((glu || fu.row_idx) && mode != MODE_FWD) return MFL_ERR_UNSUPPORTED;
     if (fu.a2 != nullptr && (mode != MODE_DX || nf4 != nullptr || fu.b2 == nullptr)) return MFL_ERR_UNSUPPORTED;
-    if (fu.at != nullptr && (mode == MODE_DW || glu || fu.bt == nullptr)) return MFL_ERR_UNSUPPORTED;
+    if (fu.at != nullptr && (mode == MODE_DW || fu.bt == nullptr || (glu && (fu.bt2 == nullptr || nf4 != nullptr)))) return MFL_ERR_UNSUPPORTED;
 #define MFL_PIPE(MODE, NF4, GLU)                                                                                \
     {                                                                                                           \
         auto kern = gemm_pipe_kernel<MB, NB, BK, S, WGM, WGN, MODE, NF4, GLU, TO>;                              \
@@ -1093,7 +1102,10 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
     }
     // MODES bit 3: the configuration is also built with the GLU epilogue (bf16 output only)
     constexpr bool GLU_OK = (MODES & 8) && WGN % 2 == 0 && sizeof(TO) == 2 && BK == 64;
-    if (glu) {
+    if (glu && fu.at != nullptr) {
+        if constexpr (GLU_OK && (MODES & 16) != 0) MFL_PIPE(MODE_FWD, false, 3)
+        else return MFL_ERR_UNSUPPORTED;
+    } else if (glu) {
         if constexpr (GLU_OK) {
             if (nf4 != nullptr) {
                 if constexpr (S == 2 && NB * 64 <= NT) MFL_PIPE(MODE_FWD, true, true)
@@ -1218,7 +1230,7 @@ namespace {
 // Checks the fusion request of a forward product and translates it for the kernel.
 // Returns MFL_ERR_UNSUPPORTED for what the pipelined kernels do not take.
 int make_fusion(const GemmFusion *f, int K, bool nf4, FwdFusion *out) {
-    *out = FwdFusion{nullptr, 1, nullptr, Nf4Params{nullptr, nullptr, 0}, nullptr, nullptr, nullptr, nullptr, nullptr, 0};
+    *out = FwdFusion{nullptr, 1, nullptr, Nf4Params{nullptr, nullptr, 0}, nullptr, nullptr, nullptr, nullptr, nullptr, 0, nullptr};
     if (f == nullptr) return MFL_OK;
     if (f->row_idx != nullptr) {
         // the kernel addresses the source rows with 32-bit byte offsets
@@ -1228,11 +1240,15 @@ int make_fusion(const GemmFusion *f, int K, bool nf4, FwdFusion *out) {
         out->idx_div = f->idx_div;
     }
     if (f->xt != nullptr) {
+        // with a second weight matrix and no second left operand (the gated unit) the thin term needs thin weights
+        // for that matrix too
+        const bool glu_thin = f->w2 != nullptr && f->x2 == nullptr;
         if (f->wt == nullptr || f->kt < 8 || f->kt % 8 != 0 || !aligned(f->xt, 16) || !aligned(f->wt, 16) ||
-            f->row_idx != nullptr || (f->w2 != nullptr && f->x2 == nullptr))
+            f->row_idx != nullptr || (glu_thin && (nf4 || f->wt2 == nullptr || !aligned(f->wt2, 16))))
             return MFL_ERR_UNSUPPORTED;
         out->at = f->xt;
         out->bt = f->wt;
+        out->bt2 = glu_thin ? f->wt2 : nullptr;
         out->kthin = f->kt;
     }
     if (f->x2 != nullptr) {

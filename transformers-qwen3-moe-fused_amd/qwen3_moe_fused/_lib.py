@@ -44,6 +44,7 @@ _SIGNATURES = {
     "mfl_gemm_fwd_nf4_gather": (_i, [_vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i,
                                      _vp]),
     "mfl_glu_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp]),
+    "mfl_glu_fwd_lora": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp]),
     "mfl_glu_fwd_nf4": (_i, [_vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _i64,
                              _i, _i, _i, _i, _vp]),
     "mfl_nf4_dequant": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _vp]),

@@ -294,3 +294,32 @@ def grouped_gemm_forward_transposed_4bit_lora(dy: torch.Tensor, w_quant: torch.T
         return grouped_gemm_forward_transposed(xt, wt, m_sizes, dtype, out=dx, accumulate=True)
     _lib.check(rc, "mfl_gemm_dx_nf4_lora")
     return dx
+
+
+def grouped_glu_forward_lora(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, xt: torch.Tensor,
+                             wt_gate: torch.Tensor, wt_up: torch.Tensor, m_sizes: torch.Tensor):
+    """``(h, e, g)`` with ``e = x w_gate^T + xt wt_gate^T``, ``g = x w_up^T + xt wt_up^T``, ``h = silu(e) * g`` in
+    one kernel: the gate and up projections of the LoRA MLP with their rank-r terms and the SiLU-mul
+    (qwen3_moe_fused/kernels/fast_lora.py:68-95).  ``xt`` (rows, r_g + r_u) holds both adapters' scaled
+    activations side by side; ``wt_gate`` / ``wt_up`` (E, N, r_g + r_u) hold each adapter's B over its own columns
+    and zeros over the other's."""
+    check_operands(m_sizes, x, w_gate, w_up, xt, wt_gate, wt_up)
+    assert x.ndim == 2 and w_gate.ndim == 3 and w_up.shape == w_gate.shape
+    rows, k = x.shape
+    experts, n, k_w = w_gate.shape
+    kt = xt.shape[1]
+    assert k_w == k and m_sizes.numel() == experts and xt.shape[0] == rows
+    assert wt_gate.shape == (experts, n, kt) and wt_up.shape == (experts, n, kt)
+    h = torch.empty((rows, n), device=x.device, dtype=x.dtype)
+    e, g = torch.empty_like(h), torch.empty_like(h)
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = _lib.lib().mfl_glu_fwd_lora(_lib.ptr(x), _lib.ptr(w_gate), _lib.ptr(w_up), _lib.ptr(xt), _lib.ptr(wt_gate),
+                                     _lib.ptr(wt_up), kt, _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(h),
+                                     _lib.ptr(e), _lib.ptr(g), rows, n, k, experts, _lib.dtype_code(x.dtype),
+                                     _lib.stream())
+    if rc == UNSUPPORTED:
+        e = grouped_gemm_forward_lora(x, w_gate, xt, wt_gate, m_sizes)
+        g = grouped_gemm_forward_lora(x, w_up, xt, wt_up, m_sizes)
+        return silu_mul_forward(e, g), e, g
+    _lib.check(rc, "mfl_glu_fwd_lora")
+    return h, e, g

@@ -25,6 +25,7 @@ from ..grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit as 
 from ..grouped_gemm.forward_transposed import grouped_gemm_forward_transposed as _dx
 from ..grouped_gemm.fused import grouped_gemm_forward_4bit_lora as _fwd4_lora
 from ..grouped_gemm.fused import grouped_gemm_forward_lora as _fwd_lora
+from ..grouped_gemm.fused import grouped_glu_forward_lora as _glu_lora
 from ..grouped_gemm.fused import grouped_gemm_forward_transposed_4bit_lora as _dx4_lora
 from ..grouped_gemm.fused import grouped_gemm_forward_transposed_lora as _dx_lora
 from ..quantize.nf4 import dequantize_nf4
@@ -80,15 +81,22 @@ class FastLora(torch.autograd.Function):
         dt = x.dtype
         x = x.contiguous()
         Ag, Bg, Au, Bu, Aw, Bw = (p.to(dt).contiguous() for p in (Ag, Bg, Au, Bu, Aw, Bw))
-        ug = uu = None
+        ug = uu = ucat = None
         if Sg == Su and Ag.shape == Au.shape and x.shape[0] >= _WIDE_ROWS:
             # one pass over x for both adapters' rank-r activations
             r = Ag.shape[1]
             ucat = _fwd(x, torch.cat((Ag, Au), dim=1), m_sizes, alpha=Sg)
             ug, uu = ucat[:, :r].contiguous(), ucat[:, r:].contiguous()
-        e, ug = _proj_fwd(x, Gq, Gqs, Ag, Bg, Sg, m_sizes, ug)
-        g, uu = _proj_fwd(x, Uq, Uqs, Au, Bu, Su, m_sizes, uu)
-        h = silu_mul_forward(e, g)
+        if (ucat is not None and Gqs is None and Uqs is None and dt == torch.bfloat16 and Gq.dtype == dt
+                and Uq.dtype == dt and Bg.shape == Bu.shape):
+            # gate, up, both rank-r terms and the SiLU-mul in one launch: each matrix's thin weights are its
+            # adapter's B over its own columns of ucat and zeros over the other's
+            zeros = torch.zeros_like(Bg)
+            h, e, g = _glu_lora(x, Gq, Uq, ucat, torch.cat((Bg, zeros), dim=2), torch.cat((zeros, Bu), dim=2), m_sizes)
+        else:
+            e, ug = _proj_fwd(x, Gq, Gqs, Ag, Bg, Sg, m_sizes, ug)
+            g, uu = _proj_fwd(x, Uq, Uqs, Au, Bu, Su, m_sizes, uu)
+            h = silu_mul_forward(e, g)
         y, _ = _proj_fwd(h, Wq, Wqs, Aw, Bw, Sw, m_sizes)
         ctx.frozen = (Gq, Gqs, Sg, Uq, Uqs, Su, Wq, Wqs, Sw, m_sizes)
         ctx.save_for_backward(x, Ag, Bg, Au, Bu, Aw, Bw, e, g, ug, uu)
