@@ -1,9 +1,14 @@
 """mfl_gemm_dw_split (dW with one side as thin as a LoRA rank, rows dealt out evenly over the workgroups)
-against the per-expert closed form dy_e^T x_e in fp32 (what the reference's own test differentiates:
-qwen3_moe_fused/grouped_gemm/backward_dw.py:64-89, test_moe_fused_linear_bwd.py:49-54), through the C ABI."""
+against the CPU oracle's weight gradient (oracle.linear_bwd_weight, the restatement of
+qwen3_moe_fused/functional.py:52-61; the product the reference's kernel computes is
+qwen3_moe_fused/grouped_gemm/backward_dw.py:64-89), through the C ABI.  Every rank the entry takes (8, 16, 32,
+64) meets the oracle on all experts, among them experts cut by a chunk border ("one": a single expert holds
+every row and is cut by every border; "zipf": the hot experts span several chunks)."""
+import numpy as np
 import pytest
 import torch
 
+import oracle
 from util import unit_scale_atol as _atol_np
 
 
@@ -47,14 +52,12 @@ def _call(x, dy, ms, out_dtype, alpha=1.0):
 
 
 def _closed_form(x, dy, ms, alpha):
-    E = ms.numel()
-    ref = torch.zeros((E, dy.shape[1], x.shape[1]), dtype=torch.float32, device=x.device)
-    start = 0
-    for e, m in enumerate(ms.tolist()):
-        if m:
-            ref[e] = alpha * (dy[start:start + m].float().T @ x[start:start + m].float())
-        start += m
-    return ref
+    """alpha * dW of the CPU oracle on the same bf16-rounded inputs (rows past sum(ms) belong to no expert)."""
+    counts = ms.cpu().numpy().astype(np.int64)
+    rows = int(counts.sum())
+    sel = oracle.sel_from_m_sizes(counts)
+    ref = oracle.linear_bwd_weight(dy[:rows].float().cpu().numpy(), x[:rows].float().cpu().numpy(), sel, ms.numel())
+    return torch.from_numpy(np.asarray(ref, dtype=np.float32) * np.float32(alpha)).to(x.device)
 
 
 CASES = [

@@ -216,10 +216,12 @@ def _near_tied(logits_row: np.ndarray, a: int, b: int) -> bool:
     return abs(la - lb) <= 2.0 ** -5 * max(abs(la), abs(lb), 1.0)
 
 
-@pytest.mark.parametrize("tokens", [16, 256])
+@pytest.mark.parametrize("tokens", [16, 256, 16384])
 def test_config5_nf4_sparse_block_matches_oracle(nf4_experts, tokens):
     """The whole sparse block with NF4 experts (router -> top-8 of 128 -> sort -> gate/up -> SiLU-mul
-    -> down -> weighted sum) against oracle.moe_block_fwd on the oracle-dequantised weights."""
+    -> down -> weighted sum) against oracle.moe_block_fwd on the oracle-dequantised weights.  Tokens are
+    independent given their routing, so at 16384 tokens the oracle evaluates a seeded sample of 320 of them;
+    the routing that is compared is the block's own (its top-k kernel's expert ids), not a second top-k."""
     from types import SimpleNamespace
 
     from qwen3_moe_fused.modular_qwen3_moe_fused import Qwen3MoeFusedSparseMoeBlock
@@ -240,15 +242,26 @@ def test_config5_nf4_sparse_block_matches_oracle(nf4_experts, tokens):
         setattr(blk, name, layer)
     blk = blk.to(DEV)
     hidden = randn((1, tokens, H), gen(tokens), 1.0, torch.bfloat16)
-    out_ref, logits_ref = oracle.moe_block_fwd(to_np32(hidden[0]), to_np32(gate_w), nf4_experts["gate"][2],
+    sample = np.arange(tokens) if tokens <= 320 else np.sort(np.random.default_rng(tokens).choice(tokens, 320, replace=False))
+    st = torch.from_numpy(sample)
+    out_ref, logits_ref = oracle.moe_block_fwd(to_np32(hidden[0][st]), to_np32(gate_w), nf4_experts["gate"][2],
                                                nf4_experts["up"][2], nf4_experts["down"][2], K8, True, oracle.round_bf16)
+    blk.keep_routing = True
     for fuse in (True, False):
         blk.fuse_front = fuse
         with torch.no_grad():
             out, logits = blk(hidden.to(DEV))
         assert out.shape == (1, tokens, H) and logits.shape == (tokens, E)
+        sel_all = blk.last_selected
+        assert sel_all.shape == (tokens, K8)
+        # the block's selections are a top-k of the block's own logits (ties aside: compare probabilities)
+        p_gpu = torch.softmax(logits.float(), -1)
+        kth = torch.gather(p_gpu, 1, sel_all.long()).min(dim=1).values
+        rest = p_gpu.scatter(1, sel_all.long(), -1.0).max(dim=1).values
+        assert (kth >= rest).all(), "a selected expert has a smaller probability than one left out"
+        out, logits = out[:, st.to(out.device)], logits[st.to(logits.device)]
         check_close(logits, logits_ref, 2e-2, 2e-2, "router logits")
-        sel_gpu = torch.topk(torch.softmax(logits.float(), -1), K8).indices.cpu().numpy()
+        sel_gpu = sel_all[st.to(sel_all.device)].cpu().numpy()
         sel_ref = oracle.softmax_topk(logits_ref, K8, True)[1]
         same = np.array([set(a) == set(b) for a, b in zip(sel_gpu, sel_ref)])
         assert same.mean() >= 0.9

@@ -262,3 +262,40 @@ def test_random_shapes_match_oracle_bf16(seed):
     check_close(dw, exp_dw, 1e-2, 1e-2 * max(1.0, np.abs(exp_dw).max()), "dw " + what)
     for e in (ms == 0).nonzero().flatten().tolist():
         assert torch.count_nonzero(dw[e]).item() == 0, "experts without rows must get exact zeros"
+
+
+# ---- the four-wave kernel (128 x 128 wave tiles): whole 256 x 256 tiles along the weight dimensions and at least
+# 64 rows per expert on average.  Row counts that end inside a 32-row step, inside its first half, on a step edge;
+# experts without rows (exact zeros, written between two experts with rows); one expert that holds most rows; rows
+# past sum(m_sizes); int64 sizes; more experts than a wave has lanes.
+WIDE_DW_CASES = [
+    # N, K, m_sizes
+    (256, 256, [64]),
+    (256, 512, [1, 0, 300, 31, 32, 33, 0, 700]),
+    (512, 256, [0, 0, 517, 0, 15, 16, 17, 480, 0]),
+    (768, 256, [96] * 7 + [0] + [1000]),
+    (256, 768, [70 + (3 * e) % 11 for e in range(130)]),
+]
+
+
+@pytest.mark.parametrize("N,K,sizes", WIDE_DW_CASES)
+@pytest.mark.parametrize("ms_dtype", [torch.int32, torch.int64])
+def test_dw_four_wave_kernel_matches_oracle(N, K, sizes, ms_dtype):
+    ms = torch.tensor(sizes, dtype=ms_dtype)
+    E, rows = ms.numel(), int(ms.sum())
+    extra = 37                                   # rows that belong to no expert
+    R = max(rows + extra, 64 * E)                # enough rows for the dispatcher to take this kernel
+    g = gen(N + K + E)
+    x = randn((R, K), g, 1.0, torch.bfloat16)
+    dy = randn((R, N), g, 1.0, torch.bfloat16)
+    x[rows:] = float("nan")
+    dy[rows:] = float("inf")
+    sel = oracle.sel_from_m_sizes(ms.numpy())
+    xd, dyd, msd = x.to(DEV), dy.to(DEV), ms.to(DEV)
+    print(f"four-wave dW N={N} K={K} E={E} R={R}", flush=True)
+    dw = grouped_gemm_backward_dw(xd, dyd, msd, torch.bfloat16)
+    exp = oracle.linear_bwd_weight(to_np32(dy[:rows]), to_np32(x[:rows]), sel, E)
+    check_close(dw, exp, 1e-2, 1e-2 * max(1.0, np.abs(exp).max()), "four-wave dW")
+    for e in (ms == 0).nonzero().flatten().tolist():
+        assert torch.count_nonzero(dw[e]).item() == 0, "experts without rows must get exact zeros"
+    assert torch.equal(grouped_gemm_backward_dw(xd, dyd, msd, torch.bfloat16), dw), "same bits from run to run"

@@ -1,0 +1,594 @@
+// bf16 grouped GEMM for CDNA4 with four waves per workgroup, one per SIMD, each holding a wave tile of up to
+// 128 x 128 outputs in its 256 accumulation registers.  Against the eight-wave tiles of gemm_bf16_pipe.hip a wave
+// reads a third fewer LDS fragment bytes per MFMA, which is what the weight-gradient product (both operands read
+// with transposing LDS reads, half the rate of plain ones) and the matrix-bound shapes of the other two products
+// are limited by.
+//
+// Operand conventions are those of gemm_bf16_pipe.hip: C[i, j] = sum_r A(i, r) * B(j, r), each operand
+// reduction-contiguous (RC) or reduction-strided (RS); FWD = RC x RC, DX = RC x RS, DW = RS x RS; the stage
+// layouts, copies and fragment reads come from pipe_parts.h.
+//
+// One stream of reduction steps per workgroup.  The tiles of a persistent workgroup are not separate pipelines:
+// a producer cursor walks (tile, step) ahead of the consumer cursor, so the copies of the next tile's first steps
+// are in flight while the current tile is multiplied and its output stored.  The ring holds SR stages.  In step g
+// the wave multiplies all sub-steps but the last, then (point P) waits for its own copies of step g+1, meets the
+// other waves at the one barrier of the step -- after it stage g is free and stage g+1 complete for everybody --
+// requests the fragments of step g+1's first sub-step, and multiplies the last sub-step of step g with the copies
+// of step g+SR dealt out between its MFMAs.  With one wave per SIMD nothing else hides a wait, so neither the
+// fragment reads nor the copies are ever asked for right before they are needed.
+//
+// The vector-memory counter of a wave counts down in order of issue; the kernel keeps the number of operations it
+// has issued (copies and output stores) and, per ring slot, that number after the slot's last copy: "step g+1 has
+// landed" is a wait for at most (issued - mark) outstanding operations, whatever was issued in between.
+//
+// Shapes: bf16 in, bf16 out, no accumulation, no scaling; E <= 512; FWD/DX: N % BN == 0, K % 64 == 0; DW: N % BM == 0,
+// K % BN == 0 (any number of rows per expert).  The caller falls back to gemm_bf16_pipe.hip otherwise.
+#include "pipe_parts.h"
+
+namespace mfl {
+
+namespace {
+
+// Tuning builds can take parts of the kernel out (timing experiments only; the results are then wrong).
+#ifdef MFL_TUNING_BUILD
+#ifndef MFL_X_NO_STORE
+#define MFL_X_NO_STORE 0
+#endif
+#ifndef MFL_X_NO_COPY
+#define MFL_X_NO_COPY 0
+#endif
+#ifndef MFL_X_NO_MFMA
+#define MFL_X_NO_MFMA 0
+#endif
+constexpr bool kNoStore = MFL_X_NO_STORE, kNoCopy = MFL_X_NO_COPY, kNoMfma = MFL_X_NO_MFMA;
+#else
+constexpr bool kNoStore = false, kNoCopy = false, kNoMfma = false;
+#endif
+
+// s_waitcnt vmcnt(n rounded down to a multiple of 8), n wave-uniform
+__device__ __forceinline__ void wait_vmcnt_upto(int n) {
+    switch (n >> 3) {
+        case 0: wait_vmcnt<0>(); break;
+        case 1: wait_vmcnt<8>(); break;
+        case 2: wait_vmcnt<16>(); break;
+        case 3: wait_vmcnt<24>(); break;
+        case 4: wait_vmcnt<32>(); break;
+        case 5: wait_vmcnt<40>(); break;
+        case 6: wait_vmcnt<48>(); break;
+        default: wait_vmcnt<56>(); break;
+    }
+}
+
+// f(IC<0>{}), ..., f(IC<N-1>{}): a loop whose index is a constant expression inside the body
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(IC<I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// 16 bytes per lane from a per-lane address to 1 KiB of consecutive LDS; POLICY 2 = non-temporal.  The copy is
+// issued when `on` (wave-uniform) is not zero.  The test sits inside the statement: a branch in the source around a
+// copy between two MFMAs cuts the sub-step into basic blocks, and two variants of a sub-step (with and without
+// copies) make the register allocator move accumulators between them.
+template <int POLICY>
+__device__ __forceinline__ void wide_copy(const unsigned char *src, uint32_t lds_addr) {
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);  // wave-uniform by construction; the asm needs an SGPR
+    if constexpr (kNoCopy)
+        asm volatile("s_nop 0" : : "v"(src), "s"(lds_addr) : "memory");
+    else if constexpr (POLICY == 2)
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" : : "v"(src), "s"(lds_addr) : "memory");
+    else
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(lds_addr) : "memory");
+}
+template <int POLICY>
+__device__ __forceinline__ void wide_copy_if(const unsigned char *src, uint32_t lds_addr, int on) {
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+    if constexpr (kNoCopy)
+        asm volatile("s_nop 0" : : "v"(src), "s"(lds_addr), "s"(on) : "memory");
+    else if constexpr (POLICY == 2)
+        asm volatile(
+            "s_cmp_eq_u32 %2, 0\n\ts_cbranch_scc1 .Lwc_skip_%=\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+            "global_load_lds_dwordx4 %0, off nt\n.Lwc_skip_%=:"
+            :
+            : "v"(src), "s"(lds_addr), "s"(on)
+            : "memory", "scc");
+    else
+        asm volatile(
+            "s_cmp_eq_u32 %2, 0\n\ts_cbranch_scc1 .Lwc_skip_%=\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+            "global_load_lds_dwordx4 %0, off\n.Lwc_skip_%=:"
+            :
+            : "v"(src), "s"(lds_addr), "s"(on)
+            : "memory", "scc");
+}
+
+// One accumulator element, fetched from its accumulation register where the statement stands.  (Left to itself
+// the compiler copies all 256 of a tile into vector registers at the top of the epilogue, and spills what else
+// is live there: the fragments and addresses of the next tile's first step.)
+__device__ __forceinline__ float acc_read(float v) {
+    float r;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(r) : "a"(v));
+    return r;
+}
+
+template <int MODE, int MB, int NB, int BK, int SR, typename TO>
+__global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict__ a, const bf16_t *__restrict__ b,
+                                                        const void *__restrict__ m_sizes, int ms_i64,
+                                                        TO *__restrict__ c, int64_t R, int N, int K, int E) {
+    static_assert(sizeof(TO) == 2, "bf16 output");
+    constexpr int WGM = 2, WGN = 2, NW = 4;
+    constexpr int BM = MB * 32, BN = NB * 32;
+    constexpr bool A_RC = MODE != MODE_DW, B_RC = MODE == MODE_FWD;
+    constexpr int TM = (MB + WGM - 1) / WGM;  // row blocks per wave, dealt round robin (the last may not exist)
+    static_assert(NB % WGN == 0, "column blocks must split evenly over the waves");
+    constexpr int TN = NB / WGN, WTN = TN * 32, KS = BK / 16;
+    static_assert(KS % 2 == 0, "fragment buffers alternate by sub-step");
+    typedef Stage<BM, BK, A_RC> SA;
+    typedef Stage<BN, BK, B_RC> SB;
+    static_assert(SA::kWaveLoads % NW == 0 && SB::kWaveLoads % NW == 0, "copies must split over the waves");
+    constexpr int LA = SA::kWaveLoads / NW, LB = SB::kWaveLoads / NW, LPW = LA + LB;
+    static_assert(LPW % 8 == 0, "the waits count in eights");
+    constexpr int STAGE_BYTES = SA::kBytes + SB::kBytes;
+    constexpr int RING_BYTES = SR * STAGE_BYTES;
+    // output staging, per wave: 32 rows of EPC columns
+    constexpr int EPC = WTN % 64 == 0 ? 64 : WTN;
+    constexpr int EP_ROWB = EPC * 2 + (EPC == 64 ? 16 : 8);
+    constexpr int EP_WAVE = 32 * EP_ROWB;
+    constexpr int STORES = TM * (WTN / EPC) * (EPC / 8 * 32 / 64);  // 16-byte stores per lane and tile
+    static_assert((EPC / 8 * 32) % 64 == 0, "whole wave stores");
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+
+    FragOffsets<BM, BK, A_RC, TM> fo_a;
+    FragOffsets<BN, BK, B_RC, TN> fo_b;
+    fo_a.init(wm * 32, WGM * 32, lane);
+    fo_b.init(wn * WTN, 32, lane);
+
+    // ---- per-expert prefix tables in LDS behind the ring and the staging area: rows and tiles before expert e
+    int *tab_rows = (int *)(smem + RING_BYTES + NW * EP_WAVE);
+    int *tab_tiles = tab_rows + (kMaxTableExperts + 1);
+    const int tiles_n = MODE == MODE_DW ? K / BN : N / BN;
+    const int per_expert = MODE == MODE_DW ? (N / BM) * tiles_n : 0;
+    {
+        int row_carry = 0, tile_carry = 0;
+        for (int e0 = 0; e0 < E; e0 += 64) {
+            const int e = e0 + lane;
+            const int m = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
+            const int t = e >= E ? 0 : MODE == MODE_DW ? per_expert : m_tiles_of<BM>(m) * tiles_n;
+            const int minc = wave_inclusive_scan(m), tinc = wave_inclusive_scan(t);
+            if (wave == 0 && e <= E) {
+                tab_rows[e] = row_carry + minc - m;
+                tab_tiles[e] = tile_carry + tinc - t;
+            }
+            row_carry += wave_last(minc);
+            tile_carry += wave_last(tinc);
+        }
+        if (wave == 0 && lane == 0 && E % 64 == 0) {
+            tab_rows[E] = row_carry;
+            tab_tiles[E] = tile_carry;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+    }
+    const int total = __builtin_amdgcn_readfirstlane(tab_tiles[E]);
+
+    // ---- tile range of this workgroup: XCD x owns a contiguous run of logical tiles (the tiles of an expert meet
+    // in one L2), dealt out with a stride inside the run
+    const int xcd = blockIdx.x % kXcd;
+    const int per_xcd = gridDim.x / kXcd;
+    const int chunk = ceil_div(total, kXcd);
+    const int L_first = xcd * chunk + blockIdx.x / kXcd;
+    int L_end = (xcd + 1) * chunk;
+    if (L_end > total) L_end = total;
+
+    // ---- what a cursor knows about a tile; every field wave-uniform
+    struct Tile {
+        int i0, i_end, j0, red, KT;
+        const unsigned char *pa, *pb;
+        TO *pc;
+    };
+    auto tile_at = [&](int L, Tile &t) {
+        if (MODE == MODE_DW) {
+            const int e = L / per_expert, local = L % per_expert;
+            t.i0 = (local / tiles_n) * BM;
+            t.i_end = t.i0 + BM;
+            t.j0 = (local % tiles_n) * BN;
+            int rb = __builtin_amdgcn_readfirstlane(tab_rows[e]);
+            int re = __builtin_amdgcn_readfirstlane(tab_rows[e + 1]);
+            if ((int64_t)re > R) re = (int)R;
+            if (rb > re) rb = re;
+            t.red = re - rb;
+            t.KT = ceil_div(t.red, BK);
+            t.pa = (const unsigned char *)(a + (int64_t)rb * N + t.i0);
+            t.pb = (const unsigned char *)(b + (int64_t)rb * K + t.j0);
+            t.pc = c + (int64_t)e * N * K;
+        } else {
+            int expert = 0;
+            for (int e0 = 0; e0 < E; e0 += 64) {
+                const int e = e0 + lane < E ? e0 + lane : E - 1;
+                const uint64_t hits = __ballot(e0 + lane < E && L >= tab_tiles[e] && L < tab_tiles[e + 1]);
+                if (hits) {
+                    expert = e0 + __ffsll((unsigned long long)hits) - 1;
+                    break;
+                }
+            }
+            expert = __builtin_amdgcn_readfirstlane(expert);
+            const int m_start = __builtin_amdgcn_readfirstlane(tab_rows[expert]);
+            const int m_size = __builtin_amdgcn_readfirstlane(tab_rows[expert + 1]) - m_start;
+            const int local = L - __builtin_amdgcn_readfirstlane(tab_tiles[expert]);
+            const int m_tiles = m_tiles_of<BM>(m_size);
+            const int rows = tile_rows_of<BM>(m_size);
+            // few row tiles: those of one column slice run side by side (they share the slice of the weights);
+            // many: the column slices of one row tile (they share its rows)
+            const bool n_fast = m_tiles > tiles_n;
+            const int mi = n_fast ? local / tiles_n : local % m_tiles;
+            const int ni = n_fast ? local % tiles_n : local / m_tiles;
+            t.i0 = m_start + mi * rows;
+            t.i_end = m_start + m_size;
+            if (t.i_end > t.i0 + rows) t.i_end = t.i0 + rows;
+            if ((int64_t)t.i_end > R) t.i_end = (int)R;
+            if (t.i0 > t.i_end) t.i0 = t.i_end;
+            t.j0 = ni * BN;
+            t.red = K;
+            t.KT = t.i_end > t.i0 ? K / BK : 0;
+            t.pa = (const unsigned char *)(a + (int64_t)t.i0 * K);
+            t.pb = B_RC ? (const unsigned char *)(b + (int64_t)expert * N * K + (int64_t)t.j0 * K)
+                        : (const unsigned char *)(b + (int64_t)expert * N * K + t.j0);
+            t.pc = c;
+        }
+    };
+    const int lda = MODE == MODE_DW ? N : K;
+    const int ldb = MODE == MODE_FWD ? K : MODE == MODE_DX ? N : K;
+    const int64_t ldc = MODE == MODE_DW ? K : N;
+    const int64_t step_a = A_RC ? (int64_t)BK * 2 : (int64_t)BK * lda * 2;
+    const int64_t step_b = B_RC ? (int64_t)BK * 2 : (int64_t)BK * ldb * 2;
+
+    // ---- producer: the (tile, step) whose copies are issued next
+    Tile pt;
+    int pL = L_first, pk = 0;
+    bool p_more = false;
+    uint32_t lane_off[LPW];
+    auto prod_offsets = [&]() {
+        const int i_lim = pt.i_end - pt.i0 < BM ? pt.i_end - pt.i0 : BM;
+#pragma unroll
+        for (int q = 0; q < LA; ++q) lane_off[q] = (uint32_t)lane_src_offset<BM, BK, A_RC>(wave * LA + q, lane, lda, i_lim);
+    };
+    auto prod_seek = [&]() {  // first tile from pL on that has steps
+        p_more = false;
+        while (pL < L_end) {
+            tile_at(pL, pt);
+            if (pt.KT > 0) {
+                p_more = true;
+                if (MODE != MODE_DW) prod_offsets();
+                break;
+            }
+            pL += per_xcd;
+        }
+        pk = 0;
+    };
+#pragma unroll
+    for (int q = 0; q < LB; ++q) lane_off[LA + q] = (uint32_t)lane_src_offset<BN, BK, B_RC>(wave * LB + q, lane, ldb, BN);
+    if (MODE == MODE_DW) {
+#pragma unroll
+        for (int q = 0; q < LA; ++q) lane_off[q] = (uint32_t)lane_src_offset<BM, BK, A_RC>(wave * LA + q, lane, lda, BM);
+    }
+    prod_seek();
+
+    int issued = 0;  // vector-memory operations this wave has issued
+    int mark[SR];    // `issued` after the last copy into ring slot s
+#pragma unroll
+    for (int s = 0; s < SR; ++s) mark[s] = 0;
+    int pg = 0;  // steps whose copies have been issued
+    const uint32_t ring_lds = (uint32_t)(uintptr_t)(lds_void_ptr)smem;
+
+    // Cache policy: the weights of the row-grouped products are read by one workgroup per column slice
+    // (non-temporal, the L2 is left to the rows); DW: both panels are shared by the tiles of an expert.
+    constexpr int A_POLICY = 0;
+    constexpr int B_POLICY = MODE == MODE_DW ? 0 : 2;
+
+    // the q-th copy of the wave for the producer's step into ring slot `slot`; full steps only
+    auto copy_one = [&](auto q_tag, int slot) {
+        constexpr int q = decltype(q_tag)::value;
+        const uint32_t st = ring_lds + slot * STAGE_BYTES;
+        if constexpr (q < LA)
+            wide_copy<A_POLICY>(pt.pa + pk * step_a + lane_off[q], st + (wave * LA + q) * 1024);
+        else
+            wide_copy<B_POLICY>(pt.pb + pk * step_b + lane_off[q], st + SA::kBytes + (wave * LB + (q - LA)) * 1024);
+    };
+    auto copy_one_if = [&](auto q_tag, int slot, int on) {
+        constexpr int q = decltype(q_tag)::value;
+        const uint32_t st = ring_lds + slot * STAGE_BYTES;
+        if constexpr (q < LA)
+            wide_copy_if<A_POLICY>(pt.pa + pk * step_a + lane_off[q], st + (wave * LA + q) * 1024, on);
+        else
+            wide_copy_if<B_POLICY>(pt.pb + pk * step_b + lane_off[q], st + SA::kBytes + (wave * LB + (q - LA)) * 1024, on);
+    };
+    // a partial last step of DW: rows of A past the end come from a chunk of zeros, rows of B past the end
+    // re-read the last row (finite values that meet zeros)
+    auto copy_tail = [&](int slot) {
+        const uint32_t st = ring_lds + slot * STAGE_BYTES;
+        const int valid = pt.red - pk * BK;  // 1 .. BK - 1 rows
+#pragma unroll
+        for (int q = 0; q < LA; ++q) {
+            const int row = SA::row_of(wave * LA + q, lane);
+            const unsigned char *p = pt.pa + pk * step_a + lane_off[q];
+            if (row >= valid) p = (const unsigned char *)&g_zero_chunk;
+            wide_copy<0>(p, st + (wave * LA + q) * 1024);
+        }
+#pragma unroll
+        for (int q = 0; q < LB; ++q) {
+            const int row = SB::row_of(wave * LB + q, lane);
+            const unsigned char *p = pt.pb + pk * step_b + lane_off[LA + q];
+            if (row >= valid) p -= (int64_t)(row - (valid - 1)) * ldb * 2;
+            wide_copy<0>(p, st + SA::kBytes + (wave * LB + q) * 1024);
+        }
+    };
+    auto prod_is_tail = [&]() { return MODE == MODE_DW && (pk + 1) * BK > pt.red; };
+    auto prod_advance = [&]() {  // after the copies of a step
+        issued += LPW;
+        mark[pg % SR] = issued;
+        ++pg;
+        if (++pk == pt.KT) {
+            pL += per_xcd;
+            prod_seek();
+        }
+    };
+    auto issue_all = [&]() {  // one whole step, back to back
+        const int slot = pg % SR;
+        if (prod_is_tail()) {
+            copy_tail(slot);
+        } else {
+            static_for<LPW>([&](auto q_tag) { copy_one(q_tag, slot); });
+        }
+        prod_advance();
+    };
+
+    // ---- consumer
+    Tile ct;
+    int cL = L_first;
+    int g = 0;  // steps multiplied so far (of the whole workgroup)
+    bf16x8 fa[2][TM], fb[2][TN];  // carried from step to step, across tiles
+
+    auto stage_of = [&](int step) { return smem + (step % SR) * STAGE_BYTES; };
+    auto load_frags = [&](const unsigned char *st, int ks, int buf) {
+#pragma unroll
+        for (int bj = 0; bj < TN; ++bj) fb[buf][bj] = fo_b.load(st + SA::kBytes, bj, ks);
+#pragma unroll
+        for (int t = 0; t < TM; ++t) fa[buf][t] = fo_a.load(st, t, ks);
+    };
+
+    // prologue: SR steps in flight, the first one landed and its first fragments requested
+#pragma unroll 1
+    for (int s = 0; s < SR; ++s)
+        if (p_more) issue_all();
+    if (pg > 0) {
+        wait_vmcnt_upto(issued - mark[0]);
+        __builtin_amdgcn_s_barrier();
+        load_frags(stage_of(0), 0, 0);
+    }
+
+    const int h = lane >> 5, rl = lane & 31;
+    unsigned char *const ep = smem + RING_BYTES + wave * EP_WAVE;
+
+#pragma unroll 1
+    for (; cL < L_end; cL += per_xcd) {
+        tile_at(cL, ct);
+        const int i_lim = ct.i_end - ct.i0 < BM ? ct.i_end - ct.i0 : BM;
+        const int n_blocks = ceil_div(i_lim, 32);
+        int active = n_blocks > wm ? ceil_div(n_blocks - wm, WGM) : 0;
+        if (active > TM || MODE == MODE_DW) active = TM;
+
+        if (ct.KT == 0) {
+            // no reduction steps: an expert without rows (DW) writes zeros, a tile without rows nothing
+            if (MODE == MODE_DW) {
+                const uint4_t z = {0u, 0u, 0u, 0u};
+                for (int q = lane; q < TM * 32 * (WTN / 8); q += 64) {
+                    const int rr = q / (WTN / 8), cc = (q % (WTN / 8)) * 8;
+                    const int row = ct.i0 + (wm + WGM * (rr / 32)) * 32 + rr % 32;
+                    const int col = ct.j0 + wn * WTN + cc;
+                    __builtin_nontemporal_store(z, (uint4_t *)((bf16_t *)ct.pc + (int64_t)row * ldc + col));
+                }
+                issued += TM * 32 * (WTN / 8) / 64;
+            }
+            continue;
+        }
+
+        // The body of a tile for a wave with TA row blocks that hold rows (a wave without any multiplies one block
+        // that nobody stores): zeroing, steps, epilogue.  One instance per TA, so that blocks past the tile's last row
+        // cost no MFMA and no branch stands between the MFMAs.
+        auto tile_body = [&](auto ta_tag) {
+        constexpr int TA = decltype(ta_tag)::value;
+        floatx16 acc[TA][TN];
+        // One reduction step.  The order of the instructions inside a sub-step is pinned: a wave that is alone on
+        // its SIMD overlaps nothing by itself, and a batch of LDS reads ahead of a batch of MFMAs costs the sum of
+        // the two (the reads of a batch queue up behind those of the other three waves while the matrix unit idles).
+        // So the NM MFMAs of sub-step ks alternate with the NU fragment reads of the sub-step after it -- after the
+        // step's barrier those of the next step's first sub-step -- and in the last sub-step also with the copies of
+        // step g+SR.  A partial last step of DW multiplies all its sub-steps: rows past the end are zeros in A.
+        constexpr int NM = TA * TN, NU = TM + TN;
+        auto read_unit = [&](auto u_tag, const unsigned char *rst, int rks, int buf) {
+            constexpr int U = decltype(u_tag)::value;
+            if constexpr (U < TN)
+                fb[buf][U] = fo_b.load(rst + SA::kBytes, U, rks);
+            else
+                fa[buf][U - TN] = fo_a.load(rst, U - TN, rks);
+        };
+        // SPREAD: the copies of the producer's step between the MFMAs, issued if `on`
+        auto substep = [&](auto ks_tag, auto spread_tag, const unsigned char *rst, int rks, int slot, int on) {
+            constexpr int ks = decltype(ks_tag)::value;
+            constexpr bool SPREAD = decltype(spread_tag)::value != 0;
+            static_for<NM>([&](auto i_tag) {
+                constexpr int I = decltype(i_tag)::value, t = I / TN, bj = I % TN;
+                if (!kNoMfma)
+                    acc[t][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks & 1][bj], fa[ks & 1][t], acc[t][bj], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                // read unit u follows MFMA u * NM / NU
+                static_for<NU>([&](auto u_tag) {
+                    if constexpr (decltype(u_tag)::value * NM / NU == I) read_unit(u_tag, rst, rks, (ks + 1) & 1);
+                });
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (SPREAD) {
+                    // copy q follows MFMA q * NM / LPW
+                    static_for<LPW>([&](auto q_tag) {
+                        if constexpr (decltype(q_tag)::value * NM / LPW == I) copy_one_if(q_tag, slot, on);
+                    });
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            });
+        };
+        auto step = [&]() {
+            const unsigned char *st = stage_of(g);
+            static_for<KS - 1>([&](auto ks_tag) { substep(ks_tag, IC<0>{}, st, decltype(ks_tag)::value + 1, 0, 0); });
+            // ---- point P: my reads of this stage are done, my copies of the next step have landed
+            const bool next_exists = g + 1 < pg;
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (next_exists) wait_vmcnt_upto(issued - mark[(g + 1) % SR]);
+            __builtin_amdgcn_s_barrier();
+            // (past the workgroup's last step the reads fetch a stage nobody uses)
+            const unsigned char *nst = stage_of(g + 1);
+            bool spread = false;
+            const int slot = pg % SR;
+            if (p_more) {
+                if (prod_is_tail()) {
+                    copy_tail(slot);
+                    prod_advance();
+                } else {
+                    spread = true;
+                }
+            }
+            substep(IC<KS - 1>{}, IC<1>{}, nst, 0, slot, __builtin_amdgcn_readfirstlane(spread ? 1 : 0));
+            if (spread) prod_advance();
+            ++g;
+        };
+        {
+            // zeros from the matrix unit: 0 x 0 + 0 (one instruction per 16 registers instead of 16 moves)
+            const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            bf16x8 zf;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) zf[u] = (bf16_t)0.f;
+#pragma unroll
+            for (int t = 0; t < TA; ++t)
+#pragma unroll
+                for (int bj = 0; bj < TN; ++bj) {
+                    asm volatile("" : "+v"(zf));  // sixteen instructions, not one and fifteen copies of its result
+                    acc[t][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(zf, zf, zero, 0, 0, 0);
+                }
+        }
+        {
+            int kc = 0;  // KT >= 1 here
+#pragma unroll 1
+            do step();
+            while (++kc < ct.KT);
+        }
+
+        // ---- epilogue: a 32-row block of EPC columns at a time through the wave's own staging area (8 bytes per
+        // lane and write), then whole 16-byte pieces of rows, streaming stores
+#pragma unroll
+        for (int t = 0; t < TA; ++t) {
+            if (t >= active) continue;
+            const int row_base = ct.i0 + (wm + WGM * t) * 32;
+#pragma unroll
+            for (int part = 0; part < WTN / EPC; ++part) {
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int bq = 0; bq < EPC / 32; ++bq) {
+                    const int bj = part * (EPC / 32) + bq;
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq) {
+                        union {
+                            bf16_t e[4];
+                            uint2_t v;
+                        } pk4;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) pk4.e[u] = (bf16_t)acc_read(acc[t][bj][4 * gq + u]);
+                        *(uint2_t *)(ep + rl * EP_ROWB + (bq * 32 + 8 * gq + 4 * h) * 2) = pk4.v;
+                    }
+                }
+                // the same wave reads back what it wrote: LDS operations of one wave complete in order
+                constexpr int CPR = EPC / 8;
+#pragma unroll
+                for (int q0 = 0; q0 < 32 * CPR; q0 += 64) {
+                    // a store whose rows all lie past the tile's last one is left out, and not counted
+                    if (MODE != MODE_DW && row_base + q0 / CPR >= ct.i_end) continue;
+                    if (!kNoStore) ++issued;
+                    const int q = q0 + lane;
+                    const int row_l = q / CPR, lcol = (q % CPR) * 8;
+                    const int row = row_base + row_l;
+                    const int col = ct.j0 + wn * WTN + part * EPC + lcol;
+                    const uint4_t v = *(const uint4_t *)(ep + row_l * EP_ROWB + lcol * 2);
+                    if (!kNoStore && (MODE == MODE_DW || row < ct.i_end))
+                        __builtin_nontemporal_store(v, (uint4_t *)((bf16_t *)ct.pc + (int64_t)row * ldc + col));
+                }
+            }
+        }
+        };  // tile_body
+        if (MODE == MODE_DW)
+            tile_body(IC<TM>{});
+        else if (TM == 1 || active <= 1)
+            tile_body(IC<1>{});
+        else if (TM == 2 || active == 2)
+            tile_body(IC<(TM >= 2 ? 2 : 1)>{});
+        else if (TM == 3 || active == 3)
+            tile_body(IC<(TM >= 3 ? 3 : 1)>{});
+        else if (TM == 4 || active == 4)
+            tile_body(IC<(TM >= 4 ? 4 : 1)>{});
+        else
+            tile_body(IC<TM>{});
+    }
+}
+
+template <int MODE, int MB, int NB, int BK, int SR>
+int launch_wide(const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N, int K,
+                int E, hipStream_t stream) {
+    constexpr int STAGE_BYTES = (MB + NB) * 32 * BK * 2;
+    constexpr int WTN = NB / 2 * 32;
+    constexpr int EPC = WTN % 64 == 0 ? 64 : WTN;
+    constexpr int EP_ROWB = EPC * 2 + (EPC == 64 ? 16 : 8);
+    constexpr int LDS_BYTES = SR * STAGE_BYTES + 4 * 32 * EP_ROWB + 2 * (kMaxTableExperts + 1) * 4;
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS capacity of a CDNA4 compute unit");
+    auto kern = gemm_wide_kernel<MODE, MB, NB, BK, SR, bf16_t>;
+    static PerDeviceOnce attr;
+    const hipError_t e = attr.run(
+        [&] { return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES); });
+    if (e != hipSuccess) return (int)e;
+    const int grid = device_info().cu_count / kXcd * kXcd;
+    kern<<<grid, 256, LDS_BYTES, stream>>>((const bf16_t *)a, (const bf16_t *)b, m_sizes, ms_i64, (bf16_t *)c, R, N, K, E);
+    return launch_status();
+}
+
+}  // namespace
+
+#ifdef MFL_TUNING_BUILD
+int g_wide_variant = 0;  // 0: 320 x 192 tiles where N allows, 1: 256 x 256 tiles
+#endif
+
+int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
+                   int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream) {
+    if (out_dtype != MFL_BF16 || accumulate || alpha != 1.0f || E > kMaxTableExperts || E < 1) return MFL_ERR_UNSUPPORTED;
+    if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, 16)) return MFL_ERR_UNSUPPORTED;
+    if (mode == MODE_DW) {
+        if (N % 256 != 0 || K % 256 != 0 || N < 256 || K < 256) return MFL_ERR_UNSUPPORTED;
+        return launch_wide<MODE_DW, 8, 8, 32, 4>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
+    }
+    if (K % 64 != 0 || K < 64 || R <= 0) return R <= 0 ? MFL_OK : MFL_ERR_UNSUPPORTED;
+#ifdef MFL_TUNING_BUILD
+    const int v = g_wide_variant;
+#else
+    const int v = 0;
+#endif
+    if (v == 0 && N % 192 == 0) {
+        if (mode == MODE_FWD) return launch_wide<MODE_FWD, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
+        return launch_wide<MODE_DX, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
+    }
+    if (N % 256 != 0) return MFL_ERR_UNSUPPORTED;
+    if (mode == MODE_FWD) return launch_wide<MODE_FWD, 8, 8, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
+    return launch_wide<MODE_DX, 8, 8, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
+}
+
+}  // namespace mfl

@@ -52,8 +52,10 @@ def route_tokens(block, hidden_2d: torch.Tensor):
     """Router half of the block, shared with the fast-LoRA forward: returns
     (router_logits, routing_weights (T,k), m_sizes, sort_idx, inv_sort_idx)."""
     router_logits = block.gate(hidden_2d)
-    routing_weights, _selected, m_sizes, sort_idx, inv_sort_idx = route_and_sort(
+    routing_weights, selected, m_sizes, sort_idx, inv_sort_idx = route_and_sort(
         router_logits.contiguous(), block.num_selected, block.norm_topk_prob, hidden_2d.dtype, block.num_experts)
+    if getattr(block, "keep_routing", False):
+        block.last_selected = selected  # (T, k) expert ids of this call, as the top-k kernel wrote them
     return router_logits, routing_weights, m_sizes, sort_idx, inv_sort_idx
 
 
@@ -84,6 +86,8 @@ class Qwen3MoeFusedSparseMoeBlock(nn.Module):
     # gather + gate_proj + up_proj + SiLU-mul as one kernel when both projections are plain (or
     # plain 4-bit) expert matrices in bf16; set to False to call the two modules one by one
     fuse_front = True
+    # set to True to keep the expert ids of the last call in ``last_selected`` (tests read the block's own routing)
+    keep_routing = False
 
     def _fused_front(self, tokens, m_sizes, sort_idx, inv_sort_idx) -> Optional[torch.Tensor]:
         from .fused_mlp import moe_fused_glu, moe_fused_glu_4bit
@@ -151,10 +155,18 @@ def _hf_subclasses():
     # load-balancing loss).  Older releases read them from the block's return value and have no table.
     record = {}
     if isinstance(getattr(Qwen3MoeModel, "_can_record_outputs", None), dict):
-        from transformers.utils.output_capturing import OutputRecorder
-
-        record = {"_can_record_outputs": {**Qwen3MoeModel._can_record_outputs,
-                                          "router_logits": OutputRecorder(Qwen3MoeFusedRouter, index=0)}}
+        # the recorder class has lived in two places; without it the model classes still build and the router
+        # logits come from the block's return value only
+        OutputRecorder = None
+        for module in ("transformers.utils.output_capturing", "transformers.utils.generic"):
+            try:
+                OutputRecorder = getattr(__import__(module, fromlist=["OutputRecorder"]), "OutputRecorder")
+                break
+            except (ImportError, AttributeError):
+                continue
+        if OutputRecorder is not None:
+            record = {"_can_record_outputs": {**Qwen3MoeModel._can_record_outputs,
+                                              "router_logits": OutputRecorder(Qwen3MoeFusedRouter, index=0)}}
 
     class Qwen3MoeFusedModel(Qwen3MoeModel):
         locals().update(record)
