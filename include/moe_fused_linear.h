@@ -300,7 +300,10 @@ MFL_API int mfl_expert_sort(const void *sel, int sel_dtype, int64_t R, int E, in
  * allocates nothing, on the device or through any library.  Limit: E <= 512 (any R up to
  * 2^31 - 1); beyond it the call returns MFL_ERR_LIMIT with nothing enqueued.  All calls on one
  * GPU share that GPU's array: calls that may overlap in time on one GPU (different streams,
- * different threads) race and must be serialised by the caller; calls on one stream are safe. */
+ * different threads) race and must be serialised by the caller; calls on one stream are safe.
+ * The first call on a device looks up the array's address and sets the kernels' launch attributes
+ * there (runtime calls that do not belong inside a stream capture): make one call per device
+ * before any capture that contains this entry point. */
 MFL_API int mfl_expert_sort_static(const void *sel, int sel_dtype, int64_t R, int E, int32_t *counts,
                            int32_t *sort_idx, int32_t *inv_sort_idx, void *stream);
 

@@ -253,6 +253,32 @@ def test_route_and_sort_equals_the_separate_calls(T, E, k, dtype):
     _check_route_outputs(logits, k, E, w, sel, m_sizes, sort_idx, inv)
 
 
+@pytest.mark.parametrize("T", [200, 4096])
+def test_route_and_sort_with_a_row_of_nan(T):
+    """A token whose logits are all NaN selects no expert (no probability compares greater than another): its
+    k selections are left out of the counts and of the sort, and every other token is routed as without it.
+    The histogram pass of the two-launch form must not count the row's "no expert" id."""
+    from qwen3_moe_fused.kernels.routing import route_and_sort
+
+    E, k, bad = 128, 8, T // 3
+    clean = randn((T, E), gen(T), 2.0, torch.float32)
+    logits = clean.clone()
+    logits[bad] = float("nan")
+    w, sel, m_sizes, sort_idx, inv = route_and_sort(logits.to(DEV), k, True, torch.float32, E)
+    torch.cuda.synchronize()
+    keep = np.ones(T, bool)
+    keep[bad] = False
+    _, sel_ref = oracle.softmax_topk(clean.numpy()[keep], k, True)
+    assert np.array_equal(sel.cpu().numpy()[keep], sel_ref), "the other tokens are routed as without the row"
+    counts_ref = oracle.expert_counts(sel_ref.reshape(-1), E)
+    assert np.array_equal(m_sizes.cpu().numpy(), counts_ref) and int(m_sizes.sum()) == (T - 1) * k
+    # the sorted positions of the other tokens' selections are those of the stable sort without the row
+    flat_keep = np.repeat(keep, k)
+    _, s_ref, _ = oracle.expert_counts_and_idx(sel_ref.reshape(-1), E)
+    orig = np.nonzero(flat_keep)[0]
+    assert np.array_equal(sort_idx.cpu().numpy()[: (T - 1) * k], orig[s_ref])
+
+
 @pytest.mark.parametrize("T,E,k", [(128, 128, 8), (100, 512, 6), (65, 40, 5)])
 def test_one_launch_entry_point_up_to_its_own_limit(T, E, k):
     # mfl_route_sort uses the one-workgroup form up to 64 tokens; the entry point itself takes up to 128

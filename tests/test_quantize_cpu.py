@@ -149,3 +149,60 @@ def test_quantizer_hook_swaps_fused_modules_and_respects_the_skip_list():
         assert "layers.1.down_proj" in quantizer.modules_to_not_convert
     finally:
         Bnb4BitHfQuantizer._process_model_before_weight_loading = original
+
+
+def test_quantizer_operations_build_the_librarys_own_parameters():
+    """The installed transformers release routes checkpoint tensors through the quantizer's conversion
+    operations, not through ``_load_from_state_dict``: after ``patch_bnb_quantizer`` those operations turn a
+    fused module's tensors into ``Nf4Params`` (a float tensor: still to be quantised on the CPU; a packed one
+    with its bitsandbytes-named entries: with its quant state) and never touch bitsandbytes for them."""
+    pytest.importorskip("transformers")
+    from transformers import BitsAndBytesConfig
+    from transformers.quantizers.quantizer_bnb_4bit import Bnb4BitHfQuantizer
+
+    from qwen3_moe_fused.quantize.layer import Nf4Params
+    from qwen3_moe_fused.quantize.nf4 import Nf4QuantState, code_of
+    from qwen3_moe_fused.quantize.quantizer import patch_bnb_quantizer
+
+    if not hasattr(Bnb4BitHfQuantizer, "get_quantize_ops"):
+        pytest.skip("this transformers release loads through _load_from_state_dict")
+    saved = {n: getattr(Bnb4BitHfQuantizer, n) for n in ("_process_model_before_weight_loading", "param_needs_quantization",
+                                                         "get_quantize_ops", "get_weight_conversions")}
+    try:
+        patch_bnb_quantizer()
+        cfg = BitsAndBytesConfig(load_in_4bit=True, bnb_4bit_quant_type="nf4", bnb_4bit_use_double_quant=False,
+                                 bnb_4bit_compute_dtype=torch.bfloat16, llm_int8_skip_modules=["lm_head"])
+        quantizer = Bnb4BitHfQuantizer(cfg)
+        model = _tiny_model()
+        quantizer._process_model_before_weight_loading(model, device_map=None)
+        name = "layers.0.gate_proj.weight"
+        module = model.layers[0].gate_proj
+
+        # a floating-point checkpoint: one tensor per parameter through the quantize operation
+        w = torch.randn(4, 8, 16)
+        out = quantizer.get_quantize_ops().convert({name: [w]}, full_layer_name=name, model=model)
+        assert set(out) == {name} and isinstance(out[name], Nf4Params)
+        assert out[name].quant_state is None and torch.equal(out[name].data, w)       # quantised on reaching the GPU
+        assert out[name].quant_type == "nf4" and out[name].module is module
+
+        # a pre-quantised checkpoint: packed bytes and bitsandbytes' entries through the deserialise operation
+        quantizer.pre_quantized = True
+        converters = quantizer.get_weight_conversions()
+        assert len(converters) == 1
+        op = converters[0].operations[0]
+        state = Nf4QuantState(absmax=torch.rand(4 * 8 * 16 // 64) + 0.5, shape=(4, 8, 16), code=code_of("nf4", "cpu"),
+                              blocksize=64, quant_type="nf4", dtype=torch.bfloat16)
+        packed = torch.randint(0, 256, (4 * 8 * 16 // 2, 1), dtype=torch.uint8)
+        entries = {"weight." + k: [v] for k, v in state.as_dict(packed=True).items()}
+        entries["weight"] = [packed]
+        got = op.convert(entries, model=model, full_layer_name=name)
+        assert set(got) == {"weight"} and isinstance(got["weight"], Nf4Params)
+        qs = got["weight"].quant_state
+        assert qs is not None and tuple(qs.shape) == (4, 8, 16) and qs.blocksize == 64 and qs.quant_type == "nf4"
+        assert torch.equal(qs.absmax, state.absmax) and torch.equal(got["weight"].data, packed)
+        assert module.quant_state is qs
+    finally:
+        for n, f in saved.items():
+            setattr(Bnb4BitHfQuantizer, n, f)
+        if hasattr(Bnb4BitHfQuantizer, "_mfl_stock_ops"):
+            del Bnb4BitHfQuantizer._mfl_stock_ops

@@ -1,7 +1,9 @@
 """The entry point that allocates nothing (mfl_expert_sort_static) against mfl_expert_sort, through
 the C ABI: same counts, sort_idx and inv_sort_idx bit for bit, on two calls in a row, the second
 with a smaller input (the library's fixed table array keeps the first call's contents), and on a
-call after other work has used the GPU."""
+call after other work has used the GPU.  "Allocates nothing" is read from the driver (free device memory
+before and after a call, once the first call on the device has looked up the array's address and set the
+kernels' attributes) as well as from torch's allocator, which would not see a hipMalloc inside the library."""
 import numpy as np
 import pytest
 import torch
@@ -53,8 +55,13 @@ def test_static_sort_matches_workspace_sort_on_two_calls_in_a_row():
         # outputs are allocated before the call; between here and the comparison the static call allocates nothing
         outs = (torch.empty(E, dtype=torch.int32, device=DEV), torch.empty(R, dtype=torch.int32, device=DEV),
                 torch.empty(R, dtype=torch.int32, device=DEV))
+        _sort_static(sel, E, outs)          # the first call on a device does the one-time set-up
+        torch.cuda.synchronize()
         before = torch.cuda.memory_stats()["allocation.all.allocated"]
+        free_before = torch.cuda.mem_get_info()[0]
         got = _sort_static(sel, E, outs)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated during the call"
         assert torch.cuda.memory_stats()["allocation.all.allocated"] == before, "torch allocated during the call"
         ref = _sort_with_workspace(sel, E)
         for a, b, name in zip(got, ref, ("counts", "sort_idx", "inv_sort_idx")):

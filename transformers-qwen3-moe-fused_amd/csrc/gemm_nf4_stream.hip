@@ -96,11 +96,10 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     using S = StreamShape<GLU>;
     constexpr int CB = S::CB, RING = S::RING;
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
-    // the pair table first, at LDS address 0 (the kernel has no static LDS): a lookup's address is then the shifted
+    // the pair table first, at LDS address 0 (the kernel has no static LDS, which the launcher checks): a lookup's address is then the shifted
     // byte itself plus a constant that fits the instruction's offset field, no add
     unsigned char *const table = smem;
     unsigned char *const ring = smem + S::kTable;
-    if ((uint32_t)(uintptr_t)(lds_void_ptr)smem != 0) __builtin_trap();
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
@@ -325,10 +324,19 @@ int launch_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf
     if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
     auto *kernel = nf4_stream_kernel<GLU, TO>;
     static PerDeviceOnce attr;
+    // The kernel's table lookups take the dynamic LDS to start at address 0: any static LDS in this kernel
+    // (a later __shared__ variable, an inlined helper that brings one) would move it, so the launcher asks the
+    // runtime once and leaves such a build to the register-decoding kernel.
+    static std::atomic<int> static_lds{-1};
     const hipError_t e = attr.run([&] {
+        hipFuncAttributes fa;
+        const hipError_t e1 = hipFuncGetAttributes(&fa, (const void *)kernel);
+        if (e1 != hipSuccess) return e1;
+        static_lds.store((int)fa.sharedSizeBytes, std::memory_order_release);
         return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     });
     if (e != hipSuccess) return (int)e;
+    if (static_lds.load(std::memory_order_acquire) != 0) return MFL_ERR_UNSUPPORTED;
     kernel<<<(unsigned)grid, 256, kLds, stream>>>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, y, e_out, g_out,
                                                           R, N, K, E, tiles_n);
     return launch_status();

@@ -651,7 +651,9 @@ __global__ __launch_bounds__(1024) void route_count_kernel(const TI *__restrict_
         const int64_t t = (int64_t)blockIdx.x * tokens_per_seg + tt;
         if (t >= T) break;
         const int sel = topk_one_token<TI, TC, VPL>(logits, t, E, k, renorm, w_f32, w_cast, idx, lane);
-        if (lane < k) atomicAdd(&lds[sel], 1);
+        // a row of NaN (or of -inf throughout) selects nothing: its lanes keep the "no expert" id, which the
+        // scatter pass skips like any key outside [0, E); it must not reach the histogram either
+        if (lane < k && (unsigned)sel < (unsigned)E) atomicAdd(&lds[sel], 1);
     }
     __syncthreads();
     for (int i = threadIdx.x; i < E; i += blockDim.x) table_raw[(int64_t)blockIdx.x * E + i] = lds[i];

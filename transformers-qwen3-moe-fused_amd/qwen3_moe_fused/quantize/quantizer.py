@@ -115,10 +115,97 @@ def _param_needs_quantization(self, model, param_name: str, **kwargs) -> bool:
     return Linear4bit is not None and isinstance(module, Linear4bit) and name != "bias"
 
 
+def _first(value):
+    return value[0] if isinstance(value, (list, tuple)) else value
+
+
+def _conversion_ops():
+    """The two weight-loading operations of the installed transformers release (its loader hands every
+    checkpoint tensor of a parameter that ``param_needs_quantization`` names to the quantizer's operation, and
+    the entries of a pre-quantised parameter to its deserialising one), extended to the fused modules.  The
+    stock operations build bitsandbytes' ``Params4bit``; for a ``MoeFusedLinear4bit`` these build the library's
+    own ``Nf4Params`` instead and leave every other module to the stock operation."""
+    from transformers.core_model_loading import ConversionOps
+    from transformers.quantizers.quantizers_utils import get_module_from_name
+
+    from .layer import Nf4Params
+    from .nf4 import Nf4QuantState
+
+    class FusedQuantize(ConversionOps):
+        """A floating-point (E, out, in) checkpoint tensor becomes an ``Nf4Params`` that is quantised on the
+        device it was loaded to (on the CPU: when the module first reaches the GPU)."""
+
+        def __init__(self, hf_quantizer, stock):
+            self.hf_quantizer, self.stock = hf_quantizer, stock
+
+        def convert(self, input_dict, full_layer_name=None, model=None, **kwargs):
+            result, rest = {}, {}
+            for param_name, value in input_dict.items():
+                module, _ = get_module_from_name(model, param_name)
+                if not isinstance(module, MoeFusedLinear4bit):
+                    rest[param_name] = value
+                    continue
+                value = _first(value)
+                old = module.weight
+                new = Nf4Params(value.contiguous(), blocksize=old.blocksize, module=module, quant_type=old.quant_type,
+                                compress_statistics=old.compress_statistics)
+                if value.is_cuda:
+                    new = new.to(value.device)
+                module._is_hf_initialized = True
+                result[param_name] = new
+            if rest:
+                result.update(self.stock.convert(rest, full_layer_name=full_layer_name, model=model, **kwargs))
+            return result
+
+    class FusedDeserialize(ConversionOps):
+        """The packed weight of a pre-quantised checkpoint with its quant-state entries (bitsandbytes' names:
+        ``absmax``, ``quant_map``, ``nested_absmax``, ``nested_quant_map``, ``quant_state.bitsandbytes__nf4``)."""
+
+        def __init__(self, hf_quantizer, stock):
+            self.hf_quantizer, self.stock = hf_quantizer, stock
+
+        def convert(self, input_dict, model=None, full_layer_name=None, **kwargs):
+            module, _ = get_module_from_name(model, full_layer_name)
+            if not isinstance(module, MoeFusedLinear4bit):
+                return self.stock.convert(input_dict, model=model, full_layer_name=full_layer_name, **kwargs)
+            if len(input_dict) == 1:
+                return input_dict
+            entries = {key: _first(value) for key, value in input_dict.items()}
+            packed = entries.pop("weight")
+            state = Nf4QuantState.from_dict({k.split("weight.", 1)[-1]: v for k, v in entries.items()},
+                                            device=packed.device)
+            new = Nf4Params(packed.reshape(-1, 1).contiguous(), quant_state=state, blocksize=int(state.blocksize),
+                            module=module, quant_type=state.quant_type, compress_statistics=state.nested)
+            module.quant_state = state
+            module._is_hf_initialized = True
+            return {"weight": new}
+
+    return FusedQuantize, FusedDeserialize
+
+
 def patch_bnb_quantizer() -> None:
-    """quantizer.py:132-133 of the reference."""
+    """quantizer.py:132-133 of the reference, plus what the installed transformers release needs beyond the
+    module swap: which parameters its loader sends through the quantizer, and the two operations that turn
+    checkpoint tensors into parameters (releases without them load through ``_load_from_state_dict``)."""
     from transformers.quantizers.quantizer_bnb_4bit import Bnb4BitHfQuantizer
 
     Bnb4BitHfQuantizer._process_model_before_weight_loading = _process_model_before_weight_loading
     if hasattr(Bnb4BitHfQuantizer, "param_needs_quantization"):
         Bnb4BitHfQuantizer.param_needs_quantization = _param_needs_quantization
+    if hasattr(Bnb4BitHfQuantizer, "get_quantize_ops") and not hasattr(Bnb4BitHfQuantizer, "_mfl_stock_ops"):
+        FusedQuantize, FusedDeserialize = _conversion_ops()
+        stock_quantize, stock_conversions = Bnb4BitHfQuantizer.get_quantize_ops, Bnb4BitHfQuantizer.get_weight_conversions
+        Bnb4BitHfQuantizer._mfl_stock_ops = (stock_quantize, stock_conversions)
+
+        def get_quantize_ops(self):
+            return FusedQuantize(self, stock_quantize(self))
+
+        def get_weight_conversions(self):
+            converters = stock_conversions(self)
+            for converter in converters:
+                converter.operations = [FusedDeserialize(self, op) if type(op).__name__ == "Bnb4bitDeserialize" else op
+                                        for op in converter.operations]
+            return converters
+
+        Bnb4BitHfQuantizer.get_quantize_ops = get_quantize_ops
+        Bnb4BitHfQuantizer.get_weight_conversions = get_weight_conversions
