@@ -60,6 +60,82 @@ def _event_us_median(fn, iters, warm, stream, blocks=5):
     return runs[len(runs) // 2]
 
 
+def _per_launch_us(fn, iters, warm, stream):
+    """Time of every launch of a loop by its own pair of events: (median, 20 % quantile, 80 % quantile), the
+    figures the reference's benchmarks report (do_bench(quantiles=[0.5, 0.2, 0.8]),
+    benchmark_moe_fused_linear.py:56-59)."""
+    import torch
+
+    for i in range(warm):
+        fn(i)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    torch.cuda.synchronize()
+    for i, (a, b) in enumerate(evs):
+        a.record(stream)
+        fn(i)
+        b.record(stream)
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)
+    return ts[len(ts) // 2], ts[len(ts) // 5], ts[len(ts) * 4 // 5]
+
+
+def _reference_sweep(dev, stream, ws, qsets):
+    """The reference's own benchmark definition (benchmark_moe_fused_linear.py:27-28,43-61, _bwd_dx.py:44-60,
+    _bwd_dw.py:42-58, _4bit.py:51-69): rows 1024 ... 16384 in steps of 1024, every row's expert drawn
+    uniformly, in_features 2048, out_features 768, 128 experts, bf16; forward, input gradient, weight gradient
+    and the 4-bit forward.  Per point: median and 20 / 80 % quantiles over per-launch event times, TFLOP/s
+    (two flops per multiply-add), and the fraction of the 8 TB/s HBM peak that the algorithmic bytes of the
+    point (each operand read once, the output written once) amount to at the median."""
+    import torch
+
+    from qwen3_moe_fused.grouped_gemm.backward_dw import grouped_gemm_backward_dw
+    from qwen3_moe_fused.grouped_gemm.forward import grouped_gemm_forward
+    from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_4bit
+    from qwen3_moe_fused.grouped_gemm.forward_transposed import grouped_gemm_forward_transposed
+
+    NB = len(ws)
+    g = torch.Generator().manual_seed(1)
+    rmax = 16384
+    x = torch.randn((rmax, HIDDEN), device=dev, dtype=torch.bfloat16)
+    dy = torch.randn((rmax, INTER), device=dev, dtype=torch.bfloat16)
+    points = []
+    wbytes = 2.0 * E * INTER * HIDDEN
+    iters, warm = 60, 20
+    # one long untimed burst first: the board's power management settles after about 150 launches
+    ms0 = torch.bincount(torch.randint(0, E, (rmax,), generator=g), minlength=E).to(torch.int32).to(dev)
+    for i in range(MIN_WARMUP):
+        grouped_gemm_forward(x, ws[i % NB], ms0)
+    for rows in range(1024, rmax + 1, 1024):
+        ms = torch.bincount(torch.randint(0, E, (rows,), generator=g), minlength=E).to(torch.int32).to(dev)
+        xr, dyr = x[:rows], dy[:rows]
+        flop = 2.0 * rows * INTER * HIDDEN
+        io = 2.0 * rows * (HIDDEN + INTER)
+        legs = {
+            "fwd": (lambda i: grouped_gemm_forward(xr, ws[i % NB], ms), io + wbytes),
+            "dx": (lambda i: grouped_gemm_forward_transposed(dyr, ws[i % NB], ms), io + wbytes),
+            "dw": (lambda i: grouped_gemm_backward_dw(xr, dyr, ms, torch.bfloat16), io + wbytes),
+            "fwd_4bit": (lambda i: grouped_gemm_forward_4bit(xr, *qsets[i % NB], ms),
+                         io + E * INTER * HIDDEN * (0.5 + 4.0 / 64)),
+        }
+        point = {"rows": rows}
+        for name, (fn, nbytes) in legs.items():
+            med, q20, q80 = _per_launch_us(fn, iters, warm, stream)
+            point[name] = {"us": round(med, 1), "us_q20": round(q20, 1), "us_q80": round(q80, 1),
+                           "tflops": round(flop / med / 1e6, 1), "gbs": round(nbytes / med / 1e3, 1),
+                           "hbm_frac": round(nbytes / med / 1e3 / PEAK_HBM_GBS, 4)}
+        points.append(point)
+    # largest step in achieved GB/s between neighbouring points, per product (a cliff marks a bad switch of
+    # tile configurations)
+    jumps = {}
+    for name in ("fwd", "dx", "dw", "fwd_4bit"):
+        gb = [p[name]["gbs"] for p in points]
+        jumps[name] = round(max(abs(b - a) / max(a, b) for a, b in zip(gb, gb[1:])), 3)
+    return {"definition": "rows 1024..16384 step 1024, uniform random experts, in 2048, out 768, 128 experts, bf16; "
+                          "median / 20 % / 80 % of 60 per-launch event times after 20 warm launches; "
+                          "three weight sets in rotation",
+            "points": points, "largest_neighbour_step_in_gbs": jumps}
+
+
 def _kernel_tour(n, dev):
     """N launches of each hot kernel at the shapes of configurations 2, 3 and 5, in a fixed order, with a line
     per kernel that states its algorithmic bytes and flops per launch.  Nothing is timed: counter passes
@@ -314,6 +390,11 @@ def main() -> int:
                                            "mfma_frac": round(flop / us / 1e6 / PEAK_BF16_TFLOPS, 4),
                                            "algorithmic_bytes": gb, "hbm_frac": round(gb / us / 1e3 / PEAK_HBM_GBS, 4)}
         del toks
+        # the down projection's forward product (N = 2048, K = 768): same flops and bytes as gate_proj
+        us = _event_us(lambda i: grouped_gemm_forward(hs[i % NB], wd[i % NB], m_sizes, out=dys[i % NB]), args.steps,
+                       wm, stream)
+        extra["fwd_down_proj"] = dict(workload="down_proj forward, h (32768, 768) x w (128, 2048, 768)",
+                                      **product_line(us))
         us = _event_us(lambda i: silu_mul_forward(hs[i % NB], hs[(i + 1) % NB]), it, wm, stream)
         b = 3.0 * ROWS * INTER * 2
         extra["silu_mul_fwd"] = {"us": round(us, 1), "gbs": round(b / us / 1e3, 1), "hbm_frac": round(b / us / 1e3 / PEAK_HBM_GBS, 4)}
@@ -377,6 +458,7 @@ def main() -> int:
         extra["nf4_gate_proj_dx"] = {"fused_us": round(us_f, 1), "dequant_then_gemm_us": round(us_u, 1),
                                      "fused_tflops": round(flop / us_f / 1e6, 1)}
         del dyg
+        extra["sweep"] = _reference_sweep(dev, stream, ws, qsets)
         del packed, qstate, qsets, x5
         # config 4: rank-16 LoRA on gate_proj, 8192 tokens, Zipf(1.2)-skewed top-8 routing (65536 rows):
         # the frozen base product and the five thin products of one forward + backward

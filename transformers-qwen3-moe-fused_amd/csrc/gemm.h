@@ -6,6 +6,22 @@ namespace mfl {
 
 enum { MODE_FWD = 0, MODE_DX = 1, MODE_DW = 2 };
 
+// Average rows per expert up to which the row-grouped bf16 products run on flat 64 x 128 tiles (the weights are all
+// the traffic there; measured cross-over against the 320 x 192 tiles between 48 and 64 rows per expert), and up to
+// which the packed-weight forward runs on the streaming / register-decoding kernels instead of the pipelined one
+// (gate_proj shape, 128 experts, uniform routing: 68 / 65 / 80 us streaming against 105 / 98 / 95 us pipelined at
+// 40 / 48 / 64 rows per expert, 104 against 95 us at 80).
+#if defined(MFL_TUNING_BUILD) && defined(MFL_X_FLAT_ROWS)
+constexpr int kFlatTileRowsPerExpert = MFL_X_FLAT_ROWS;
+#else
+constexpr int kFlatTileRowsPerExpert = 48;
+#endif
+#if defined(MFL_TUNING_BUILD) && defined(MFL_X_NF4_ROWS)
+constexpr int kNf4DecodeRowsPerExpert = MFL_X_NF4_ROWS;
+#else
+constexpr int kNf4DecodeRowsPerExpert = 72;
+#endif
+
 // Any shape / any float type; plain FMA.
 int gemm_generic(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
                  int K, int E, int in_dtype, int out_dtype, float alpha, int accumulate, hipStream_t stream);

@@ -1028,13 +1028,13 @@ int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, i
     const bool glu = fusion != nullptr && fusion->b2 != nullptr && fusion->a2 == nullptr;
     int cfg = g_pipe_config;
     if (glu && (cfg == 0 || nf4 != nullptr)) {
-        cfg = R >= (int64_t)512 * E ? 8 : (R <= (int64_t)32 * E && nf4 == nullptr) ? 15 : 3;
+        cfg = R >= (int64_t)512 * E ? 8 : (R <= (int64_t)kFlatTileRowsPerExpert * E && nf4 == nullptr) ? 15 : 3;
     } else if (cfg == 0 || nf4 != nullptr) {
         if (mode == MODE_DW)
             cfg = (N <= 64 || K <= 64) ? 11 : 8;
         else
             cfg = (N <= 64 && nf4 == nullptr) ? 10
-                  : (R <= (int64_t)32 * E && nf4 == nullptr) ? 15
+                  : (R <= (int64_t)kFlatTileRowsPerExpert * E && nf4 == nullptr) ? 15
                   : R >= (int64_t)512 * E ? 8 : 3;
     }
     switch (cfg) {
@@ -1149,9 +1149,9 @@ int gemm_nf4_pipe(const void *x, const uint8_t *wq, const float *code16, const f
     while ((1 << shift) < blocksize) ++shift;
     // a 16-byte LDS chunk (8 weights along K) must not straddle two absmax blocks
     if (K % 64 != 0 || N % 8 != 0 || N < 8 || blocksize < 8) return MFL_ERR_UNSUPPORTED;
-    // With a handful of rows per expert the 128 x 128 tiles of the register-staged kernel spread
-    // the weight stream over more workgroups; measured cross-over near 32 rows per expert.
-    if (R < (int64_t)32 * E && fusion == nullptr) return MFL_ERR_UNSUPPORTED;
+    // With few rows per expert the streaming kernel (32-row tiles, weights decoded once per tile from packed
+    // bytes in LDS) is ahead; the caller tries it first.
+    if (R < (int64_t)kNf4DecodeRowsPerExpert * E && fusion == nullptr) return MFL_ERR_UNSUPPORTED;
     if (!aligned(x, 16) || !aligned(wq, 4) || !aligned(y, 16)) return MFL_ERR_UNSUPPORTED;
     if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
     FwdFusion fu;

@@ -104,6 +104,54 @@ __device__ __forceinline__ void wide_copy_if(const unsigned char *src, uint32_t 
             : "memory", "scc");
 }
 
+// Up to four copies of the wave as one statement: 16 bytes per lane each, from base + voff[q] + q * 1024 (the
+// instruction's offset field, which the hardware adds to the global and to the LDS address alike) to the 1 KiB
+// of LDS at lds_addr + q * 1024.  One M0 write for the group, no vector-ALU instruction; issued if `on`
+// (wave-uniform).  The callers fold "- q * 1024 + kCopyBias" into voff and "- kCopyBias" into base.
+constexpr int kCopyBias = 4096;
+#define MFL_WC_HEAD "s_cmp_eq_u32 %[on], 0\n\ts_cbranch_scc1 .Lwg_skip_%=\n\ts_mov_b32 m0, %[lds]\n\ts_nop 0\n\t"
+#define MFL_WC_LOAD(V, OFF, NT) "global_load_lds_dwordx4 %[" V "], %[base] offset:" OFF NT "\n\t"
+#define MFL_WC_TAIL ".Lwg_skip_%=:"
+template <int POLICY>
+__device__ __forceinline__ void wide_copy4(uint64_t base, uint32_t v0, uint32_t v1, uint32_t v2, uint32_t v3,
+                                           uint32_t lds_addr, int on) {
+    on = __builtin_amdgcn_readfirstlane(on);  // wave-uniform by construction; the statement needs scalar registers
+    if constexpr (kNoCopy)
+        asm volatile("s_nop 0" : : [base] "s"(base), [v0] "v"(v0), [v1] "v"(v1), [v2] "v"(v2), [v3] "v"(v3),
+                     [lds] "s"(lds_addr), [on] "s"(on) : "memory");
+    else if constexpr (POLICY == 2)
+        asm volatile(MFL_WC_HEAD MFL_WC_LOAD("v0", "0", " nt") MFL_WC_LOAD("v1", "1024", " nt")
+                     MFL_WC_LOAD("v2", "2048", " nt") MFL_WC_LOAD("v3", "3072", " nt") MFL_WC_TAIL
+                     : : [base] "s"(base), [v0] "v"(v0), [v1] "v"(v1), [v2] "v"(v2), [v3] "v"(v3), [lds] "s"(lds_addr),
+                     [on] "s"(on) : "memory", "scc");
+    else
+        asm volatile(MFL_WC_HEAD MFL_WC_LOAD("v0", "0", "") MFL_WC_LOAD("v1", "1024", "") MFL_WC_LOAD("v2", "2048", "")
+                     MFL_WC_LOAD("v3", "3072", "") MFL_WC_TAIL
+                     : : [base] "s"(base), [v0] "v"(v0), [v1] "v"(v1), [v2] "v"(v2), [v3] "v"(v3), [lds] "s"(lds_addr),
+                     [on] "s"(on) : "memory", "scc");
+}
+template <int POLICY>
+__device__ __forceinline__ void wide_copy2(uint64_t base, uint32_t v0, uint32_t v1, uint32_t lds_addr, int on) {
+    on = __builtin_amdgcn_readfirstlane(on);
+    if constexpr (kNoCopy)
+        asm volatile("s_nop 0" : : [base] "s"(base), [v0] "v"(v0), [v1] "v"(v1), [lds] "s"(lds_addr), [on] "s"(on) : "memory");
+    else if constexpr (POLICY == 2)
+        asm volatile(MFL_WC_HEAD MFL_WC_LOAD("v0", "0", " nt") MFL_WC_LOAD("v1", "1024", " nt") MFL_WC_TAIL
+                     : : [base] "s"(base), [v0] "v"(v0), [v1] "v"(v1), [lds] "s"(lds_addr), [on] "s"(on) : "memory", "scc");
+    else
+        asm volatile(MFL_WC_HEAD MFL_WC_LOAD("v0", "0", "") MFL_WC_LOAD("v1", "1024", "") MFL_WC_TAIL
+                     : : [base] "s"(base), [v0] "v"(v0), [v1] "v"(v1), [lds] "s"(lds_addr), [on] "s"(on) : "memory", "scc");
+}
+#undef MFL_WC_HEAD
+#undef MFL_WC_LOAD
+#undef MFL_WC_TAIL
+
+// a 64-bit value that is the same in every lane, held in scalar registers
+__device__ __forceinline__ uint64_t uniform64(uint64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
+
 // One accumulator element, fetched from its accumulation register where the statement stands.  (Left to itself
 // the compiler copies all 256 of a tile into vector registers at the top of the epilogue, and spills what else
 // is live there: the fragments and addresses of the next tile's first step.)
@@ -249,15 +297,30 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     const int64_t step_a = A_RC ? (int64_t)BK * 2 : (int64_t)BK * lda * 2;
     const int64_t step_b = B_RC ? (int64_t)BK * 2 : (int64_t)BK * ldb * 2;
 
-    // ---- producer: the (tile, step) whose copies are issued next
+    // ---- producer: the (tile, step) whose copies are issued next.  A step's copies go out in groups of up to
+    // four (one statement, one M0 write, scalar base + per-lane 32-bit offset + the instruction's offset field).
+    static_assert(LA % 2 == 0 && LB % 2 == 0, "copy groups hold two or four copies");
+    constexpr int GA = (LA + 3) / 4, GB = (LB + 3) / 4, NG = GA + GB;  // groups per step: A's first, then B's
+    // With three stages or more a step's copies have two steps to land: the second half of the groups goes out in
+    // the first sub-step of the consumer's next step, so that no sub-step carries more than half of them.
+    constexpr bool SPLIT = SR >= 3 && NG >= 2;
+    constexpr int NG1 = SPLIT ? (NG + 1) / 2 : NG;  // groups in the sub-step after point P
     Tile pt;
-    int pL = L_first, pk = 0;
+    int pL = L_first, pk = 0, p_full = 0;  // p_full: steps of the producer's tile that are whole
     bool p_more = false;
-    uint32_t lane_off[LPW];
+    uint64_t pa_cur = 0, pb_cur = 0;  // operand addresses of the producer's step, minus kCopyBias
+    uint32_t lane_off[LPW];           // per-lane source offsets of the wave's copies (tile origin, step 0)
+    uint32_t voff[LPW];               // the same, prepared for the grouped copies
+    auto prep_voff = [&](int q0, int q1) {
+#pragma unroll
+        for (int q = 0; q < LPW; ++q)
+            if (q >= q0 && q < q1) voff[q] = lane_off[q] + kCopyBias - ((q < LA ? q : q - LA) % 4) * 1024;
+    };
     auto prod_offsets = [&]() {
         const int i_lim = pt.i_end - pt.i0 < BM ? pt.i_end - pt.i0 : BM;
 #pragma unroll
         for (int q = 0; q < LA; ++q) lane_off[q] = (uint32_t)lane_src_offset<BM, BK, A_RC>(wave * LA + q, lane, lda, i_lim);
+        prep_voff(0, LA);
     };
     auto prod_seek = [&]() {  // first tile from pL on that has steps
         p_more = false;
@@ -271,6 +334,9 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
             pL += per_xcd;
         }
         pk = 0;
+        p_full = MODE == MODE_DW ? pt.red / BK : pt.KT;
+        pa_cur = uniform64((uint64_t)(uintptr_t)pt.pa - kCopyBias);
+        pb_cur = uniform64((uint64_t)(uintptr_t)pt.pb - kCopyBias);
     };
 #pragma unroll
     for (int q = 0; q < LB; ++q) lane_off[LA + q] = (uint32_t)lane_src_offset<BN, BK, B_RC>(wave * LB + q, lane, ldb, BN);
@@ -278,90 +344,111 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
 #pragma unroll
         for (int q = 0; q < LA; ++q) lane_off[q] = (uint32_t)lane_src_offset<BM, BK, A_RC>(wave * LA + q, lane, lda, BM);
     }
+    prep_voff(0, LPW);
     prod_seek();
 
-    int issued = 0;  // vector-memory operations this wave has issued
-    int mark[SR];    // `issued` after the last copy into ring slot s
+    // `issued` counts the vector-memory operations of this wave (copies and output stores); mark[s] is its value
+    // after the last copy into ring slot s.
+    unsigned issued = 0, pg = 0;  // pg: steps whose copies have been issued
+    unsigned mark[SR];
 #pragma unroll
     for (int s = 0; s < SR; ++s) mark[s] = 0;
-    int pg = 0;  // steps whose copies have been issued
     const uint32_t ring_lds = (uint32_t)(uintptr_t)(lds_void_ptr)smem;
+    const uint32_t wave_a_lds = ring_lds + wave * LA * 1024, wave_b_lds = ring_lds + SA::kBytes + wave * LB * 1024;
 
     // Cache policy: the weights of the row-grouped products are read by one workgroup per column slice
     // (non-temporal, the L2 is left to the rows); DW: both panels are shared by the tiles of an expert.
+#if defined(MFL_TUNING_BUILD) && defined(MFL_X_DW_POLICY)
+    constexpr int A_POLICY = MODE == MODE_DW ? (MFL_X_DW_POLICY & 1) * 2 : 0;
+    constexpr int B_POLICY = MODE == MODE_DW ? (MFL_X_DW_POLICY >> 1) * 2 : 2;
+#else
     constexpr int A_POLICY = 0;
     constexpr int B_POLICY = MODE == MODE_DW ? 0 : 2;
+#endif
 
-    // the q-th copy of the wave for the producer's step into ring slot `slot`; full steps only
-    auto copy_one = [&](auto q_tag, int slot) {
-        constexpr int q = decltype(q_tag)::value;
-        const uint32_t st = ring_lds + slot * STAGE_BYTES;
-        if constexpr (q < LA)
-            wide_copy<A_POLICY>(pt.pa + pk * step_a + lane_off[q], st + (wave * LA + q) * 1024);
-        else
-            wide_copy<B_POLICY>(pt.pb + pk * step_b + lane_off[q], st + SA::kBytes + (wave * LB + (q - LA)) * 1024);
-    };
-    auto copy_one_if = [&](auto q_tag, int slot, int on) {
-        constexpr int q = decltype(q_tag)::value;
-        const uint32_t st = ring_lds + slot * STAGE_BYTES;
-        if constexpr (q < LA)
-            wide_copy_if<A_POLICY>(pt.pa + pk * step_a + lane_off[q], st + (wave * LA + q) * 1024, on);
-        else
-            wide_copy_if<B_POLICY>(pt.pb + pk * step_b + lane_off[q], st + SA::kBytes + (wave * LB + (q - LA)) * 1024, on);
+    // group j of the producer's step (a whole step) into the ring slot at byte offset slot_off
+    auto copy_group = [&](auto j_tag, uint32_t slot_off, int on) {
+        constexpr int j = decltype(j_tag)::value;
+        if constexpr (j < GA) {
+            constexpr int q = 4 * j, n = LA - q >= 4 ? 4 : 2;
+            const uint32_t lds = __builtin_amdgcn_readfirstlane(wave_a_lds + slot_off + q * 1024);
+            const uint64_t base = uniform64(pa_cur);
+            if constexpr (n == 4) wide_copy4<A_POLICY>(base, voff[q], voff[q + 1], voff[q + 2], voff[q + 3], lds, on);
+            else wide_copy2<A_POLICY>(base, voff[q], voff[q + 1], lds, on);
+        } else {
+            constexpr int qb = 4 * (j - GA), q = LA + qb, n = LB - qb >= 4 ? 4 : 2;
+            const uint32_t lds = __builtin_amdgcn_readfirstlane(wave_b_lds + slot_off + qb * 1024);
+            const uint64_t base = uniform64(pb_cur);
+            if constexpr (n == 4) wide_copy4<B_POLICY>(base, voff[q], voff[q + 1], voff[q + 2], voff[q + 3], lds, on);
+            else wide_copy2<B_POLICY>(base, voff[q], voff[q + 1], lds, on);
+        }
     };
     // a partial last step of DW: rows of A past the end come from a chunk of zeros, rows of B past the end
-    // re-read the last row (finite values that meet zeros)
-    auto copy_tail = [&](int slot) {
-        const uint32_t st = ring_lds + slot * STAGE_BYTES;
+    // re-read the last row (finite values that meet zeros); per-lane addresses, all copies at once
+    auto copy_tail = [&](uint32_t slot_off) {
+        const uint32_t st = ring_lds + slot_off;
         const int valid = pt.red - pk * BK;  // 1 .. BK - 1 rows
+        const unsigned char *pa = (const unsigned char *)(uintptr_t)(pa_cur + kCopyBias);
+        const unsigned char *pb = (const unsigned char *)(uintptr_t)(pb_cur + kCopyBias);
 #pragma unroll
         for (int q = 0; q < LA; ++q) {
             const int row = SA::row_of(wave * LA + q, lane);
-            const unsigned char *p = pt.pa + pk * step_a + lane_off[q];
+            const unsigned char *p = pa + lane_off[q];
             if (row >= valid) p = (const unsigned char *)&g_zero_chunk;
             wide_copy<0>(p, st + (wave * LA + q) * 1024);
         }
 #pragma unroll
         for (int q = 0; q < LB; ++q) {
             const int row = SB::row_of(wave * LB + q, lane);
-            const unsigned char *p = pt.pb + pk * step_b + lane_off[LA + q];
+            const unsigned char *p = pb + lane_off[LA + q];
             if (row >= valid) p -= (int64_t)(row - (valid - 1)) * ldb * 2;
             wide_copy<0>(p, st + SA::kBytes + (wave * LB + q) * 1024);
         }
     };
-    auto prod_is_tail = [&]() { return MODE == MODE_DW && (pk + 1) * BK > pt.red; };
-    auto prod_advance = [&]() {  // after the copies of a step
+    auto prod_advance = [&]() {  // after the last copy of a step
         issued += LPW;
         mark[pg % SR] = issued;
         ++pg;
+        pa_cur += step_a;
+        pb_cur += step_b;
         if (++pk == pt.KT) {
             pL += per_xcd;
             prod_seek();
         }
     };
     auto issue_all = [&]() {  // one whole step, back to back
-        const int slot = pg % SR;
-        if (prod_is_tail()) {
-            copy_tail(slot);
-        } else {
-            static_for<LPW>([&](auto q_tag) { copy_one(q_tag, slot); });
-        }
+        const uint32_t slot_off = (pg % SR) * STAGE_BYTES;
+        bool tail = false;
+        if constexpr (MODE == MODE_DW) tail = pk >= p_full;
+        if (tail) copy_tail(slot_off);
+        else static_for<NG>([&](auto j_tag) { copy_group(j_tag, slot_off, 1); });
         prod_advance();
     };
 
     // ---- consumer
     Tile ct;
     int cL = L_first;
-    int g = 0;  // steps multiplied so far (of the whole workgroup)
+    unsigned g = 0;  // steps multiplied so far (of the whole workgroup)
     bf16x8 fa[2][TM], fb[2][TN];  // carried from step to step, across tiles
-
-    auto stage_of = [&](int step) { return smem + (step % SR) * STAGE_BYTES; };
-    auto load_frags = [&](const unsigned char *st, int ks, int buf) {
+    // The fragment offsets carry the ring slot they read: moved on by one stage at point P.
 #pragma unroll
-        for (int bj = 0; bj < TN; ++bj) fb[buf][bj] = fo_b.load(st + SA::kBytes, bj, ks);
+    for (int i = 0; i < decltype(fo_b)::kCount; ++i) fo_b.off[i] += SA::kBytes;
+    auto frags_to_next_slot = [&]() {
+        const int delta = (g + 1) % SR == 0 ? -(SR - 1) * STAGE_BYTES : STAGE_BYTES;
 #pragma unroll
-        for (int t = 0; t < TM; ++t) fa[buf][t] = fo_a.load(st, t, ks);
+        for (int i = 0; i < decltype(fo_a)::kCount; ++i) fo_a.off[i] += delta;
+#pragma unroll
+        for (int i = 0; i < decltype(fo_b)::kCount; ++i) fo_b.off[i] += delta;
     };
+    auto load_frags = [&](int ks, int buf) {
+#pragma unroll
+        for (int bj = 0; bj < TN; ++bj) fb[buf][bj] = fo_b.load(smem, bj, ks);
+#pragma unroll
+        for (int t = 0; t < TM; ++t) fa[buf][t] = fo_a.load(smem, t, ks);
+    };
+    // second half of a step's copy groups, owed to the next sub-step 0 (SPLIT)
+    int owed = 0;
+    uint32_t owed_slot = 0;
 
     // prologue: SR steps in flight, the first one landed and its first fragments requested
 #pragma unroll 1
@@ -370,7 +457,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     if (pg > 0) {
         wait_vmcnt_upto(issued - mark[0]);
         __builtin_amdgcn_s_barrier();
-        load_frags(stage_of(0), 0, 0);
+        load_frags(0, 0);
     }
 
     const int h = lane >> 5, rl = lane & 31;
@@ -412,17 +499,17 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
         // step's barrier those of the next step's first sub-step -- and in the last sub-step also with the copies of
         // step g+SR.  A partial last step of DW multiplies all its sub-steps: rows past the end are zeros in A.
         constexpr int NM = TA * TN, NU = TM + TN;
-        auto read_unit = [&](auto u_tag, const unsigned char *rst, int rks, int buf) {
+        auto read_unit = [&](auto u_tag, int rks, int buf) {
             constexpr int U = decltype(u_tag)::value;
             if constexpr (U < TN)
-                fb[buf][U] = fo_b.load(rst + SA::kBytes, U, rks);
+                fb[buf][U] = fo_b.load(smem, U, rks);
             else
-                fa[buf][U - TN] = fo_a.load(rst, U - TN, rks);
+                fa[buf][U - TN] = fo_a.load(smem, U - TN, rks);
         };
-        // SPREAD: the copies of the producer's step between the MFMAs, issued if `on`
-        auto substep = [&](auto ks_tag, auto spread_tag, const unsigned char *rst, int rks, int slot, int on) {
-            constexpr int ks = decltype(ks_tag)::value;
-            constexpr bool SPREAD = decltype(spread_tag)::value != 0;
+        // Sub-step ks: its MFMAs, the fragment reads of sub-step rks (of this step, or after point P of the next
+        // one) and the copy groups [G0, G1) of the producer's step, issued if `on`.
+        auto substep = [&](auto ks_tag, auto g0_tag, auto g1_tag, int rks, uint32_t slot_off, int on) {
+            constexpr int ks = decltype(ks_tag)::value, G0 = decltype(g0_tag)::value, G1 = decltype(g1_tag)::value;
             static_for<NM>([&](auto i_tag) {
                 constexpr int I = decltype(i_tag)::value, t = I / TN, bj = I % TN;
                 if (!kNoMfma)
@@ -430,40 +517,64 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
                 __builtin_amdgcn_sched_barrier(0);
                 // read unit u follows MFMA u * NM / NU
                 static_for<NU>([&](auto u_tag) {
-                    if constexpr (decltype(u_tag)::value * NM / NU == I) read_unit(u_tag, rst, rks, (ks + 1) & 1);
+                    if constexpr (decltype(u_tag)::value * NM / NU == I) read_unit(u_tag, rks, (ks + 1) & 1);
                 });
                 __builtin_amdgcn_sched_barrier(0);
-                if constexpr (SPREAD) {
-                    // copy q follows MFMA q * NM / LPW
-                    static_for<LPW>([&](auto q_tag) {
-                        if constexpr (decltype(q_tag)::value * NM / LPW == I) copy_one_if(q_tag, slot, on);
+                if constexpr (G1 > G0) {
+                    // copy group j follows MFMA (j - G0) * NM / (G1 - G0)
+                    static_for<NG>([&](auto j_tag) {
+                        constexpr int J = decltype(j_tag)::value;
+                        if constexpr (J >= G0 && J < G1 && (J - G0) * NM / (G1 - G0) == I) copy_group(j_tag, slot_off, on);
                     });
                     __builtin_amdgcn_sched_barrier(0);
                 }
             });
         };
         auto step = [&]() {
-            const unsigned char *st = stage_of(g);
-            static_for<KS - 1>([&](auto ks_tag) { substep(ks_tag, IC<0>{}, st, decltype(ks_tag)::value + 1, 0, 0); });
+            // first sub-step: with it the copy groups that the previous step's point P left for later
+            if constexpr (SPLIT) {
+                substep(IC<0>{}, IC<NG1>{}, IC<NG>{}, 1, owed_slot, owed);
+                if (owed) prod_advance();
+                owed = 0;
+            } else {
+                substep(IC<0>{}, IC<0>{}, IC<0>{}, 1, 0, 0);
+            }
+            static_for<KS - 2>([&](auto k_tag) {
+                constexpr int ks = decltype(k_tag)::value + 1;
+                substep(IC<ks>{}, IC<0>{}, IC<0>{}, ks + 1, 0, 0);
+            });
             // ---- point P: my reads of this stage are done, my copies of the next step have landed
-            const bool next_exists = g + 1 < pg;
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            if (next_exists) wait_vmcnt_upto(issued - mark[(g + 1) % SR]);
+            if (g + 1 < pg) {
+                const unsigned n = issued - mark[(g + 1) % SR];
+                if (n == (SR - 2) * LPW) wait_vmcnt<(SR - 2) * LPW>();  // the steady state
+                else wait_vmcnt_upto((int)n);
+            }
             __builtin_amdgcn_s_barrier();
             // (past the workgroup's last step the reads fetch a stage nobody uses)
-            const unsigned char *nst = stage_of(g + 1);
-            bool spread = false;
-            const int slot = pg % SR;
+            frags_to_next_slot();
+            int spread = 0;
+            const uint32_t slot_off = (pg % SR) * STAGE_BYTES;
             if (p_more) {
-                if (prod_is_tail()) {
-                    copy_tail(slot);
+                bool tail = false;
+                if constexpr (MODE == MODE_DW) tail = pk >= p_full;
+                if (tail) {
+                    copy_tail(slot_off);
                     prod_advance();
                 } else {
-                    spread = true;
+                    spread = 1;
                 }
             }
-            substep(IC<KS - 1>{}, IC<1>{}, nst, 0, slot, __builtin_amdgcn_readfirstlane(spread ? 1 : 0));
-            if (spread) prod_advance();
+            spread = __builtin_amdgcn_readfirstlane(spread);
+            substep(IC<KS - 1>{}, IC<0>{}, IC<NG1>{}, 0, slot_off, spread);
+            if (spread) {
+                if constexpr (SPLIT) {
+                    owed = 1;
+                    owed_slot = slot_off;
+                } else {
+                    prod_advance();
+                }
+            }
             ++g;
         };
         {

@@ -288,7 +288,7 @@ int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const
                     const void *m_sizes, int ms_i64, void *y, int64_t R, int N, int K, int E, int out_dtype,
                     hipStream_t stream, const GemmFusion *fusion) {
     // decode-sized batches only: with more rows per expert every 32-row tile decodes the weights again
-    if (R > (int64_t)32 * E || R <= 0) return R <= 0 ? MFL_OK : MFL_ERR_UNSUPPORTED;
+    if (R > (int64_t)kNf4DecodeRowsPerExpert * E || R <= 0) return R <= 0 ? MFL_OK : MFL_ERR_UNSUPPORTED;
     int shift = 0;
     while ((1 << shift) < blocksize) ++shift;
     if (K % 64 != 0 || N % 8 != 0 || N < 8 || blocksize < 8) return MFL_ERR_UNSUPPORTED;
