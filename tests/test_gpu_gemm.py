@@ -299,3 +299,35 @@ def test_dw_four_wave_kernel_matches_oracle(N, K, sizes, ms_dtype):
     for e in (ms == 0).nonzero().flatten().tolist():
         assert torch.count_nonzero(dw[e]).item() == 0, "experts without rows must get exact zeros"
     assert torch.equal(grouped_gemm_backward_dw(xd, dyd, msd, torch.bfloat16), dw), "same bits from run to run"
+
+
+# the same kernel in the row-grouped products (forward and input gradient with N >= 2 K and 64 to 512 rows per
+# expert on average): tiles of 320 x 192, so N = 200, 520 and 2048 end in a partial column tile; experts of 0, 1,
+# 319, 320, 321 and 700 rows (no tile, one block, a full tile, a tile and one row, several tiles).
+WIDE_ROW_CASES = [
+    # N, K, m_sizes
+    (200, 64, [300, 0, 1, 319, 320, 321, 700, 95]),
+    (520, 128, [257] * 5 + [0, 64, 512]),
+    (2048, 768, [250 + 7 * (e % 5) for e in range(16)]),
+    (384, 192, [100 + e for e in range(70)]),
+]
+
+
+@pytest.mark.parametrize("N,K,sizes", WIDE_ROW_CASES)
+def test_row_grouped_products_on_the_four_wave_kernel_match_oracle(N, K, sizes):
+    ms = torch.tensor(sizes, dtype=torch.int32)
+    E, R = ms.numel(), int(ms.sum())
+    assert 64 * E <= R < 512 * E and N >= 2 * K
+    x, w, _, _, sel = _case(N + K + E, R, N, K, E, torch.bfloat16, m_sizes=ms)
+    xd, wd, msd = x.to(DEV), w.to(DEV), ms.to(DEV)
+    print(f"four-wave fwd/dX N={N} K={K} E={E} R={R}", flush=True)
+    y = grouped_gemm_forward(xd, wd, msd)
+    check_close(y, oracle.linear_fwd(to_np32(x), to_np32(w), sel), 1e-2, 1e-2, "four-wave fwd")
+    assert torch.equal(grouped_gemm_forward(xd, wd, msd), y)
+    # input gradient with the roles the kernel sees: dy (R, K) against w2 (E, K, N) -> (R, N)
+    g = gen(7 + N)
+    dy = randn((R, K), g, 1.0, torch.bfloat16)
+    w2 = randn((E, K, N), g, 0.02, torch.bfloat16)
+    dx = grouped_gemm_forward_transposed(dy.to(DEV), w2.to(DEV), msd)
+    exp = oracle.linear_bwd_input(to_np32(dy), to_np32(w2), sel)
+    check_close(dx, exp, 1e-2, 1e-2, "four-wave dX")

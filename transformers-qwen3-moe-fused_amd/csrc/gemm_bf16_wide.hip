@@ -21,7 +21,7 @@
 // has issued (copies and output stores) and, per ring slot, that number after the slot's last copy: "step g+1 has
 // landed" is a wait for at most (issued - mark) outstanding operations, whatever was issued in between.
 //
-// Shapes: bf16 in, bf16 out, no accumulation, no scaling; E <= 512; FWD/DX: N % BN == 0, K % 64 == 0; DW: N % BM == 0,
+// Shapes: bf16 in, bf16 out, no accumulation, no scaling; E <= 512; FWD/DX: N % 8 == 0, K % 64 == 0; DW: N % BM == 0,
 // K % BN == 0 (any number of rows per expert).  The caller falls back to gemm_bf16_pipe.hip otherwise.
 #include "pipe_parts.h"
 
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     // ---- per-expert prefix tables in LDS behind the ring and the staging area: rows and tiles before expert e
     int *tab_rows = (int *)(smem + RING_BYTES + NW * EP_WAVE);
     int *tab_tiles = tab_rows + (kMaxTableExperts + 1);
-    const int tiles_n = MODE == MODE_DW ? K / BN : N / BN;
+    const int tiles_n = MODE == MODE_DW ? K / BN : ceil_div(N, BN);  // row-grouped products: the last may be partial
     const int per_expert = MODE == MODE_DW ? (N / BM) * tiles_n : 0;
     {
         int row_carry = 0, tile_carry = 0;
@@ -274,7 +274,11 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
             const int rows = tile_rows_of<BM>(m_size);
             // few row tiles: those of one column slice run side by side (they share the slice of the weights);
             // many: the column slices of one row tile (they share its rows)
+#if defined(MFL_TUNING_BUILD) && defined(MFL_X_ORDER)
+            const bool n_fast = MFL_X_ORDER == 1;
+#else
             const bool n_fast = m_tiles > tiles_n;
+#endif
             const int mi = n_fast ? local / tiles_n : local % m_tiles;
             const int ni = n_fast ? local % tiles_n : local / m_tiles;
             t.i0 = m_start + mi * rows;
@@ -316,11 +320,15 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
         for (int q = 0; q < LPW; ++q)
             if (q >= q0 && q < q1) voff[q] = lane_off[q] + kCopyBias - ((q < LA ? q : q - LA) % 4) * 1024;
     };
-    auto prod_offsets = [&]() {
+    auto prod_offsets = [&]() {  // row-grouped products: rows past the tile's last and columns past N are clamped
         const int i_lim = pt.i_end - pt.i0 < BM ? pt.i_end - pt.i0 : BM;
+        const int j_lim = N - pt.j0 < BN ? N - pt.j0 : BN;
 #pragma unroll
         for (int q = 0; q < LA; ++q) lane_off[q] = (uint32_t)lane_src_offset<BM, BK, A_RC>(wave * LA + q, lane, lda, i_lim);
-        prep_voff(0, LA);
+#pragma unroll
+        for (int q = 0; q < LB; ++q)
+            lane_off[LA + q] = (uint32_t)lane_src_offset<BN, BK, B_RC>(wave * LB + q, lane, ldb, j_lim);
+        prep_voff(0, LPW);
     };
     auto prod_seek = [&]() {  // first tile from pL on that has steps
         p_more = false;
@@ -625,15 +633,16 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
                 constexpr int CPR = EPC / 8;
 #pragma unroll
                 for (int q0 = 0; q0 < 32 * CPR; q0 += 64) {
-                    // a store whose rows all lie past the tile's last one is left out, and not counted
-                    if (MODE != MODE_DW && row_base + q0 / CPR >= ct.i_end) continue;
+                    // a store whose rows all lie past the tile's last one, or whose columns all lie past N, is left
+                    // out, and not counted
+                    if (MODE != MODE_DW && (row_base + q0 / CPR >= ct.i_end || ct.j0 + wn * WTN + part * EPC >= N)) continue;
                     if (!kNoStore) ++issued;
                     const int q = q0 + lane;
                     const int row_l = q / CPR, lcol = (q % CPR) * 8;
                     const int row = row_base + row_l;
                     const int col = ct.j0 + wn * WTN + part * EPC + lcol;
                     const uint4_t v = *(const uint4_t *)(ep + row_l * EP_ROWB + lcol * 2);
-                    if (!kNoStore && (MODE == MODE_DW || row < ct.i_end))
+                    if (!kNoStore && (MODE == MODE_DW || (row < ct.i_end && col < N)))
                         __builtin_nontemporal_store(v, (uint4_t *)((bf16_t *)ct.pc + (int64_t)row * ldc + col));
                 }
             }
@@ -693,11 +702,11 @@ int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, 
 #else
     const int v = 0;
 #endif
-    if (v == 0 && N % 192 == 0) {
+    if (N % 8 != 0 || N < 8) return MFL_ERR_UNSUPPORTED;
+    if (v == 0) {
         if (mode == MODE_FWD) return launch_wide<MODE_FWD, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
         return launch_wide<MODE_DX, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
     }
-    if (N % 256 != 0) return MFL_ERR_UNSUPPORTED;
     if (mode == MODE_FWD) return launch_wide<MODE_FWD, 8, 8, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
     return launch_wide<MODE_DX, 8, 8, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
 }
