@@ -311,6 +311,11 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     constexpr int NG1 = SPLIT ? (NG + 1) / 2 : NG;  // groups in the sub-step after point P
     Tile pt;
     int pL = L_first, pk = 0, p_full = 0;  // p_full: steps of the producer's tile that are whole
+    // Row-grouped products: copy groups of A whose stage rows all lie past the tile's last row are left out (nothing
+    // that is stored reads them): bit j of p_amask says that this wave issues group j, p_copies how many copies
+    // a step of the producer's tile comes to for this wave.
+    unsigned p_amask = ~0u;
+    int p_copies = LPW;
     bool p_more = false;
     uint64_t pa_cur = 0, pb_cur = 0;  // operand addresses of the producer's step, minus kCopyBias
     uint32_t lane_off[LPW];           // per-lane source offsets of the wave's copies (tile origin, step 0)
@@ -329,6 +334,15 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
         for (int q = 0; q < LB; ++q)
             lane_off[LA + q] = (uint32_t)lane_src_offset<BN, BK, B_RC>(wave * LB + q, lane, ldb, j_lim);
         prep_voff(0, LPW);
+        p_amask = 0, p_copies = LB;
+#pragma unroll
+        for (int j = 0; j < GA; ++j) {
+            const int first_row = SA::row_of(wave * LA + 4 * j, 0);
+            if (first_row < i_lim) {
+                p_amask |= 1u << j;
+                p_copies += LA - 4 * j >= 4 ? 4 : 2;
+            }
+        }
     };
     auto prod_seek = [&]() {  // first tile from pL on that has steps
         p_more = false;
@@ -381,6 +395,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
             constexpr int q = 4 * j, n = LA - q >= 4 ? 4 : 2;
             const uint32_t lds = __builtin_amdgcn_readfirstlane(wave_a_lds + slot_off + q * 1024);
             const uint64_t base = uniform64(pa_cur);
+            if constexpr (A_RC) on = on & (int)((p_amask >> j) & 1u);
             if constexpr (n == 4) wide_copy4<A_POLICY>(base, voff[q], voff[q + 1], voff[q + 2], voff[q + 3], lds, on);
             else wide_copy2<A_POLICY>(base, voff[q], voff[q + 1], lds, on);
         } else {
@@ -414,7 +429,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
         }
     };
     auto prod_advance = [&]() {  // after the last copy of a step
-        issued += LPW;
+        issued += p_copies;
         mark[pg % SR] = issued;
         ++pg;
         pa_cur += step_a;
