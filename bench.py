@@ -177,6 +177,7 @@ def _kernel_tour(n, dev):
         ("gemm_fwd gate_proj 4096 tokens", gemm_b, gemm_f, lambda i: grouped_gemm_forward(x, w_gate, m_sizes)),
         ("gemm_dx down_proj 4096 tokens", gemm_b, gemm_f, lambda i: grouped_gemm_forward_transposed(dy, w_down, m_sizes)),
         ("gemm_dw down_proj 4096 tokens", gemm_b, gemm_f, lambda i: grouped_gemm_backward_dw(h, dy, m_sizes, bf)),
+        ("gemm_fwd down_proj 4096 tokens", gemm_b, gemm_f, lambda i: grouped_gemm_forward(h, w_down, m_sizes)),
         ("glu_fwd (gather + gate + up + SiLU-mul) 4096 tokens",
          2.0 * (TOKENS * HIDDEN + 2 * E * INTER * HIDDEN + ROWS * INTER), 2 * gemm_f,
          lambda i: grouped_glu_forward(hidden, w_gate, w_up, m_sizes, sort_idx, TOPK)),

@@ -45,6 +45,23 @@ constexpr bool kNoStore = MFL_X_NO_STORE, kNoCopy = MFL_X_NO_COPY, kNoMfma = MFL
 constexpr bool kNoStore = false, kNoCopy = false, kNoMfma = false;
 #endif
 
+#if defined(MFL_TUNING_BUILD) && defined(MFL_X_TRACE)
+// time stamps of one workgroup's first wave, kept in LDS (behind everything else) and copied out at the end
+__device__ unsigned int g_wide_trace[4096];
+__device__ int g_wide_trace_n;
+#define MFL_TR_LDS 155648
+#define MFL_TR(tag)                                                                                          \
+    if (blockIdx.x == MFL_X_TRACE && wave == 0 && tr_n < 1000) {                                               \
+        if (lane == 0) {                                                                                     \
+            ((unsigned int *)(smem + MFL_TR_LDS))[2 * tr_n] = (tag);                                          \
+            ((unsigned int *)(smem + MFL_TR_LDS))[2 * tr_n + 1] = (unsigned int)__builtin_readcyclecounter(); \
+        }                                                                                                    \
+        ++tr_n;                                                                                              \
+    }
+#else
+#define MFL_TR(tag)
+#endif
+
 // s_waitcnt vmcnt(n rounded down to a multiple of 8), n wave-uniform
 __device__ __forceinline__ void wait_vmcnt_upto(int n) {
     switch (n >> 3) {
@@ -192,6 +209,9 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
+#if defined(MFL_TUNING_BUILD) && defined(MFL_X_TRACE)
+    int tr_n = 0;
+#endif
 
     FragOffsets<BM, BK, A_RC, TM> fo_a;
     FragOffsets<BN, BK, B_RC, TN> fo_b;
@@ -554,6 +574,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
             });
         };
         auto step = [&]() {
+            MFL_TR(1)
             // first sub-step: with it the copy groups that the previous step's point P left for later
             if constexpr (SPLIT) {
                 substep(IC<0>{}, IC<NG1>{}, IC<NG>{}, 1, owed_slot, owed);
@@ -567,13 +588,16 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
                 substep(IC<ks>{}, IC<0>{}, IC<0>{}, ks + 1, 0, 0);
             });
             // ---- point P: my reads of this stage are done, my copies of the next step have landed
+            MFL_TR(2)
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             if (g + 1 < pg) {
                 const unsigned n = issued - mark[(g + 1) % SR];
                 if (n == (SR - 2) * LPW) wait_vmcnt<(SR - 2) * LPW>();  // the steady state
                 else wait_vmcnt_upto((int)n);
             }
+            MFL_TR(3)
             __builtin_amdgcn_s_barrier();
+            MFL_TR(4)
             // (past the workgroup's last step the reads fetch a stage nobody uses)
             frags_to_next_slot();
             int spread = 0;
@@ -620,6 +644,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
             do step();
             while (++kc < ct.KT);
         }
+        MFL_TR(5)
 
         // ---- epilogue: a 32-row block of EPC columns at a time through the wave's own staging area (8 bytes per
         // lane and write), then whole 16-byte pieces of rows, streaming stores
@@ -662,6 +687,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
                 }
             }
         }
+        MFL_TR(6)
         };  // tile_body
         if (MODE == MODE_DW)
             tile_body(IC<TM>{});
@@ -676,6 +702,13 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
         else
             tile_body(IC<TM>{});
     }
+#if defined(MFL_TUNING_BUILD) && defined(MFL_X_TRACE)
+    if (blockIdx.x == MFL_X_TRACE && wave == 0) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        for (int i = lane; i < 2 * tr_n; i += 64) g_wide_trace[i] = ((unsigned int *)(smem + MFL_TR_LDS))[i];
+        if (lane == 0) g_wide_trace_n = tr_n;
+    }
+#endif
 }
 
 template <int MODE, int MB, int NB, int BK, int SR>
@@ -685,7 +718,11 @@ int launch_wide(const void *a, const void *b, const void *m_sizes, int ms_i64, v
     constexpr int WTN = NB / 2 * 32;
     constexpr int EPC = WTN % 64 == 0 ? 64 : WTN;
     constexpr int EP_ROWB = EPC * 2 + (EPC == 64 ? 16 : 8);
+#if defined(MFL_TUNING_BUILD) && defined(MFL_X_TRACE)
+    constexpr int LDS_BYTES = 160 * 1024;
+#else
     constexpr int LDS_BYTES = SR * STAGE_BYTES + 4 * 32 * EP_ROWB + 2 * (kMaxTableExperts + 1) * 4;
+#endif
     static_assert(LDS_BYTES <= 160 * 1024, "LDS capacity of a CDNA4 compute unit");
     auto kern = gemm_wide_kernel<MODE, MB, NB, BK, SR, bf16_t>;
     static PerDeviceOnce attr;
