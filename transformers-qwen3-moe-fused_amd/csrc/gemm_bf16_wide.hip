@@ -506,6 +506,23 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     const int h = lane >> 5, rl = lane & 31;
     unsigned char *const ep = smem + RING_BYTES + wave * EP_WAVE;
 
+    // Store u of a part covers pieces 64 u .. 64 u + 63 of its 32 x CPR pieces (row-major); the lanes' places
+    // repeat every NPER stores, RPP rows further down.
+    constexpr int CPR = EPC / 8, NST = 32 * CPR / 64;
+    constexpr int NPER = CPR % 8 == 0 ? 1 : CPR % 4 == 0 ? CPR / 4 : CPR % 2 == 0 ? CPR / 2 : CPR;
+    constexpr int RPP = 64 * NPER / CPR;
+    static_assert(NST % NPER == 0 && (64 * NPER) % CPR == 0, "whole periods");
+    uint32_t st_voff[NPER], st_lds[NPER], st_rc[NPER];  // global offset, LDS address, row | column << 8
+#pragma unroll
+    for (int e = 0; e < NPER; ++e) {
+        const int q = e * 64 + lane, row = q / CPR, col = (q % CPR) * 8;
+        st_voff[e] = (uint32_t)((row * (int)ldc + col) * 2);
+        st_lds[e] = (uint32_t)(uintptr_t)(lds_void_ptr)(ep + row * EP_ROWB + col * 2);
+        st_rc[e] = (uint32_t)(row | col << 8);
+    }
+
+    constexpr int PPT = WTN / EPC;  // parts (32 rows x EPC columns) per row block
+
 #pragma unroll 1
     for (; cL < L_end; cL += per_xcd) {
         tile_at(cL, ct);
@@ -647,45 +664,78 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
         MFL_TR(5)
 
         // ---- epilogue: a 32-row block of EPC columns at a time through the wave's own staging area (8 bytes per
-        // lane and write), then whole 16-byte pieces of rows, streaming stores
+        // lane and write), then whole 16-byte pieces of rows, streaming stores from a scalar base plus a per-lane
+        // offset that is the same for every tile.  Accumulators are fetched sixteen at a time into registers of their
+        // own, so that converting and writing one group does not wait for the fetch of the next.
+        const uint64_t c_tile = uniform64((uint64_t)(uintptr_t)ct.pc +
+                                          (((int64_t)(ct.i0 + wm * 32)) * ldc + ct.j0 + wn * WTN) * 2);
+        // Part p (a 32-row block of one row block t, EPC columns) is fetched while the staged pieces of part p - 1
+        // are on their way back from LDS, and converted and staged after the stores of part p - 1 have gone out.
+        constexpr int NP = TA * PPT, BPP = EPC / 32;  // parts, 32-column blocks per part
+        float v[BPP][16];
+        uint4_t piece[NST];
+        auto fetch = [&](auto p_tag) {
+            constexpr int p = decltype(p_tag)::value, t = p / PPT, part = p % PPT;
 #pragma unroll
-        for (int t = 0; t < TA; ++t) {
-            if (t >= active) continue;
+            for (int bq = 0; bq < BPP; ++bq)
+#pragma unroll
+                for (int u = 0; u < 16; ++u) v[bq][u] = acc_read(acc[t][part * BPP + bq][u]);
+        };
+        auto stage = [&]() {
+#pragma unroll
+            for (int bq = 0; bq < BPP; ++bq)
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) {
+                    union {
+                        bf16_t e[4];
+                        uint2_t v;
+                    } pk4;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) pk4.e[u] = (bf16_t)v[bq][4 * gq + u];
+                    *(uint2_t *)(ep + rl * EP_ROWB + (bq * 32 + 8 * gq + 4 * h) * 2) = pk4.v;
+                }
+        };
+        auto store = [&](auto p_tag) {
+            constexpr int p = decltype(p_tag)::value, t = p / PPT, part = p % PPT;
             const int row_base = ct.i0 + (wm + WGM * t) * 32;
+            const int col0 = ct.j0 + wn * WTN + part * EPC;
+            const uint64_t c_part = c_tile + ((int64_t)t * (WGM * 32) * ldc + part * EPC) * 2;
 #pragma unroll
-            for (int part = 0; part < WTN / EPC; ++part) {
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int bq = 0; bq < EPC / 32; ++bq) {
-                    const int bj = part * (EPC / 32) + bq;
-#pragma unroll
-                    for (int gq = 0; gq < 4; ++gq) {
-                        union {
-                            bf16_t e[4];
-                            uint2_t v;
-                        } pk4;
-#pragma unroll
-                        for (int u = 0; u < 4; ++u) pk4.e[u] = (bf16_t)acc_read(acc[t][bj][4 * gq + u]);
-                        *(uint2_t *)(ep + rl * EP_ROWB + (bq * 32 + 8 * gq + 4 * h) * 2) = pk4.v;
-                    }
-                }
-                // the same wave reads back what it wrote: LDS operations of one wave complete in order
-                constexpr int CPR = EPC / 8;
-#pragma unroll
-                for (int q0 = 0; q0 < 32 * CPR; q0 += 64) {
-                    // a store whose rows all lie past the tile's last one, or whose columns all lie past N, is left
-                    // out, and not counted
-                    if (MODE != MODE_DW && (row_base + q0 / CPR >= ct.i_end || ct.j0 + wn * WTN + part * EPC >= N)) continue;
-                    if (!kNoStore) ++issued;
-                    const int q = q0 + lane;
-                    const int row_l = q / CPR, lcol = (q % CPR) * 8;
-                    const int row = row_base + row_l;
-                    const int col = ct.j0 + wn * WTN + part * EPC + lcol;
-                    const uint4_t v = *(const uint4_t *)(ep + row_l * EP_ROWB + lcol * 2);
-                    if (!kNoStore && (MODE == MODE_DW || (row < ct.i_end && col < N)))
-                        __builtin_nontemporal_store(v, (uint4_t *)((bf16_t *)ct.pc + (int64_t)row * ldc + col));
-                }
+            for (int u = 0; u < NST; ++u) {
+                // a store whose rows all lie past the tile's last one, or whose columns all lie past N, is left
+                // out, and not counted
+                if (MODE != MODE_DW && (row_base + u * 64 / CPR >= ct.i_end || col0 >= N)) continue;
+                if (kNoStore) continue;
+#if defined(MFL_TUNING_BUILD) && defined(MFL_X_HALF_STORE)
+                if (p >= NP / 2) continue;
+#endif
+                ++issued;
+                const int down = (u / NPER) * RPP;
+                const uint64_t c_rows = c_part + (int64_t)down * ldc * 2;
+                const uint32_t off = st_voff[u % NPER];  // (operands of a statement in a nested lambda: its own locals)
+                const uint4_t data = piece[u];
+                const int st_row = (int)(st_rc[u % NPER] & 255u), st_col = (int)(st_rc[u % NPER] >> 8);
+                if (MODE == MODE_DW || (row_base + down + st_row < ct.i_end && col0 + st_col < N))
+                    asm volatile("global_store_dwordx4 %0, %1, %2 nt" : : "v"(off), "v"(data), "s"(c_rows) : "memory");
             }
+        };
+        if (active > 0) {
+            fetch(IC<0>{});
+            stage();
+            static_for<NP>([&](auto p_tag) {
+                constexpr int p = decltype(p_tag)::value;
+                __builtin_amdgcn_sched_barrier(0);
+                // the same wave reads back what it wrote: LDS operations of one wave complete in order
+#pragma unroll
+                for (int u = 0; u < NST; ++u)
+                    piece[u] = *(const __attribute__((address_space(3))) uint4_t *)(st_lds[u % NPER] + (u / NPER) * RPP * EP_ROWB);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (p + 1 < NP) fetch(IC<p + 1>{});
+                __builtin_amdgcn_sched_barrier(0);
+                store(p_tag);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (p + 1 < NP) stage();
+            });
         }
         MFL_TR(6)
         };  // tile_body
