@@ -215,6 +215,33 @@ MFL_API int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_
                     int m_sizes_dtype, void *h, void *e_out, void *g_out, int64_t R, int N, int K,
                     int E, int dtype, void *stream);
 
+/* Tile-ordered scales for decode-sized batches.  At a few rows per expert the NF4 kernels are bound by the
+ * number of memory requests, and the 64 scales that a wave needs per 128-wide reduction stage lie in 32
+ * different lines of absmax.  mfl_nf4_tile_absmax writes them once more, in the order of consumption:
+ * out[((e * ceil(N/32) + t) * (K/128) + s) * 64 + l] = the scale of weight (e, min(32 t + l/2, N-1),
+ * 128 s + 64 (l % 2)), mfl_nf4_tiled_absmax_floats floats in all (0: the shape has no such copy -- K not a
+ * multiple of 128, or blocks of fewer than 64 weights; mfl_nf4_tile_absmax then returns MFL_ERR_UNSUPPORTED).
+ * A caller builds the copy once per quantisation state and hands it to the two entry points below, which
+ * are mfl_gemm_fwd_nf4 / mfl_gemm_fwd_nf4_gather (row_idx NULL: x_src is x, src_rows and idx_div ignored)
+ * and mfl_glu_fwd_nf4 with one more argument per matrix; absmax_tiled may be NULL (then they are those
+ * entry points), and results are bit-identical with and without it.  No counterpart in the reference, whose
+ * 4-bit product (qwen3_moe_fused/grouped_gemm/forward_4bit.py:99-106) reads absmax in place. */
+MFL_API int64_t mfl_nf4_tiled_absmax_floats(int blocksize, int N, int K, int E);
+MFL_API int mfl_nf4_tile_absmax(const float *absmax, int blocksize, int N, int K, int E, float *out,
+                        void *stream);
+MFL_API int mfl_gemm_fwd_nf4_tiled(const void *x_src, int64_t src_rows, const int32_t *row_idx, int idx_div,
+                           const uint8_t *wq, const float *code16, const float *absmax,
+                           const float *absmax_tiled, int blocksize, const void *m_sizes,
+                           int m_sizes_dtype, void *y, int64_t R, int N, int K, int E, int in_dtype,
+                           int out_dtype, void *stream);
+MFL_API int mfl_glu_fwd_nf4_tiled(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div,
+                          const uint8_t *wq_gate, const float *code16_gate, const float *absmax_gate,
+                          const float *absmax_tiled_gate, int blocksize_gate, const uint8_t *wq_up,
+                          const float *code16_up, const float *absmax_up,
+                          const float *absmax_tiled_up, int blocksize_up, const void *m_sizes,
+                          int m_sizes_dtype, void *h, void *e_out, void *g_out, int64_t R, int N, int K,
+                          int E, int dtype, void *stream);
+
 /* ---- NF4 / blockwise dequantisation ----------------------------------------------- */
 
 /* out[i] = code16[nibble(i)] * absmax[i / blocksize], i < n (n even).  Stands in for the

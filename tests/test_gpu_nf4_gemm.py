@@ -119,6 +119,100 @@ def test_streaming_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, out_d
     assert torch.equal(y2[:R - 3], y[:R - 3])
 
 
+def _tile_ordered(absmax, E, N, K, blocksize):
+    """The scales in the order the streaming kernel's waves consume them: [expert][32-column tile][128-wide
+    stage][column of the tile][half of the stage], columns past N repeating the last one."""
+    a = np.asarray(absmax, dtype=np.float32).reshape(-1)
+    tiles, stages = -(-N // 32), K // 128
+    e, t, s, l = np.meshgrid(np.arange(E), np.arange(tiles), np.arange(stages), np.arange(64), indexing="ij")
+    col = np.minimum(32 * t + l // 2, N - 1)
+    first_weight = (e.astype(np.int64) * N + col) * K + 128 * s + 64 * (l % 2)
+    return a[first_weight // blocksize].reshape(-1)
+
+
+# Scales handed over in the order of consumption: the copy is the permutation it is documented to be, and the plain,
+# the gathered and the gated product return the same bits with it as without (column counts that are and are not
+# multiples of 32 and 128, blocks of 64 to 512 weights, several row tiles per expert, empty experts).
+@pytest.mark.parametrize("m_sizes,N,K,blocksize", [([3, 0, 1, 7], 8, 128, 64), ([33, 0, 70, 1, 0, 12], 200, 256, 128),
+                                                   ([9, 31, 32, 2], 264, 640, 512), ([5, 17, 0, 2], 768, 2048, 64)])
+def test_tile_ordered_scales(m_sizes, N, K, blocksize):
+    from qwen3_moe_fused import _lib
+    from qwen3_moe_fused.grouped_gemm.fused import grouped_glu_forward_4bit
+    E, k_sel = len(m_sizes), 2
+    ms = torch.tensor(m_sizes, dtype=torch.int32).to(DEV)
+    R = int(sum(m_sizes))
+    packed, state, _ = _quantised(E, N, K, blocksize, N + K + 1)
+    packed_u, state_u, _ = _quantised(E, N, K, blocksize, N + K + 2)
+    count = int(_lib.lib().mfl_nf4_tiled_absmax_floats(blocksize, N, K, E))
+    assert count == E * -(-N // 32) * (K // 128) * 64
+    tiled = torch.full((count,), -1.0, device=DEV)
+    _lib.check(_lib.lib().mfl_nf4_tile_absmax(_lib.ptr(state.absmax), blocksize, N, K, E, _lib.ptr(tiled),
+                                              _lib.stream()), "mfl_nf4_tile_absmax")
+    assert np.array_equal(tiled.cpu().numpy(), _tile_ordered(state.absmax.cpu().numpy(), E, N, K, blocksize))
+    tiled_u = torch.empty_like(tiled)
+    _lib.check(_lib.lib().mfl_nf4_tile_absmax(_lib.ptr(state_u.absmax), blocksize, N, K, E, _lib.ptr(tiled_u),
+                                              _lib.stream()), "mfl_nf4_tile_absmax")
+    g = gen(N)
+    src = randn((-(-R // k_sel), K), g, 1.0, torch.bfloat16).to(DEV)
+    row_idx = torch.randperm(src.shape[0] * k_sel, generator=g)[:R].to(torch.int32).to(DEV)
+    x = src[(row_idx // k_sel).long()].contiguous()
+    bf, i32 = _lib.dtype_code(torch.bfloat16), _lib.itype_code(torch.int32)
+
+    def fwd(rows, idx, t):
+        y = torch.zeros((R, N), device=DEV, dtype=torch.bfloat16)
+        rc = _lib.lib().mfl_gemm_fwd_nf4_tiled(_lib.ptr(rows), rows.shape[0], _lib.ptr(idx), k_sel, _lib.ptr(packed),
+                                               _lib.ptr(state.code), _lib.ptr(state.absmax), _lib.ptr(t), blocksize,
+                                               _lib.ptr(ms), i32, _lib.ptr(y), R, N, K, E, bf, bf, _lib.stream())
+        _lib.check(rc, "mfl_gemm_fwd_nf4_tiled")
+        return y
+
+    def glu(tg, tu):
+        out = [torch.zeros((R, N), device=DEV, dtype=torch.bfloat16) for _ in range(3)]
+        rc = _lib.lib().mfl_glu_fwd_nf4_tiled(_lib.ptr(src), src.shape[0], _lib.ptr(row_idx), k_sel, _lib.ptr(packed),
+                                              _lib.ptr(state.code), _lib.ptr(state.absmax), _lib.ptr(tg), blocksize,
+                                              _lib.ptr(packed_u), _lib.ptr(state_u.code), _lib.ptr(state_u.absmax),
+                                              _lib.ptr(tu), blocksize, _lib.ptr(ms), i32, _lib.ptr(out[0]),
+                                              _lib.ptr(out[1]), _lib.ptr(out[2]), R, N, K, E, bf, _lib.stream())
+        _lib.check(rc, "mfl_glu_fwd_nf4_tiled")
+        return out
+
+    plain = fwd(x, None, None)
+    assert torch.equal(fwd(x, None, tiled), plain), "plain product"
+    assert torch.equal(fwd(src, row_idx, None), plain) and torch.equal(fwd(src, row_idx, tiled), plain), "gathered rows"
+    for a, b in zip(glu(tiled, tiled_u), glu(None, None)):
+        assert torch.equal(a, b), "gated product"
+    for a, b in zip(glu(tiled, None), glu(None, None)):  # one copy alone is not used
+        assert torch.equal(a, b)
+    # the wrappers build the copy once per state and take the same route
+    assert torch.equal(grouped_gemm_forward_4bit(x, packed, state, ms), plain)
+    first = state._mfl_absmax_tiled[3]
+    grouped_gemm_forward_4bit(x, packed, state, ms)
+    assert state._mfl_absmax_tiled[3] is first and torch.equal(first, tiled)
+    h = grouped_glu_forward_4bit(src, packed, state, packed_u, state_u, ms, row_idx, k_sel)
+    assert torch.equal(h, glu(None, None)[0])
+
+
+def test_tile_ordered_scales_shapes_without_a_copy():
+    from qwen3_moe_fused import _lib
+    assert _lib.lib().mfl_nf4_tiled_absmax_floats(32, 64, 128, 2) == 0    # blocks under 64 weights
+    assert _lib.lib().mfl_nf4_tiled_absmax_floats(64, 64, 192, 2) == 0    # K not a multiple of 128
+    a = torch.ones(2 * 64 * 192 // 64, device=DEV)
+    out = torch.zeros(16, device=DEV)
+    assert _lib.lib().mfl_nf4_tile_absmax(_lib.ptr(a), 64, 64, 192, 2, _lib.ptr(out), _lib.stream()) == -6
+    # a product over such a shape takes the pointer and ignores it
+    packed, state, w_deq = _quantised(2, 64, 192, 64, 5)
+    x = randn((6, 192), gen(3), 1.0, torch.bfloat16)
+    ms = torch.tensor([4, 2], dtype=torch.int32)
+    y = torch.zeros((6, 64), device=DEV, dtype=torch.bfloat16)
+    xd, msd = x.to(DEV), ms.to(DEV)
+    bf = _lib.dtype_code(torch.bfloat16)
+    rc = _lib.lib().mfl_gemm_fwd_nf4_tiled(_lib.ptr(xd), 6, None, 1, _lib.ptr(packed), _lib.ptr(state.code),
+                                           _lib.ptr(state.absmax), _lib.ptr(out), 64, _lib.ptr(msd),
+                                           _lib.itype_code(torch.int32), _lib.ptr(y), 6, 64, 192, 2, bf, bf, _lib.stream())
+    _lib.check(rc, "mfl_gemm_fwd_nf4_tiled")
+    check_close(y, oracle.linear_fwd(to_np32(x), w_deq, oracle.sel_from_m_sizes(ms.numpy())), what="ignored copy")
+
+
 # The matrix-vector kernel (at most two rows per expert on average, 256 < K <= 2048, K a multiple of the block
 # size, N a multiple of 32; up to K = 1024 with 32 lanes to a column): lanes past the end of a row (K not a multiple of 512), experts of one to five rows
 # (up to three row groups), empty experts, more than 64 experts, more units than workgroups and fewer, one

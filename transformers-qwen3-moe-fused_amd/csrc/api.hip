@@ -127,9 +127,12 @@ int mfl_gemm_dw_split(const void *x, const void *dy, const void *m_sizes, int m_
                          (hipStream_t)stream);
 }
 
-int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
-                     const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K, int E, int in_dtype,
-                     int out_dtype, void *stream) {
+// The NF4 forward product, with or without gathered rows (row_idx null: x is (R, K)) and with or without the
+// tile-ordered copy of the scales.
+static int fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div, const uint8_t *wq,
+                   const float *code16, const float *absmax, const float *absmax_tiled, int blocksize,
+                   const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K, int E, int in_dtype,
+                   int out_dtype, void *stream) {
     if (R < 0 || N <= 0 || K <= 0 || E <= 0 || R > 0x7fffffff) return MFL_ERR_SHAPE;
     if (blocksize < 2 || (blocksize & (blocksize - 1)) != 0) return MFL_ERR_SHAPE;
     if (K % 2 != 0 || ((int64_t)E * N * K) % blocksize != 0) return MFL_ERR_SHAPE;
@@ -137,14 +140,56 @@ int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, cons
     if (!wq || !code16 || !absmax || !m_sizes || (R > 0 && (!x || !y))) return MFL_ERR_NULL;
     if (R == 0) return MFL_OK;
     if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
-    int rc = gemm_nf4_decode(x, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E,
-                             out_dtype, (hipStream_t)stream);
+    if (absmax_tiled != nullptr && nf4_tiled_absmax_floats(blocksize, N, K, E) == 0) absmax_tiled = nullptr;
+    const int ms_i64 = m_sizes_dtype == MFL_I64;
+    GemmFusion fu = {row_idx, idx_div, src_rows, nullptr, nullptr, nullptr, 0, nullptr, nullptr};
+    fu.absmax_tiled = absmax_tiled;
+    const GemmFusion *pf = (row_idx != nullptr || absmax_tiled != nullptr) ? &fu : nullptr;
+    int rc = gemm_nf4_decode(x, wq, code16, absmax, blocksize, m_sizes, ms_i64, y, R, N, K, E, out_dtype,
+                             (hipStream_t)stream, pf);
     if (rc != MFL_ERR_UNSUPPORTED) return rc;
-    rc = gemm_nf4_pipe(x, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E,
-                           out_dtype, (hipStream_t)stream);
-    if (rc != MFL_ERR_UNSUPPORTED) return rc;
-    return gemm_nf4_mfma(x, wq, code16, absmax, blocksize, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E, out_dtype,
+    pf = row_idx != nullptr ? &fu : nullptr;
+    rc = gemm_nf4_pipe(x, wq, code16, absmax, blocksize, m_sizes, ms_i64, y, R, N, K, E, out_dtype,
+                       (hipStream_t)stream, pf);
+    if (rc != MFL_ERR_UNSUPPORTED || row_idx != nullptr) return rc;
+    return gemm_nf4_mfma(x, wq, code16, absmax, blocksize, m_sizes, ms_i64, y, R, N, K, E, out_dtype,
                          (hipStream_t)stream);
+}
+
+int mfl_gemm_fwd_nf4(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
+                     const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K, int E, int in_dtype,
+                     int out_dtype, void *stream) {
+    return fwd_nf4(x, 0, nullptr, 1, wq, code16, absmax, nullptr, blocksize, m_sizes, m_sizes_dtype, y, R, N, K, E,
+                   in_dtype, out_dtype, stream);
+}
+
+int64_t mfl_nf4_tiled_absmax_floats(int blocksize, int N, int K, int E) {
+    return nf4_tiled_absmax_floats(blocksize, N, K, E);
+}
+
+int mfl_nf4_tile_absmax(const float *absmax, int blocksize, int N, int K, int E, float *out, void *stream) {
+    if (N <= 0 || K <= 0 || E <= 0 || blocksize < 2 || (blocksize & (blocksize - 1)) != 0) return MFL_ERR_SHAPE;
+    if (((int64_t)E * N * K) % blocksize != 0) return MFL_ERR_SHAPE;
+    if (!absmax || !out) return MFL_ERR_NULL;
+    if (!aligned(absmax, 4) || !aligned(out, 4)) return MFL_ERR_ALIGN;
+    return nf4_tile_absmax(absmax, blocksize, N, K, E, out, (hipStream_t)stream);
+}
+
+namespace {
+int check_fused(int64_t src_rows, const int32_t *row_idx, int idx_div, const void *m_sizes, int ms_dtype, int64_t R,
+                int N, int K, int E, int in_dtype, int out_dtype);
+}
+
+int mfl_gemm_fwd_nf4_tiled(const void *x_src, int64_t src_rows, const int32_t *row_idx, int idx_div, const uint8_t *wq,
+                           const float *code16, const float *absmax, const float *absmax_tiled, int blocksize,
+                           const void *m_sizes, int m_sizes_dtype, void *y, int64_t R, int N, int K, int E,
+                           int in_dtype, int out_dtype, void *stream) {
+    if (row_idx != nullptr) {
+        const int rc = check_fused(src_rows, row_idx, idx_div, m_sizes, m_sizes_dtype, R, N, K, E, in_dtype, out_dtype);
+        if (rc) return rc;
+    }
+    return fwd_nf4(x_src, src_rows, row_idx, idx_div, wq, code16, absmax, absmax_tiled, blocksize, m_sizes,
+                   m_sizes_dtype, y, R, N, K, E, in_dtype, out_dtype, stream);
 }
 
 int mfl_gemm_dx_nf4(const void *dy, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
@@ -324,11 +369,11 @@ int mfl_glu_fwd_lora(const void *x, const void *w_gate, const void *w_up, const 
                           (hipStream_t)stream, &fu);
 }
 
-int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div, const uint8_t *wq_gate,
-                    const float *code16_gate, const float *absmax_gate, int blocksize_gate, const uint8_t *wq_up,
-                    const float *code16_up, const float *absmax_up, int blocksize_up, const void *m_sizes,
-                    int m_sizes_dtype, void *h, void *e_out, void *g_out, int64_t R, int N, int K, int E, int dtype,
-                    void *stream) {
+int mfl_glu_fwd_nf4_tiled(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div, const uint8_t *wq_gate,
+                          const float *code16_gate, const float *absmax_gate, const float *absmax_tiled_gate,
+                          int blocksize_gate, const uint8_t *wq_up, const float *code16_up, const float *absmax_up,
+                          const float *absmax_tiled_up, int blocksize_up, const void *m_sizes, int m_sizes_dtype,
+                          void *h, void *e_out, void *g_out, int64_t R, int N, int K, int E, int dtype, void *stream) {
     int rc = check_fused(src_rows, row_idx, idx_div, m_sizes, m_sizes_dtype, R, N, K, E, dtype, dtype);
     if (rc) return rc;
     for (int bs : {blocksize_gate, blocksize_up}) {
@@ -339,13 +384,29 @@ int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int
         return MFL_ERR_NULL;
     if (R == 0) return MFL_OK;
     if (dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
-    const GemmFusion fu = {row_idx, idx_div, src_rows, wq_up, code16_up, absmax_up, blocksize_up, e_out, g_out};
+    GemmFusion fu = {row_idx, idx_div, src_rows, wq_up, code16_up, absmax_up, blocksize_up, e_out, g_out};
+    // the tile-ordered scales serve where both matrices have them
+    if (absmax_tiled_gate != nullptr && absmax_tiled_up != nullptr &&
+        nf4_tiled_absmax_floats(blocksize_gate, N, K, E) != 0 && nf4_tiled_absmax_floats(blocksize_up, N, K, E) != 0) {
+        fu.absmax_tiled = absmax_tiled_gate;
+        fu.absmax_tiled_2 = absmax_tiled_up;
+    }
     const int ms_i64 = m_sizes_dtype == MFL_I64;
     rc = gemm_nf4_decode(x, wq_gate, code16_gate, absmax_gate, blocksize_gate, m_sizes, ms_i64, h, R, N, K, E, MFL_BF16,
                          (hipStream_t)stream, &fu);
     if (rc != MFL_ERR_UNSUPPORTED) return rc;
     return gemm_nf4_pipe(x, wq_gate, code16_gate, absmax_gate, blocksize_gate, m_sizes, ms_i64, h, R, N, K, E, MFL_BF16,
                          (hipStream_t)stream, &fu);
+}
+
+int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_idx, int idx_div, const uint8_t *wq_gate,
+                    const float *code16_gate, const float *absmax_gate, int blocksize_gate, const uint8_t *wq_up,
+                    const float *code16_up, const float *absmax_up, int blocksize_up, const void *m_sizes,
+                    int m_sizes_dtype, void *h, void *e_out, void *g_out, int64_t R, int N, int K, int E, int dtype,
+                    void *stream) {
+    return mfl_glu_fwd_nf4_tiled(x, src_rows, row_idx, idx_div, wq_gate, code16_gate, absmax_gate, nullptr,
+                                 blocksize_gate, wq_up, code16_up, absmax_up, nullptr, blocksize_up, m_sizes,
+                                 m_sizes_dtype, h, e_out, g_out, R, N, K, E, dtype, stream);
 }
 
 int mfl_nf4_dequant(const uint8_t *wq, const float *code16, const float *absmax, int blocksize, void *out, int64_t n,

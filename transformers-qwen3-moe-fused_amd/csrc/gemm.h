@@ -52,6 +52,8 @@ struct GemmFusion {
     int kt;
     // the same with the gated unit (w2 given, x2 not): thin weights of the second matrix; xt is shared
     const void *wt2;
+    // NF4: tile-ordered copies of the scales of w and w2 (see Nf4Matrix), or null
+    const float *absmax_tiled, *absmax_tiled_2;
 };
 
 // Pipelined bf16 MFMA kernels (direct global->LDS copies, multi-stage) for aligned shapes.
@@ -80,7 +82,15 @@ struct Nf4Matrix {
     const float *code16;
     const float *absmax;
     int bs_shift;  // log2 of the quantisation block size
+    // The scales once more in the order in which the streaming kernel's waves consume them (nf4_tile_absmax),
+    // or null: [expert][32-column tile][128-wide reduction stage][column of the tile][half of the stage].
+    const float *absmax_tiled = nullptr;
 };
+
+// Writes the tile-ordered copy of an (E, N, K) matrix's scales: E * ceil(N / 32) * (K / 128) * 64 floats
+// (nf4_tiled_absmax_floats; 0 for a shape without such a copy: K % 128 != 0 or blocks under 64 weights).
+int64_t nf4_tiled_absmax_floats(int blocksize, int N, int K, int E);
+int nf4_tile_absmax(const float *absmax, int blocksize, int N, int K, int E, float *out, hipStream_t stream);
 
 // The streaming form of gemm_nf4_decode (all operands copied straight to LDS, scale applied per block to the
 // partial sums): K % 128 == 0 and blocks of at least 64 weights, MFL_ERR_UNSUPPORTED otherwise.

@@ -294,7 +294,8 @@ int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const
     if (K % 64 != 0 || N % 8 != 0 || N < 8 || blocksize < 8) return MFL_ERR_UNSUPPORTED;
     if (!aligned(x, 16) || !aligned(wq, 16) || !aligned(y, 16)) return MFL_ERR_UNSUPPORTED;
     if (out_dtype != MFL_BF16 && out_dtype != MFL_F32) return MFL_ERR_UNSUPPORTED;
-    const Nf4Matrix w0 = {wq, code16, absmax, shift};
+    Nf4Matrix w0 = {wq, code16, absmax, shift};
+    if (fusion != nullptr) w0.absmax_tiled = fusion->absmax_tiled;
     Nf4Matrix w1 = w0;
     const int32_t *row_idx = nullptr;
     int idx_div = 1;
@@ -313,7 +314,7 @@ int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const
                 !aligned(fusion->w2, 16) || !aligned(fusion->e_out, 8) || !aligned(fusion->g_out, 8))
                 return MFL_ERR_UNSUPPORTED;
             glu = true;
-            w1 = Nf4Matrix{(const uint8_t *)fusion->w2, fusion->code16_2, fusion->absmax_2, shift2};
+            w1 = Nf4Matrix{(const uint8_t *)fusion->w2, fusion->code16_2, fusion->absmax_2, shift2, fusion->absmax_tiled_2};
             e_out = fusion->e_out;
             g_out = fusion->g_out;
         }

@@ -85,7 +85,7 @@ struct StreamShape {
     static constexpr int kOps = 2 * CB + 2 + CB;  // copies per wave and stage
 };
 
-template <bool GLU, typename TO>
+template <bool GLU, bool TILED, typename TO>
 __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restrict__ x,
                                                          const int32_t *__restrict__ row_idx, int idx_div,
                                                          Nf4Matrix w0, Nf4Matrix w1,
@@ -186,18 +186,25 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
         if (row_idx != nullptr) src_row = (uint32_t)row_idx[src_row] / (uint32_t)idx_div;
         x_src[j] = x + src_row * K + c * 8;
     }
-    const int NS = K / 128;
+    const int NS = K / 128, tiles32 = (N + 31) / 32;
+    // A copy of rows whose four rows all lie past the tile's last row is left out (nobody stores what the MFMAs
+    // make of that part of the stage): x_copies of the wave's two, the same number in every stage.
+    const int x_copies = rows > 8 * wave + 4 ? 2 : rows > 8 * wave ? 1 : 0;
     auto issue = [&](int stg) {
         unsigned char *const base = ring + (stg % RING) * S::kStage;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) copy16_to_lds(x_src[j] + (int64_t)stg * 128, base + (wave * 2 + j) * 1024);
+        for (int j = 0; j < 2; ++j)
+            if (j < x_copies) copy16_to_lds(x_src[j] + (int64_t)stg * 128, base + (wave * 2 + j) * 1024);
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
                 copy16_to_lds(w_src[cb][j] + (int64_t)stg * 64, base + S::kX + (wave * CB + cb) * S::kW + j * 1024);
-            copy4_to_lds(mat[cb].absmax + ((a_el[cb] + (int64_t)stg * 128) >> mat[cb].bs_shift),
-                         base + S::kX + 4 * CB * S::kW + (wave * CB + cb) * S::kA);
+            // the wave's 64 scales of the stage: 256 consecutive bytes of the tile-ordered copy where the caller
+            // brought one (two lines per copy), else two neighbours out of each column's own run (32 lines)
+            const float *a_src = TILED ? mat[cb].absmax_tiled + ((((int64_t)expert * tiles32 + j0 / 32) * NS + stg) * 64 + lane)
+                                       : mat[cb].absmax + ((a_el[cb] + (int64_t)stg * 128) >> mat[cb].bs_shift);
+            copy4_to_lds(a_src, base + S::kX + 4 * CB * S::kW + (wave * CB + cb) * S::kA);
         }
     };
     // ---- where this lane reads a stage: its 16 bytes of packed weights of step s2, its 16 bytes of row n for
@@ -216,13 +223,16 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
 #pragma unroll
         for (int r = 0; r < 16; ++r) tot[cb][r] = 0.f;
 
-    // Every wave issues the same S::kOps copies per stage, unconditionally (past the end they repeat the last
-    // stage, into a slot that is free), so "at most (RING - 2) * kOps of my copies outstanding" means that the
-    // stage about to be read has landed.
+    // Every wave issues the same number of copies per stage (S::kOps less the row copies it leaves out),
+    // unconditionally (past the end they repeat the last stage, into a slot that is free), so "at most RING - 2
+    // stages' worth of my copies outstanding" means that the stage about to be read has landed.
 #pragma unroll
     for (int q = 0; q < RING - 1; ++q) issue(q < NS ? q : NS - 1);
     for (int q = 0; q < NS; ++q) {
-        wait_vmcnt<(RING - 2) * S::kOps>();
+        // at most (RING - 2) stages' worth of this wave's copies outstanding
+        if (x_copies == 2) wait_vmcnt<(RING - 2) * S::kOps>();
+        else if (x_copies == 1) wait_vmcnt<(RING - 2) * (S::kOps - 1)>();
+        else wait_vmcnt<(RING - 2) * (S::kOps - 2)>();
         __syncthreads();  // stage q is whole (the first time round: so is the pair table); nobody reads stage q - 1 any more
         const unsigned char *const base = ring + (q % RING) * S::kStage;
         // the stage's packed weights and scales are asked of the LDS before the next copies are set up (some
@@ -312,7 +322,7 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     }
 }
 
-template <bool GLU, typename TO>
+template <bool GLU, bool TILED, typename TO>
 int launch_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
                   const void *m_sizes, int ms_i64, TO *y, TO *e_out, TO *g_out, int64_t R, int N, int K, int E,
                   hipStream_t stream) {
@@ -322,7 +332,7 @@ int launch_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf
     const int64_t row_tiles = R / 32 + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / 32)
     const int64_t grid = (row_tiles + 7) / 8 * 8 * tiles_n;  // row tiles in eights: one per XCD
     if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
-    auto *kernel = nf4_stream_kernel<GLU, TO>;
+    auto *kernel = nf4_stream_kernel<GLU, TILED, TO>;
     static PerDeviceOnce attr;
     // The kernel's table lookups take the dynamic LDS to start at address 0: any static LDS in this kernel
     // (a later __shared__ variable, an inlined helper that brings one) would move it, so the launcher asks the
@@ -342,7 +352,41 @@ int launch_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf
     return launch_status();
 }
 
+// out[((e * tiles32 + t) * NS + s) * 64 + l] = the scale of column 32 t + (l >> 1) (the last column past N), weights
+// 128 s + 64 (l & 1) .. + 63 of its reduction
+__global__ __launch_bounds__(256) void nf4_tile_absmax_kernel(const float *__restrict__ absmax, int bs_shift, int N, int K,
+                                                              int tiles32, int64_t total, float *__restrict__ out) {
+    const int NS = K / 128;
+    for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < total; i += gridDim.x * 256ll) {
+        const int l = (int)(i & 63);
+        const int64_t q = i >> 6;
+        const int s = (int)(q % NS);
+        const int64_t et = q / NS;
+        const int t = (int)(et % tiles32);
+        const int64_t e = et / tiles32;
+        int col = 32 * t + (l >> 1);
+        if (col >= N) col = N - 1;
+        out[i] = absmax[((e * N + col) * K + 128 * s + 64 * (l & 1)) >> bs_shift];
+    }
+}
+
 }  // namespace
+
+int64_t nf4_tiled_absmax_floats(int blocksize, int N, int K, int E) {
+    if (blocksize < 64 || (blocksize & (blocksize - 1)) != 0 || K % 128 != 0 || N <= 0 || E <= 0) return 0;
+    return (int64_t)E * ceil_div(N, 32) * (K / 128) * 64;
+}
+
+int nf4_tile_absmax(const float *absmax, int blocksize, int N, int K, int E, float *out, hipStream_t stream) {
+    const int64_t total = nf4_tiled_absmax_floats(blocksize, N, K, E);
+    if (total == 0) return MFL_ERR_UNSUPPORTED;
+    int shift = 0;
+    while ((1 << shift) < blocksize) ++shift;
+    const int64_t blocks = (total + 255) / 256;
+    nf4_tile_absmax_kernel<<<(unsigned)(blocks < 65536 ? blocks : 65536), 256, 0, stream>>>(absmax, shift, N, K,
+                                                                                          ceil_div(N, 32), total, out);
+    return launch_status();
+}
 
 int gemm_nf4_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
                     bool glu, const void *m_sizes, int ms_i64, void *y, void *e_out, void *g_out, int64_t R, int N,
@@ -350,14 +394,16 @@ int gemm_nf4_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const 
     // a 64-wide step must lie inside one quantisation block, and the scales are copied four bytes at a time
     if (K % 128 != 0 || w0.bs_shift < 6 || w1.bs_shift < 6) return MFL_ERR_UNSUPPORTED;
     if (!aligned(w0.absmax, 4) || !aligned(w1.absmax, 4)) return MFL_ERR_UNSUPPORTED;
-    if (glu)
-        return launch_stream<true, bf16_t>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (bf16_t *)y, (bf16_t *)e_out,
-                                           (bf16_t *)g_out, R, N, K, E, stream);
-    if (out_dtype == MFL_BF16)
-        return launch_stream<false, bf16_t>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (bf16_t *)y, nullptr, nullptr,
-                                            R, N, K, E, stream);
-    return launch_stream<false, float>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, (float *)y, nullptr, nullptr, R, N,
-                                       K, E, stream);
+    // the tile-ordered scales are used where the caller brought them for every matrix of the product
+    const bool tiled = w0.absmax_tiled != nullptr && (!glu || w1.absmax_tiled != nullptr) &&
+                       aligned(w0.absmax_tiled, 4) && (!glu || aligned(w1.absmax_tiled, 4));
+#define MFL_STREAM(GLU, TO, Y, EO, GO)                                                                          \
+    (tiled ? launch_stream<GLU, true, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream) \
+           : launch_stream<GLU, false, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream))
+    if (glu) return MFL_STREAM(true, bf16_t, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out);
+    if (out_dtype == MFL_BF16) return MFL_STREAM(false, bf16_t, (bf16_t *)y, nullptr, nullptr);
+    return MFL_STREAM(false, float, (float *)y, nullptr, nullptr);
+#undef MFL_STREAM
 }
 
 }  // namespace mfl

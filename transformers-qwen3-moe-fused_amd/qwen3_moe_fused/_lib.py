@@ -47,6 +47,12 @@ _SIGNATURES = {
     "mfl_glu_fwd_lora": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp]),
     "mfl_glu_fwd_nf4": (_i, [_vp, _i64, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _i64,
                              _i, _i, _i, _i, _vp]),
+    "mfl_nf4_tiled_absmax_floats": (_i64, [_i, _i, _i, _i]),
+    "mfl_nf4_tile_absmax": (_i, [_vp, _i, _i, _i, _i, _vp, _vp]),
+    "mfl_gemm_fwd_nf4_tiled": (_i, [_vp, _i64, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i,
+                                    _i, _vp]),
+    "mfl_glu_fwd_nf4_tiled": (_i, [_vp, _i64, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp,
+                                   _vp, _vp, _i64, _i, _i, _i, _i, _vp]),
     "mfl_nf4_dequant": (_i, [_vp, _vp, _vp, _i, _vp, _i64, _i, _vp]),
     "mfl_dequant_blockwise_u8": (_i, [_vp, _vp, _vp, _i, _f, _vp, _i64, _vp]),
     "mfl_nf4_quant": (_i, [_vp, _i, _i64, _i, _vp, _vp, _vp, _vp]),

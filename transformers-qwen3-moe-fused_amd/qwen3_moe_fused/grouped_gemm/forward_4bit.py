@@ -15,7 +15,7 @@ from typing import Optional
 import torch
 
 from .. import _lib
-from ..quantize.nf4 import resolve_absmax
+from ..quantize.nf4 import resolve_absmax, tiled_absmax
 from ._common import is_int_tensor
 
 
@@ -46,9 +46,16 @@ def grouped_gemm_forward_4bit(x: torch.Tensor, w_quant: torch.Tensor, w_quant_st
 
     y = torch.empty((rows, n), device=x.device, dtype=x.dtype if dtype is None else dtype)
     ms = _lib.as_index_tensor(m_sizes)
-    rc = _lib.lib().mfl_gemm_fwd_nf4(_lib.ptr(x), _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), blocksize,
-                                     _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(y), rows, n, k, experts,
-                                     _lib.dtype_code(x.dtype), _lib.dtype_code(y.dtype), _lib.stream())
+    tiled = tiled_absmax(w_quant_state, absmax, rows)  # decode-sized batches: scales in the order of consumption
+    if tiled is not None:
+        rc = _lib.lib().mfl_gemm_fwd_nf4_tiled(_lib.ptr(x), rows, None, 1, _lib.ptr(w_quant), _lib.ptr(code),
+                                               _lib.ptr(absmax), _lib.ptr(tiled), blocksize, _lib.ptr(ms),
+                                               _lib.itype_code(ms.dtype), _lib.ptr(y), rows, n, k, experts,
+                                               _lib.dtype_code(x.dtype), _lib.dtype_code(y.dtype), _lib.stream())
+    else:
+        rc = _lib.lib().mfl_gemm_fwd_nf4(_lib.ptr(x), _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), blocksize,
+                                         _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(y), rows, n, k, experts,
+                                         _lib.dtype_code(x.dtype), _lib.dtype_code(y.dtype), _lib.stream())
     if rc == -6:  # MFL_ERR_UNSUPPORTED (fp32 / fp16 rows, K % 8 != 0, blocksize < 8): dequantise, then the plain product
         from ..quantize.nf4 import dequantize_nf4
         from .forward import grouped_gemm_forward

@@ -23,7 +23,7 @@ import torch
 from .. import _lib
 from ..kernels.routing import _gather as gather_kernel
 from ..kernels.silu_mul import silu_mul_forward
-from ..quantize.nf4 import resolve_absmax
+from ..quantize.nf4 import resolve_absmax, tiled_absmax
 from ._common import check_operands, is_int_tensor
 from .forward import grouped_gemm_forward
 from .forward_4bit import grouped_gemm_forward_4bit
@@ -92,10 +92,19 @@ def grouped_gemm_forward_4bit_gathered(x_src: torch.Tensor, row_idx: torch.Tenso
     assert m_sizes.numel() == experts
     y = torch.empty((rows, n), device=x_src.device, dtype=x_src.dtype if dtype is None else dtype)
     ms = _lib.as_index_tensor(m_sizes)
-    rc = _lib.lib().mfl_gemm_fwd_nf4_gather(_lib.ptr(x_src), x_src.shape[0], _lib.ptr(row_idx), idx_div,
-                                            _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), blocksize,
-                                            _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(y), rows, n, k, experts,
-                                            _lib.dtype_code(x_src.dtype), _lib.dtype_code(y.dtype), _lib.stream())
+    tiled = tiled_absmax(w_quant_state, absmax, rows)
+    if tiled is not None:
+        rc = _lib.lib().mfl_gemm_fwd_nf4_tiled(_lib.ptr(x_src), x_src.shape[0], _lib.ptr(row_idx), idx_div,
+                                               _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), _lib.ptr(tiled),
+                                               blocksize, _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(y), rows,
+                                               n, k, experts, _lib.dtype_code(x_src.dtype),
+                                               _lib.dtype_code(y.dtype), _lib.stream())
+    else:
+        rc = _lib.lib().mfl_gemm_fwd_nf4_gather(_lib.ptr(x_src), x_src.shape[0], _lib.ptr(row_idx), idx_div,
+                                                _lib.ptr(w_quant), _lib.ptr(code), _lib.ptr(absmax), blocksize,
+                                                _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(y), rows, n, k,
+                                                experts, _lib.dtype_code(x_src.dtype), _lib.dtype_code(y.dtype),
+                                                _lib.stream())
     if rc == UNSUPPORTED:
         return grouped_gemm_forward_4bit(_gather(x_src, row_idx, idx_div), w_quant, w_quant_state, m_sizes, dtype)
     _lib.check(rc, "mfl_gemm_fwd_nf4_gather")
@@ -144,18 +153,20 @@ def grouped_glu_forward_4bit(x: torch.Tensor, gate_quant: torch.Tensor, gate_sta
     e = torch.empty_like(h) if return_products else None
     g = torch.empty_like(h) if return_products else None
     ms = _lib.as_index_tensor(m_sizes)
-    rc = _lib.lib().mfl_glu_fwd_nf4(_lib.ptr(x), x.shape[0], _lib.ptr(row_idx), idx_div,
-                                    _lib.ptr(gate_quant), _lib.ptr(code_g), _lib.ptr(absmax_g), bs_g,
-                                    _lib.ptr(up_quant), _lib.ptr(code_u), _lib.ptr(absmax_u), bs_u,
-                                    _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(h), _lib.ptr(e), _lib.ptr(g), rows,
-                                    n, k, experts, _lib.dtype_code(x.dtype), _lib.stream())
+    tiled_g, tiled_u = tiled_absmax(gate_state, absmax_g, rows), tiled_absmax(up_state, absmax_u, rows)
+    rc = _lib.lib().mfl_glu_fwd_nf4_tiled(_lib.ptr(x), x.shape[0], _lib.ptr(row_idx), idx_div,
+                                          _lib.ptr(gate_quant), _lib.ptr(code_g), _lib.ptr(absmax_g), _lib.ptr(tiled_g),
+                                          bs_g, _lib.ptr(up_quant), _lib.ptr(code_u), _lib.ptr(absmax_u),
+                                          _lib.ptr(tiled_u), bs_u, _lib.ptr(ms), _lib.itype_code(ms.dtype), _lib.ptr(h),
+                                          _lib.ptr(e), _lib.ptr(g), rows, n, k, experts, _lib.dtype_code(x.dtype),
+                                          _lib.stream())
     if rc == UNSUPPORTED:
         xg = x if row_idx is None else _gather(x, row_idx, idx_div)
         e = grouped_gemm_forward_4bit(xg, gate_quant, gate_state, m_sizes)
         g = grouped_gemm_forward_4bit(xg, up_quant, up_state, m_sizes)
         h = silu_mul_forward(e, g)
     else:
-        _lib.check(rc, "mfl_glu_fwd_nf4")
+        _lib.check(rc, "mfl_glu_fwd_nf4_tiled")
     return (h, e, g) if return_products else h
 
 

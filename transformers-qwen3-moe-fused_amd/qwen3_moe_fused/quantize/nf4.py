@@ -170,6 +170,38 @@ def resolve_absmax(quant_state) -> torch.Tensor:
     return absmax.contiguous()
 
 
+# rows per expert up to which the library's NF4 products run on the kernels that read tile-ordered scales
+_TILED_ROWS_PER_EXPERT = 72
+
+
+def tiled_absmax(quant_state, absmax: torch.Tensor, rows: int):
+    """The scales of an (E, N, K) NF4 matrix once more in the order in which the decode-sized kernels consume
+    them (``mfl_nf4_tile_absmax``), built on the first decode-sized call and kept on the quant state; ``None``
+    where it does not apply (a larger batch, a double-quantised state whose fp32 scales are rebuilt per call,
+    a shape without such a copy).  Costs as many bytes again as ``absmax`` (3 % of the packed weights)."""
+    cached = getattr(quant_state, "_mfl_absmax_tiled", None)
+    if cached is not None and cached[0] is absmax and cached[1] == absmax._version:
+        return cached[3] if rows <= cached[2] else None  # the path of every call but the first
+    if getattr(quant_state, "nested", False) or len(quant_state.shape) != 3:
+        return None
+    experts, n, k = (int(v) for v in quant_state.shape)
+    max_rows = _TILED_ROWS_PER_EXPERT * experts
+    if rows > max_rows:
+        return None
+    blocksize = int(quant_state.blocksize)
+    count = int(_lib.lib().mfl_nf4_tiled_absmax_floats(blocksize, n, k, experts))
+    out = None
+    if count > 0:
+        out = torch.empty(count, device=absmax.device, dtype=torch.float32)
+        rc = _lib.lib().mfl_nf4_tile_absmax(_lib.ptr(absmax), blocksize, n, k, experts, _lib.ptr(out), _lib.stream())
+        _lib.check(rc, "mfl_nf4_tile_absmax")
+    try:
+        quant_state._mfl_absmax_tiled = (absmax, absmax._version, max_rows, out)
+    except AttributeError:  # a state type with fixed attributes: rebuilt per call
+        pass
+    return out
+
+
 def _quantize_absmax(absmax: torch.Tensor, blocksize2: int = 256):
     """Second level of a double quantisation, as bitsandbytes does it: subtract the mean, then blockwise
     8-bit quantisation against the dynamic code book (nearest entry of x / max|block|).  Load-time work on
