@@ -62,18 +62,84 @@ __device__ int g_wide_trace_n;
 #define MFL_TR(tag)
 #endif
 
-// s_waitcnt vmcnt(n rounded down to a multiple of 8), n wave-uniform
+// s_waitcnt vmcnt(min(n, 63)), n wave-uniform.  Exact, not rounded down: a wait for a few operations fewer than
+// necessary also waits for the first copies of the step after the one that is needed.  The instruction takes its
+// count as an immediate only, so this is a computed jump into a table of 64 of them (8 bytes an entry; the three
+// instructions between s_getpc_b64 and the table are 12 bytes).
 __device__ __forceinline__ void wait_vmcnt_upto(int n) {
-    switch (n >> 3) {
-        case 0: wait_vmcnt<0>(); break;
-        case 1: wait_vmcnt<8>(); break;
-        case 2: wait_vmcnt<16>(); break;
-        case 3: wait_vmcnt<24>(); break;
-        case 4: wait_vmcnt<32>(); break;
-        case 5: wait_vmcnt<40>(); break;
-        case 6: wait_vmcnt<48>(); break;
-        default: wait_vmcnt<56>(); break;
-    }
+    uint32_t t;
+    n = __builtin_amdgcn_readfirstlane(n);
+    asm volatile(
+        "s_min_u32 %[t], %[n], 63\n\ts_lshl_b32 %[t], %[t], 3\n\ts_add_u32 %[t], %[t], 12\n\t"
+        "s_getpc_b64 s[98:99]\n\ts_add_u32 s98, s98, %[t]\n\ts_addc_u32 s99, s99, 0\n\ts_setpc_b64 s[98:99]\n\t"
+        "s_waitcnt vmcnt(0)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(1)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(2)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(3)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(4)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(5)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(6)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(7)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(8)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(9)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(10)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(11)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(12)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(13)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(14)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(15)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(16)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(17)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(18)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(19)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(20)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(21)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(22)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(23)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(24)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(25)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(26)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(27)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(28)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(29)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(30)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(31)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(32)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(33)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(34)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(35)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(36)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(37)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(38)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(39)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(40)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(41)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(42)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(43)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(44)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(45)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(46)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(47)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(48)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(49)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(50)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(51)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(52)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(53)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(54)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(55)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(56)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(57)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(58)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(59)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(60)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(61)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(62)\n\ts_branch .Lwv_end_%=\n\t"
+        "s_waitcnt vmcnt(63)\n\ts_branch .Lwv_end_%=\n\t"
+        ".Lwv_end_%=:"
+        : [t] "=&s"(t)
+        : [n] "s"(n)
+        : "memory", "scc", "s98", "s99");
 }
 
 // f(IC<0>{}), ..., f(IC<N-1>{}): a loop whose index is a constant expression inside the body
