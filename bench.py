@@ -619,9 +619,13 @@ def main() -> int:
             out.backward(gouts[i % NB])
             blk.zero_grad(set_to_none=True)
 
-        us = _event_us(train_step, 20, 10, stream)
+        blk.fuse_backward = True    # the gated unit's backward in the epilogue of the down projection's input gradient
+        us_fb = _event_us(train_step, 30, 15, stream)
+        blk.fuse_backward = False   # the default: dh is written, then read by silu_mul_backward
+        us = _event_us(train_step, 30, 15, stream)
         bf16_block["block_fwd_bwd"] = {"us": round(us, 1), "tokens_per_s": round(TOKENS / us * 1e6),
-                                       "tflops": round(9 * flop / us / 1e6, 1)}   # 3 products x (fwd + dX + dW)
+                                       "tflops": round(9 * flop / us / 1e6, 1),   # 3 products x (fwd + dX + dW)
+                                       "silu_mul_backward_in_dx_epilogue_us": round(us_fb, 1)}
         extra["bf16_sparse_block_fwd_config2"] = bf16_block
         del blk, toks
         out["extra"] = extra

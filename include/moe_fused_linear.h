@@ -130,6 +130,17 @@ MFL_API int mfl_gemm_dx_dual(const void *dy1, const void *w1, const void *dy2, c
                      const void *m_sizes, int m_sizes_dtype, void *dx, int64_t R, int N, int K,
                      int E, int in_dtype, int out_dtype, void *stream);
 
+/* The input gradient of the down projection with the backward of the gated unit in its epilogue:
+ * dh = mfl_gemm_dx(dy, w) is not stored; de, dg (and h = silu(e) * g again where h is not NULL) leave the kernel
+ * as mfl_silu_mul_bwd computes them from a stored bf16 dh, bit for bit.  dy (R,K), w (E,K,N) as in mfl_gemm_dx;
+ * e, g, de, dg, h (R,N); de may be e and dg may be g (in place).  bf16 only.  Saves the (R,N) round trip of dh
+ * and one launch per training step (qwen3_moe_fused/kernels/fast_lora.py:133-137 followed by
+ * kernels/silu_mul.py:84-111 in the reference).  MFL_ERR_UNSUPPORTED for shapes outside the pipelined kernels:
+ * the caller then runs mfl_gemm_dx and mfl_silu_mul_bwd. */
+MFL_API int mfl_gemm_dx_silu_bwd(const void *dy, const void *w, const void *e, const void *g,
+                         const void *m_sizes, int m_sizes_dtype, void *de, void *dg, void *h, int64_t R,
+                         int N, int K, int E, int dtype, void *stream);
+
 /* A product with the rank-r term of a LoRA adapter in the same reduction: one accumulator, one
  * rounding, one pass over the output, where the reference adds the two products
  * (qwen3_moe_fused/lora.py:134; matmul_lora at kernels/fast_lora.py:65-88,127-131,151-152).

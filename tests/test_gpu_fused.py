@@ -271,6 +271,62 @@ def test_two_term_input_gradient(R, N, K, E):
         check_close(dx, to_np32(dx_cat), what="two-term dx vs concatenated product")
 
 
+from qwen3_moe_fused.grouped_gemm.fused import grouped_gemm_forward_transposed_silu_bwd  # noqa: E402
+from qwen3_moe_fused.kernels.silu_mul import silu_mul_backward  # noqa: E402
+
+
+# (de, dg[, h]) = silu_mul_backward(dy (R, K) @ w[e] (K, N), e, g): the product's epilogue against the two kernels, bit
+# for bit (the product is rounded to bf16 before it meets e and g, as when it is stored), and against the oracle.
+# Shapes: the down projection's (several tiles per expert, experts without rows), a width that leaves the last
+# column tile partly empty, one reduction step, more experts than rows; the last two have no pipelined kernel
+# (N % 8 != 0; fp32) and run as two launches.
+@pytest.mark.parametrize("R,N,K,E,dtype", [(3000, 768, 2048, 8, torch.bfloat16), (700, 200, 64, 5, torch.bfloat16),
+                                           (33, 8, 192, 40, torch.bfloat16), (5000, 392, 128, 2, torch.bfloat16),
+                                           (9000, 768, 256, 4, torch.bfloat16),   # 256 x 256 tiles
+                                           (64, 20, 72, 4, torch.bfloat16), (50, 24, 64, 3, torch.float32)])
+def test_input_gradient_with_silu_mul_backward_in_the_epilogue(R, N, K, E, dtype):
+    gn = gen(R + N)
+    dy = randn((R, K), gn, 1.0, dtype).to(DEV)
+    w = randn((E, K, N), gn, 0.05, dtype).to(DEV)
+    e, g = randn((R, N), gn, 2.0, dtype).to(DEV), randn((R, N), gn, 1.0, dtype).to(DEV)
+    ms = m_sizes_uniform(R, E, gn)
+    if E >= 4:
+        ms[1] += ms[2]
+        ms[2] = 0                                # an expert without rows
+    msd = ms.to(DEV)
+    dh = grouped_gemm_forward_transposed(dy, w, msd)
+    de_ref, dg_ref = silu_mul_backward(dh, e, g)
+    de, dg, h = grouped_gemm_forward_transposed_silu_bwd(dy, w, e, g, msd, return_h=True)
+    assert torch.equal(de, de_ref) and torch.equal(dg, dg_ref), "the same bits as product, then silu_mul_backward"
+    assert torch.equal(h, silu_mul_forward(e, g))
+    de2, dg2 = grouped_gemm_forward_transposed_silu_bwd(dy, w, e, g, msd)
+    assert torch.equal(de2, de_ref) and torch.equal(dg2, dg_ref)
+    if dtype == torch.bfloat16:
+        sel = oracle.sel_from_m_sizes(ms.numpy())
+        dh_o = oracle.round_bf16(oracle.linear_bwd_input(to_np32(dy), to_np32(w), sel))
+        _, de_o, dg_o = oracle.silu_mul_bwd_f32(dh_o, to_np32(e), to_np32(g))
+        check_close(de, de_o, 3e-2, 3e-2 * float(np.abs(de_o).max()), "de vs oracle")
+        check_close(dg, dg_o, 3e-2, 3e-2 * float(np.abs(dg_o).max()), "dg vs oracle")
+
+
+def test_input_gradient_with_silu_mul_backward_in_place():
+    """de may be e and dg may be g: every piece is read before it is written, by the lane that writes it."""
+    from qwen3_moe_fused import _lib
+    R, N, K, E = 1500, 392, 256, 6
+    gn = gen(7)
+    dy = randn((R, K), gn, 1.0, torch.bfloat16).to(DEV)
+    w = randn((E, K, N), gn, 0.05, torch.bfloat16).to(DEV)
+    e, g = randn((R, N), gn, 2.0, torch.bfloat16).to(DEV), randn((R, N), gn, 1.0, torch.bfloat16).to(DEV)
+    ms = m_sizes_uniform(R, E, gn).to(DEV)
+    de_ref, dg_ref, h_ref = grouped_gemm_forward_transposed_silu_bwd(dy, w, e, g, ms, return_h=True)
+    e2, g2, h2 = e.clone(), g.clone(), torch.empty_like(e)
+    rc = _lib.lib().mfl_gemm_dx_silu_bwd(_lib.ptr(dy), _lib.ptr(w), _lib.ptr(e2), _lib.ptr(g2), _lib.ptr(ms),
+                                         _lib.itype_code(ms.dtype), _lib.ptr(e2), _lib.ptr(g2), _lib.ptr(h2), R, N, K, E,
+                                         _lib.dtype_code(torch.bfloat16), _lib.stream())
+    _lib.check(rc, "mfl_gemm_dx_silu_bwd")
+    assert torch.equal(e2, de_ref) and torch.equal(g2, dg_ref) and torch.equal(h2, h_ref)
+
+
 from qwen3_moe_fused.grouped_gemm.fused import (grouped_gemm_forward_lora,  # noqa: E402
                                                 grouped_gemm_forward_transposed_lora)
 

@@ -324,18 +324,25 @@ def test_fused_front_of_block_matches_module_by_module_path(T, E, k, H, I):
     hidden = randn((1, T, H), gen(T), 1.0, torch.bfloat16).to(DEV)
     gout = randn((1, T, H), gen(T + 1), 1.0, torch.bfloat16).to(DEV)
     results = []
-    for fuse in (True, False):
-        blk.fuse_front = fuse
+    for fuse, fuse_backward in ((True, True), (False, False), (True, False)):
+        blk.fuse_front, blk.fuse_backward = fuse, fuse_backward
         blk.zero_grad(set_to_none=True)
         h = hidden.clone().requires_grad_()
         out, logits = blk(h)
         out.backward(gout)
         results.append((out.detach(), h.grad, {n: p.grad.clone() for n, p in blk.named_parameters()}))
-    (o1, g1, p1), (o2, g2, p2) = results
+    (o1, g1, p1), (o2, g2, p2), (o3, g3, p3) = results
+    assert torch.equal(o3, o1) and torch.equal(g3, g1), "the backward epilogue changes no bit of the fused path"
+    for n in p1:
+        assert torch.equal(p3[n], p1[n]), n
     assert torch.equal(o1, o2), "same kernels' arithmetic, same roundings"
     _grads_close(g1, g2, "d hidden")
     for n in p1:
         _grads_close(p1[n], p2[n], n)
+    # the gated unit's backward in the down projection's input gradient returns the bits of the separate kernel:
+    # the three weight gradients, products over the same de, dg and h, are the same bits too
+    for n in ("gate_proj.weight", "up_proj.weight", "down_proj.weight"):
+        assert torch.equal(p1[n], p2[n]), n
     # inference: no products are kept, same output
     blk.fuse_front = True
     with torch.no_grad():

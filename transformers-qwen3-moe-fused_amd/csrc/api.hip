@@ -219,6 +219,24 @@ int mfl_gemm_dx_dual(const void *dy1, const void *w1, const void *dy2, const voi
                           (hipStream_t)stream, &fu);
 }
 
+int mfl_gemm_dx_silu_bwd(const void *dy, const void *w, const void *e, const void *g, const void *m_sizes,
+                         int m_sizes_dtype, void *de, void *dg, void *h, int64_t R, int N, int K, int E, int dtype,
+                         void *stream) {
+    int rc = check_gemm(dy, w, m_sizes, m_sizes_dtype, de, R, N, K, E, dtype, dtype);
+    if (rc) return rc;
+    if (R > 0 && (!e || !g || !dg)) return MFL_ERR_NULL;
+    if (R == 0) return MFL_OK;
+    if (dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    GemmFusion fu = {nullptr, 1, 0, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr};
+    fu.bw_e = e;
+    fu.bw_g = g;
+    fu.bw_de = de;
+    fu.bw_dg = dg;
+    fu.bw_h = h;
+    return gemm_bf16_pipe(MODE_DX, dy, w, m_sizes, m_sizes_dtype == MFL_I64, nullptr, R, N, K, E, MFL_BF16, 1.0f, 0,
+                          (hipStream_t)stream, &fu);
+}
+
 int mfl_gemm_fwd_lora(const void *x, const void *w, const void *xt, const void *wt, int KT, const void *m_sizes,
                       int m_sizes_dtype, void *y, int64_t R, int N, int K, int E, int in_dtype, int out_dtype,
                       void *stream) {

@@ -52,6 +52,20 @@ __device__ __forceinline__ T silu_fwd_one(T e, T g) {
     return from_f32<T>(to_f32(f) * to_f32(g));
 }
 
+// Backward of h = silu(e) * g for one element: h again, de and dg from dh (the rounding chain of the reference's
+// kernel, qwen3_moe_fused/kernels/silu_mul.py:84-111).
+template <typename T>
+__device__ __forceinline__ void silu_bwd_one(T dh, T e, T g, T &h, T &de, T &dg) {
+    const float e32 = to_f32(e), g32 = to_f32(g), dh32 = to_f32(dh);
+    const float se = sigmoid_f32(e32);
+    const float ese = e32 * se;
+    const float f = to_f32(from_f32<T>(ese));
+    const float df = to_f32(from_f32<T>(dh32 * g32));
+    h = from_f32<T>(f * g32);
+    dg = from_f32<T>(f * dh32);
+    de = from_f32<T>(df * se * (1.0f + e32 - ese));
+}
+
 __device__ __forceinline__ int load_msize(const void *m_sizes, int is_i64, int e) {
     return is_i64 ? (int)((const int64_t *)m_sizes)[e] : ((const int32_t *)m_sizes)[e];
 }

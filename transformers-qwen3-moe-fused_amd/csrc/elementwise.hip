@@ -35,18 +35,6 @@ __device__ __forceinline__ void st_vec(T *p, const Vec<T> &r) {
 // ---------------------------------------------------------------- SiLU-mul
 
 template <typename T>
-__device__ __forceinline__ void silu_bwd_one(T dh, T e, T g, T &h, T &de, T &dg) {
-    const float e32 = to_f32(e), g32 = to_f32(g), dh32 = to_f32(dh);
-    const float se = sigmoid_f32(e32);
-    const float ese = e32 * se;
-    const float f = to_f32(from_f32<T>(ese));
-    const float df = to_f32(from_f32<T>(dh32 * g32));
-    h = from_f32<T>(f * g32);
-    dg = from_f32<T>(f * dh32);
-    de = from_f32<T>(df * se * (1.0f + e32 - ese));
-}
-
-template <typename T>
 __global__ __launch_bounds__(256) void silu_fwd_kernel(const T *e, const T *g, T *h, int64_t n, int vec_ok) {
     constexpr int V = Vec<T>::N;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;

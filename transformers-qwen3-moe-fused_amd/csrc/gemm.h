@@ -54,6 +54,11 @@ struct GemmFusion {
     const void *wt2;
     // NF4: tile-ordered copies of the scales of w and w2 (see Nf4Matrix), or null
     const float *absmax_tiled, *absmax_tiled_2;
+    // DX with the backward of the gated unit in its epilogue (bw_e given): the product dh = dy w is not stored;
+    // de, dg (and h = silu(e) g where bw_h is given) are computed from it and the forward products e, g (all
+    // (R, N) bf16; de may be e and dg may be g) as silu_mul_bwd computes them from a stored dh
+    const void *bw_e, *bw_g;
+    void *bw_de, *bw_dg, *bw_h;
 };
 
 // Pipelined bf16 MFMA kernels (direct global->LDS copies, multi-stage) for aligned shapes.

@@ -76,11 +76,16 @@ struct FwdFusion {
     // with the GLU epilogue: the thin weights of the second (up) matrix; at is shared (its columns are the two
     // adapters' activations side by side, and each matrix's thin weights are zero over the other's columns)
     const void *bt2;
+    // DX: the backward of the gated unit in the epilogue (see GemmFusion::bw_e)
+    const void *bw_e, *bw_g;
+    void *bw_de, *bw_dg, *bw_h;
 };
 
 // FUSE: 0 plain, 1 two weight matrices and the silu(gate) * up epilogue, 2 a thin last term in the reduction (built
 // as a kernel of its own: the test for it in every step cost the plain products 3-5 %), 3 both: each of the two
-// matrices with thin weights of its own, against one thin left operand.
+// matrices with thin weights of its own, against one thin left operand; 4 the input gradient with the gated unit's
+// backward in its epilogue (a kernel of its own: its epilogue holds pieces of e and g in registers beside the
+// accumulators, which the plain input gradient has no room for).
 template <int MB, int NB, int BK, int S, int WGM, int WGN, int MODE, bool NF4, int FUSE, typename TO>
 __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *__restrict__ a,
                                                                   const bf16_t *__restrict__ b,
@@ -88,7 +93,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                                                                   TO *__restrict__ c, int64_t R, int N, int K, int E,
                                                                   float alpha, int accumulate, Nf4Params nf4,
                                                                   FwdFusion fu) {
-    constexpr bool GLU = FUSE == 1 || FUSE == 3, THIN = FUSE >= 2;
+    constexpr bool GLU = FUSE == 1 || FUSE == 3, THIN = FUSE == 2 || FUSE == 3, BWG = FUSE == 4;
+    static_assert(!BWG || (MODE == MODE_DX && sizeof(TO) == 2), "the gated unit's backward: input gradient, bf16");
     static_assert(!THIN || MODE != MODE_DW, "the thin last term belongs to the row-grouped products");
     static_assert(!NF4 || (MODE != MODE_DW && S == 2 && BK == 64), "NF4 weights: row-grouped products, two stages");
     static_assert(!GLU || (MODE == MODE_FWD && WGN % 2 == 0 && sizeof(TO) == 2 && BK == 64),
@@ -829,6 +835,51 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_pipe_kernel(const bf16_t *
                     }
                 // the same wave reads back what it wrote: LDS operations of one wave complete in order
                 const int row_base = i0 + (wm + WGM * t) * 32;
+                if constexpr (BWG) {
+                    // the product is the gradient of h = silu(e) g: its pieces meet the same pieces of e and g
+                    // (requested for the whole block first) and leave as de and dg, h where asked for
+                    // One piece at a time: with two in flight the 320 x 192 tile spills ten registers, with a whole
+                    // block's twelve loads fifty, and either is slower.
+                    constexpr int NQ = (32 * CPR + 63) / 64, QB = 1;  // pieces per lane; requested QB at a time
+#pragma unroll
+                    for (int q0 = 0; q0 < NQ; q0 += QB) {
+                        uint4_t e_in[QB], g_in[QB];
+#pragma unroll
+                        for (int qi = 0; qi < QB; ++qi) {
+                            const int q = (q0 + qi) * 64 + lane, row = row_base + q / CPR, col = j0 + wn * WTN + (q % CPR) * 8;
+                            if (q0 + qi >= NQ || q >= 32 * CPR || row >= i_end || col >= j_end) continue;
+                            const int64_t o = (int64_t)row * ldc + col;
+                            e_in[qi] = __builtin_nontemporal_load((const uint4_t *)((const bf16_t *)fu.bw_e + o));
+                            g_in[qi] = __builtin_nontemporal_load((const uint4_t *)((const bf16_t *)fu.bw_g + o));
+                        }
+#pragma unroll
+                        for (int qi = 0; qi < QB; ++qi) {
+                            const int q = (q0 + qi) * 64 + lane, row_l = q / CPR, lcol = (q % CPR) * 8;
+                            const int row = row_base + row_l, col = j0 + wn * WTN + lcol;
+                            if (q0 + qi >= NQ || q >= 32 * CPR || row >= i_end || col >= j_end) continue;
+                            union {
+                                uint4_t u;
+                                bf16x8 v;
+                            } dh8, e8, g8, h8, de8, dg8;
+                            dh8.u = *(const uint4_t *)(ep + row_l * ROWB + lcol * 2);
+                            e8.u = e_in[qi];
+                            g8.u = g_in[qi];
+#pragma unroll
+                            for (int u = 0; u < 8; ++u) {
+                                bf16_t h1, de1, dg1;
+                                silu_bwd_one<bf16_t>(dh8.v[u], e8.v[u], g8.v[u], h1, de1, dg1);
+                                h8.v[u] = h1;
+                                de8.v[u] = de1;
+                                dg8.v[u] = dg1;
+                            }
+                            const int64_t o = (int64_t)row * ldc + col;
+                            __builtin_nontemporal_store(de8.u, (uint4_t *)((bf16_t *)fu.bw_de + o));
+                            __builtin_nontemporal_store(dg8.u, (uint4_t *)((bf16_t *)fu.bw_dg + o));
+                            if (fu.bw_h) __builtin_nontemporal_store(h8.u, (uint4_t *)((bf16_t *)fu.bw_h + o));
+                        }
+                    }
+                    continue;
+                }
                 for (int q = lane; q < 32 * CPR; q += 64) {
                     const int row_l = q / CPR, lcol = (q % CPR) * 8;
                     const int row = row_base + row_l;
@@ -974,6 +1025,14 @@ int launch_pipe(int mode, const void *a, const void *b, const void *m_sizes, int
         } else {
             return MFL_ERR_UNSUPPORTED;
         }
+    } else if (fu.bw_e != nullptr) {
+        // the gated unit's backward in the epilogue: built with the configurations that have the GLU epilogue
+        if constexpr ((MODES & 8) != 0 && (MODES & 2) != 0 && sizeof(TO) == 2) {
+            if (mode != MODE_DX || nf4 != nullptr || accumulate) return MFL_ERR_UNSUPPORTED;
+            MFL_PIPE(MODE_DX, false, 4)
+        } else {
+            return MFL_ERR_UNSUPPORTED;
+        }
     } else if (nf4 != nullptr && mode == MODE_DX) {
         if constexpr ((MODES & 2) && S == 2 && BK == 64 && NB * 64 <= NT) MFL_PIPE(MODE_DX, true, false)
         else return MFL_ERR_UNSUPPORTED;
@@ -1091,6 +1150,17 @@ int make_fusion(const GemmFusion *f, int K, bool nf4, FwdFusion *out) {
         out->bt2 = glu_thin ? f->wt2 : nullptr;
         out->kthin = f->kt;
     }
+    if (f->bw_e != nullptr) {
+        if (nf4 || f->bw_g == nullptr || f->bw_de == nullptr || f->bw_dg == nullptr || f->row_idx != nullptr ||
+            f->x2 != nullptr || f->w2 != nullptr || f->xt != nullptr || !aligned(f->bw_e, 16) || !aligned(f->bw_g, 16) ||
+            !aligned(f->bw_de, 16) || !aligned(f->bw_dg, 16) || !aligned(f->bw_h, 16))
+            return MFL_ERR_UNSUPPORTED;
+        out->bw_e = f->bw_e;
+        out->bw_g = f->bw_g;
+        out->bw_de = f->bw_de;
+        out->bw_dg = f->bw_dg;
+        out->bw_h = f->bw_h;
+    }
     if (f->x2 != nullptr) {
         // two-term input gradient: whole reduction steps only, bf16 weights
         if (nf4 || f->w2 == nullptr || K % 64 != 0 || !aligned(f->x2, 16) || !aligned(f->w2, 16) ||
@@ -1129,7 +1199,10 @@ int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, 
     if (fusion != nullptr) {
         // two full terms: DX; a thin last term: FWD or DX; everything else: FWD
         if (mode == MODE_DW || (fusion->x2 != nullptr && mode != MODE_DX) ||
-            (mode == MODE_DX && fusion->x2 == nullptr && fusion->xt == nullptr))
+            (mode == MODE_DX && fusion->x2 == nullptr && fusion->xt == nullptr && fusion->bw_e == nullptr))
+            return MFL_ERR_UNSUPPORTED;
+        // the gated unit's backward sits in the bf16, non-accumulating epilogue of DX
+        if (fusion->bw_e != nullptr && (mode != MODE_DX || out_dtype != MFL_BF16 || accumulate || alpha != 1.0f))
             return MFL_ERR_UNSUPPORTED;
         if (fusion->x2 == nullptr && fusion->w2 != nullptr && (out_dtype != MFL_BF16 || accumulate || alpha != 1.0f))
             return MFL_ERR_UNSUPPORTED;

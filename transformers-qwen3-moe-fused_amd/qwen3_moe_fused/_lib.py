@@ -36,6 +36,7 @@ _SIGNATURES = {
     "mfl_gemm_fwd_nf4": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
     "mfl_gemm_dx_nf4": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _f, _i, _vp]),
     "mfl_gemm_dx_dual": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
+    "mfl_gemm_dx_silu_bwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp]),
     "mfl_gemm_fwd_lora": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
     "mfl_gemm_dx_lora": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
     "mfl_gemm_fwd_nf4_lora": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _vp]),

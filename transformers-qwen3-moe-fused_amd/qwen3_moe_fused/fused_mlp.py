@@ -12,8 +12,9 @@ from __future__ import annotations
 import torch
 
 from .grouped_gemm.backward_dw import grouped_gemm_backward_dw
-from .grouped_gemm.fused import (grouped_gemm_forward_transposed_dual, grouped_glu_forward,
-                                 grouped_glu_forward_4bit)
+from .grouped_gemm.forward import grouped_gemm_forward
+from .grouped_gemm.fused import (grouped_gemm_forward_transposed_dual, grouped_gemm_forward_transposed_silu_bwd,
+                                 grouped_glu_forward, grouped_glu_forward_4bit)
 from .kernels.routing import _combine, _gather, _scatter
 from .kernels.silu_mul import silu_mul_backward
 from .grouped_gemm.forward_4bit import grouped_gemm_forward_transposed_4bit
@@ -59,6 +60,52 @@ def moe_fused_glu(tokens: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor
     Result (T * num_selected, intermediate), rows grouped by expert.  Differentiable in
     ``tokens``, ``w_gate`` and ``w_up``."""
     return _GluGathered.apply(tokens, w_gate, w_up, m_sizes, sort_idx, inv_sort_idx, num_selected)
+
+
+class _MlpGathered(torch.autograd.Function):
+    """``moe_fused_glu`` followed by the down projection, as one node of the graph: its backward runs the down
+    projection's input gradient with the gated unit's backward in the epilogue (``dh`` is never written), then
+    what ``_GluGathered.backward`` runs."""
+
+    @staticmethod
+    def forward(ctx, tokens, w_gate, w_up, w_down, m_sizes, sort_idx, inv_sort_idx, k):
+        need = any(ctx.needs_input_grad[:4])
+        out = grouped_glu_forward(tokens, w_gate, w_up, m_sizes, sort_idx, k, return_products=need)
+        h, e, g = out if need else (out, None, None)
+        y = grouped_gemm_forward(h, w_down, m_sizes)
+        if need:
+            ctx.save_for_backward(tokens, w_gate, w_up, w_down, m_sizes, sort_idx, inv_sort_idx, e, g, h)
+            ctx.k = k
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        tokens, w_gate, w_up, w_down, m_sizes, sort_idx, inv_sort_idx, e, g, h = ctx.saved_tensors
+        dy = dy.contiguous()
+        d_tokens = d_gate = d_up = d_down = None
+        if ctx.needs_input_grad[3]:
+            d_down = grouped_gemm_backward_dw(h, dy, m_sizes, w_down.dtype)
+        if any(ctx.needs_input_grad[:3]):
+            de, dg = grouped_gemm_forward_transposed_silu_bwd(dy, w_down, e, g, m_sizes)
+            if ctx.needs_input_grad[0]:
+                dx = grouped_gemm_forward_transposed_dual(de, w_gate, dg, w_up, m_sizes, tokens.dtype)
+                d_tokens = _combine(dx, inv_sort_idx, None, tokens.shape[0], ctx.k)
+            if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+                xg = _scatter(tokens, inv_sort_idx, ctx.k, None) if ctx.k > 1 else _gather(tokens, sort_idx, ctx.k, None)
+                if ctx.needs_input_grad[1]:
+                    d_gate = grouped_gemm_backward_dw(xg, de, m_sizes, w_gate.dtype)
+                if ctx.needs_input_grad[2]:
+                    d_up = grouped_gemm_backward_dw(xg, dg, m_sizes, w_up.dtype)
+        return d_tokens, d_gate, d_up, d_down, None, None, None, None
+
+
+def moe_fused_mlp(tokens: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
+                  m_sizes: torch.Tensor, sort_idx: torch.Tensor, inv_sort_idx: torch.Tensor,
+                  num_selected: int) -> torch.Tensor:
+    """``moe_fused_linear(moe_fused_glu(tokens, w_gate, w_up, ...), w_down, m_sizes)``: the three expert
+    projections of the block (modular_qwen3_moe_fused.py:95-110 of the reference) as one differentiable op.
+    ``w_down`` (E, hidden, intermediate).  Result (T * num_selected, hidden), rows grouped by expert."""
+    return _MlpGathered.apply(tokens, w_gate, w_up, w_down, m_sizes, sort_idx, inv_sort_idx, num_selected)
 
 
 class _GluGathered4bit(torch.autograd.Function):

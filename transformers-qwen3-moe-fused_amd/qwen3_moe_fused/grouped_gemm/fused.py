@@ -194,6 +194,39 @@ def grouped_gemm_forward_transposed_dual(dy1: torch.Tensor, w1: torch.Tensor, dy
     return dx
 
 
+def grouped_gemm_forward_transposed_silu_bwd(dy: torch.Tensor, w: torch.Tensor, e: torch.Tensor, g: torch.Tensor,
+                                             m_sizes: torch.Tensor, return_h: bool = False):
+    """``silu_mul_backward(grouped_gemm_forward_transposed(dy, w, m_sizes), e, g)`` in one kernel: the input
+    gradient of the down projection never reaches memory, its pieces meet those of ``e`` and ``g`` in the
+    product's epilogue.  Returns ``(de, dg)`` or ``(de, dg, h)``; the same bits as the two kernels."""
+    from ..kernels.silu_mul import silu_mul_forward
+    from .forward_transposed import grouped_gemm_forward_transposed
+
+    check_operands(m_sizes, dy, w, e, g)
+    assert dy.ndim == 2 and w.ndim == 3 and e.shape == g.shape
+    rows, k = dy.shape
+    experts, k_w, n = w.shape
+    assert k_w == k and m_sizes.numel() == experts and e.shape == (rows, n)
+    de, dg = torch.empty_like(e), torch.empty_like(g)
+    h = torch.empty_like(e) if return_h else None
+    ms = _lib.as_index_tensor(m_sizes)
+    rc = UNSUPPORTED
+    if dy.dtype == torch.bfloat16 and w.dtype == dy.dtype and e.dtype == dy.dtype and g.dtype == dy.dtype:
+        rc = _lib.lib().mfl_gemm_dx_silu_bwd(_lib.ptr(dy), _lib.ptr(w), _lib.ptr(e), _lib.ptr(g), _lib.ptr(ms),
+                                             _lib.itype_code(ms.dtype), _lib.ptr(de), _lib.ptr(dg), _lib.ptr(h), rows, n,
+                                             k, experts, _lib.dtype_code(dy.dtype), _lib.stream())
+    if rc == UNSUPPORTED:
+        from ..kernels.silu_mul import silu_mul_backward
+
+        dh = grouped_gemm_forward_transposed(dy, w, m_sizes, e.dtype)
+        de, dg = silu_mul_backward(dh, e, g)
+        if return_h:
+            h = silu_mul_forward(e, g)
+    else:
+        _lib.check(rc, "mfl_gemm_dx_silu_bwd")
+    return (de, dg, h) if return_h else (de, dg)
+
+
 def grouped_gemm_forward_lora(x: torch.Tensor, w: torch.Tensor, xt: torch.Tensor, wt: torch.Tensor,
                               m_sizes: torch.Tensor, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """``grouped_gemm_forward(x, w, m_sizes) + grouped_gemm_forward(xt, wt, m_sizes)`` in one kernel: a product
