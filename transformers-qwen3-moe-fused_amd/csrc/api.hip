@@ -45,11 +45,10 @@ int run_gemm(int mode, const void *a, const void *b, const void *m_sizes, int ms
     if (in_dtype == MFL_BF16) {
         // weight gradient from about 64 rows per expert on: the four-wave kernel (85.6 against 99.5 us at 64 rows per
         // expert, 156 against 170 us at 256, N = 2048, K = 768, E = 128; below that the eight-wave tiles are ahead)
-        // the same kernel for the row-grouped products with a short reduction and a wide output (the down
-        // projection's forward product, the gate projection's input gradient: N = 2048, K = 768): many short tiles
-        // per workgroup, where one stream of reduction steps across tiles and output stores that leave under the
-        // next tile's steps pay (153 against 158 us forward, 150 against 157 us input gradient at 256 rows per expert)
-        const bool wide_rows = mode != MODE_DW && N >= 2 * K && R >= (int64_t)64 * E && R < (int64_t)512 * E;
+        // and for the row-grouped products from 64 rows per expert on (same box, one after the other, us: gate_proj
+        // forward 135.9 against 138.5, down_proj input gradient 135.3 against 138.8, down_proj forward 146.5 against
+        // 152.2, skewed routing at 65536 rows 264 against 286 forward and 286 against 302 input gradient)
+        const bool wide_rows = mode != MODE_DW && R >= (int64_t)64 * E;
         if ((mode == MODE_DW && R >= (int64_t)64 * E) || wide_rows) {
             rc = gemm_bf16_wide(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, s);
             if (rc != MFL_ERR_UNSUPPORTED) return rc;

@@ -865,10 +865,12 @@ int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, 
         return launch_wide<MODE_DW, 8, 8, 32, 4>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
     }
     if (K % 64 != 0 || K < 64 || R <= 0) return R <= 0 ? MFL_OK : MFL_ERR_UNSUPPORTED;
+    // 320 x 192 tiles (an expert of up to 320 rows is one tile per column slice) up to about 512 rows per expert,
+    // 256 x 256 beyond (fewer bytes per flop)
 #ifdef MFL_TUNING_BUILD
-    const int v = g_wide_variant;
+    const int v = g_wide_variant >= 0 ? g_wide_variant : (R >= (int64_t)512 * E ? 1 : 0);
 #else
-    const int v = 0;
+    const int v = R >= (int64_t)512 * E ? 1 : 0;
 #endif
     if (N % 8 != 0 || N < 8) return MFL_ERR_UNSUPPORTED;
     if (v == 0) {
