@@ -48,7 +48,9 @@ int run_gemm(int mode, const void *a, const void *b, const void *m_sizes, int ms
         // and for the row-grouped products from 64 rows per expert on (same box, one after the other, us: gate_proj
         // forward 135.9 against 138.5, down_proj input gradient 135.3 against 138.8, down_proj forward 146.5 against
         // 152.2, skewed routing at 65536 rows 264 against 286 forward and 286 against 302 input gradient)
-        const bool wide_rows = mode != MODE_DW && R >= (int64_t)64 * E;
+        // (an output of at most 64 columns stays on the eight-wave kernel's thin tiles: 48 against 99 us for the rank-16
+        // product x A^T at 65536 rows)
+        const bool wide_rows = mode != MODE_DW && R >= (int64_t)64 * E && N > 64;
         if ((mode == MODE_DW && R >= (int64_t)64 * E) || wide_rows) {
             rc = gemm_bf16_wide(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, s);
             if (rc != MFL_ERR_UNSUPPORTED) return rc;
