@@ -25,8 +25,8 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch of the benchmarked kernel: not measured by this run but taken from the FETCH_SIZE /
 # WRITE_SIZE counter passes summarised in profiles/gemm_fwd_gate_proj_config2_hbm_traffic.txt
-# (537.2 MB read + 53.5 MB written); the JSON line names that file as the source
-MEASURED_TRAFFIC_BYTES = 590.7e6
+# (537.6 MB read + 57.7 MB written); the JSON line names that file as the source
+MEASURED_TRAFFIC_BYTES = 595.3e6
 TRAFFIC_SOURCE = "profiles/gemm_fwd_gate_proj_config2_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not this run)"
 # A burst of back-to-back launches starts in a transient of the board's power management (boost clocks for
 # the first ten launches, a dip around launch 20, settled after about 150): every timed loop is preceded by
