@@ -45,12 +45,13 @@ int run_gemm(int mode, const void *a, const void *b, const void *m_sizes, int ms
     if (in_dtype == MFL_BF16) {
         // weight gradient from about 64 rows per expert on: the four-wave kernel (85.6 against 99.5 us at 64 rows per
         // expert, 156 against 170 us at 256, N = 2048, K = 768, E = 128; below that the eight-wave tiles are ahead)
-        // and for the row-grouped products from 64 rows per expert on (same box, one after the other, us: gate_proj
+        // and for the row-grouped products from where the flat tiles end (same box, one after the other, us: gate_proj
         // forward 135.9 against 138.5, down_proj input gradient 135.3 against 138.8, down_proj forward 146.5 against
-        // 152.2, skewed routing at 65536 rows 264 against 286 forward and 286 against 302 input gradient)
+        // 152.2, skewed routing at 65536 rows 264 against 286 forward and 286 against 302 input gradient; at 48 to 64
+        // rows per expert forward 95-97 against 97-99, input gradient with N = 2048, K = 768 91-97 against 102-108)
         // (an output of at most 64 columns stays on the eight-wave kernel's thin tiles: 48 against 99 us for the rank-16
         // product x A^T at 65536 rows)
-        const bool wide_rows = mode != MODE_DW && R >= (int64_t)64 * E && N > 64;
+        const bool wide_rows = mode != MODE_DW && R >= (int64_t)kFlatTileRowsPerExpert * E && N > 64;
         if ((mode == MODE_DW && R >= (int64_t)64 * E) || wide_rows) {
             rc = gemm_bf16_wide(mode, a, b, m_sizes, ms_i64, c, R, N, K, E, out_dtype, alpha, accumulate, s);
             if (rc != MFL_ERR_UNSUPPORTED) return rc;
