@@ -247,7 +247,8 @@ __device__ __forceinline__ float acc_read(float v) {
 template <int MODE, int MB, int NB, int BK, int SR, typename TO>
 __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict__ a, const bf16_t *__restrict__ b,
                                                         const void *__restrict__ m_sizes, int ms_i64,
-                                                        TO *__restrict__ c, int64_t R, int N, int K, int E) {
+                                                        TO *__restrict__ c, int64_t R, int N, int K, int E,
+                                                        const bf16_t *__restrict__ a2, const bf16_t *__restrict__ b2) {
     static_assert(sizeof(TO) == 2, "bf16 output");
     constexpr int WGM = 2, WGN = 2, NW = 4;
     constexpr int BM = MB * 32, BN = NB * 32;
@@ -322,6 +323,10 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     if (L_end > total) L_end = total;
 
     // ---- what a cursor knows about a tile; every field wave-uniform
+    // DX with a second term (a2, b2 shaped like a, b): the tile's reduction runs over (a, b) and goes on over
+    // (a2, b2), in one accumulator: dx = a b + a2 b2 (the input gradient of the gated unit, de w_gate + dg w_up)
+    const bool two_term = MODE == MODE_DX && a2 != nullptr;
+    const int64_t second_a = (int64_t)((intptr_t)a2 - (intptr_t)a), second_b = (int64_t)((intptr_t)b2 - (intptr_t)b);
     struct Tile {
         int i0, i_end, j0, red, KT;
         const unsigned char *pa, *pb;
@@ -374,7 +379,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
             if (t.i0 > t.i_end) t.i0 = t.i_end;
             t.j0 = ni * BN;
             t.red = K;
-            t.KT = t.i_end > t.i0 ? K / BK : 0;
+            t.KT = t.i_end > t.i0 ? (two_term ? 2 : 1) * (K / BK) : 0;
             t.pa = (const unsigned char *)(a + (int64_t)t.i0 * K);
             t.pb = B_RC ? (const unsigned char *)(b + (int64_t)expert * N * K + (int64_t)t.j0 * K)
                         : (const unsigned char *)(b + (int64_t)expert * N * K + t.j0);
@@ -523,6 +528,10 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
         if (++pk == pt.KT) {
             pL += per_xcd;
             prod_seek();
+        } else if (MODE == MODE_DX && two_term && pk == K / BK) {
+            // the second term starts at the beginning of its own operands
+            pa_cur = uniform64((uint64_t)((intptr_t)pt.pa + second_a) - kCopyBias);
+            pb_cur = uniform64((uint64_t)((intptr_t)pt.pb + second_b) - kCopyBias);
         }
     };
     auto issue_all = [&]() {  // one whole step, back to back
@@ -829,7 +838,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
 
 template <int MODE, int MB, int NB, int BK, int SR>
 int launch_wide(const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N, int K,
-                int E, hipStream_t stream) {
+                int E, hipStream_t stream, const void *a2 = nullptr, const void *b2 = nullptr) {
     constexpr int STAGE_BYTES = (MB + NB) * 32 * BK * 2;
     constexpr int WTN = NB / 2 * 32;
     constexpr int EPC = WTN % 64 == 0 ? 64 : WTN;
@@ -846,7 +855,8 @@ int launch_wide(const void *a, const void *b, const void *m_sizes, int ms_i64, v
         [&] { return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES); });
     if (e != hipSuccess) return (int)e;
     const int grid = device_info().cu_count / kXcd * kXcd;
-    kern<<<grid, 256, LDS_BYTES, stream>>>((const bf16_t *)a, (const bf16_t *)b, m_sizes, ms_i64, (bf16_t *)c, R, N, K, E);
+    kern<<<grid, 256, LDS_BYTES, stream>>>((const bf16_t *)a, (const bf16_t *)b, m_sizes, ms_i64, (bf16_t *)c, R, N, K, E,
+                                           (const bf16_t *)a2, (const bf16_t *)b2);
     return launch_status();
 }
 
@@ -857,9 +867,12 @@ int g_wide_variant = 0;  // 0: 320 x 192 tiles where N allows, 1: 256 x 256 tile
 #endif
 
 int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
-                   int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream) {
+                   int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream, const void *a2,
+                   const void *b2) {
     if (out_dtype != MFL_BF16 || accumulate || alpha != 1.0f || E > kMaxTableExperts || E < 1) return MFL_ERR_UNSUPPORTED;
     if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, 16)) return MFL_ERR_UNSUPPORTED;
+    if ((a2 != nullptr) != (b2 != nullptr) || (a2 != nullptr && mode != MODE_DX) || !aligned(a2, 16) || !aligned(b2, 16))
+        return MFL_ERR_UNSUPPORTED;
     if (mode == MODE_DW) {
         if (N % 256 != 0 || K % 256 != 0 || N < 256 || K < 256) return MFL_ERR_UNSUPPORTED;
         return launch_wide<MODE_DW, 8, 8, 32, 4>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
@@ -875,10 +888,10 @@ int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, 
     if (N % 8 != 0 || N < 8) return MFL_ERR_UNSUPPORTED;
     if (v == 0) {
         if (mode == MODE_FWD) return launch_wide<MODE_FWD, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
-        return launch_wide<MODE_DX, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
+        return launch_wide<MODE_DX, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream, a2, b2);
     }
     if (mode == MODE_FWD) return launch_wide<MODE_FWD, 8, 8, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
-    return launch_wide<MODE_DX, 8, 8, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
+    return launch_wide<MODE_DX, 8, 8, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream, a2, b2);
 }
 
 }  // namespace mfl
