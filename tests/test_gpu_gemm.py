@@ -301,15 +301,20 @@ def test_dw_four_wave_kernel_matches_oracle(N, K, sizes, ms_dtype):
     assert torch.equal(grouped_gemm_backward_dw(xd, dyd, msd, torch.bfloat16), dw), "same bits from run to run"
 
 
-# the same kernel in the row-grouped products (forward and input gradient with N >= 2 K and 64 to 512 rows per
-# expert on average): tiles of 320 x 192, so N = 200, 520 and 2048 end in a partial column tile; experts of 0, 1,
-# 319, 320, 321 and 700 rows (no tile, one block, a full tile, a tile and one row, several tiles).
+# the same kernel in the row-grouped products (forward and input gradient with more than 64 output columns, from 48
+# rows per expert on average): tiles of 320 x 192 up to 512 rows per expert, so N = 200, 520 and 2048 end in a partial
+# column tile; experts of 0, 1, 319, 320, 321 and 700 rows (no tile, one block, a full tile, a tile and one row,
+# several tiles); a reduction longer than the output is wide; 256 x 256 tiles from 512 rows per expert on (N = 520:
+# two tiles and eight columns).
 WIDE_ROW_CASES = [
     # N, K, m_sizes
     (200, 64, [300, 0, 1, 319, 320, 321, 700, 95]),
     (520, 128, [257] * 5 + [0, 64, 512]),
     (2048, 768, [250 + 7 * (e % 5) for e in range(16)]),
     (384, 192, [100 + e for e in range(70)]),
+    (768, 2048, [48, 60, 0, 130, 50, 49]),
+    (520, 128, [1000, 0, 700]),
+    (768, 256, [513, 2047, 256, 1300]),
 ]
 
 
@@ -317,7 +322,7 @@ WIDE_ROW_CASES = [
 def test_row_grouped_products_on_the_four_wave_kernel_match_oracle(N, K, sizes):
     ms = torch.tensor(sizes, dtype=torch.int32)
     E, R = ms.numel(), int(ms.sum())
-    assert 64 * E <= R < 512 * E and N >= 2 * K
+    assert 48 * E <= R and N > 64 and K % 64 == 0
     x, w, _, _, sel = _case(N + K + E, R, N, K, E, torch.bfloat16, m_sizes=ms)
     xd, wd, msd = x.to(DEV), w.to(DEV), ms.to(DEV)
     print(f"four-wave fwd/dX N={N} K={K} E={E} R={R}", flush=True)
