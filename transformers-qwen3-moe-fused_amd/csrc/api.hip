@@ -255,6 +255,11 @@ int mfl_gemm_fwd_lora(const void *x, const void *w, const void *xt, const void *
     if (R > 0 && (!xt || !wt)) return MFL_ERR_NULL;
     if (R == 0) return MFL_OK;
     if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    if (R >= (int64_t)kFlatTileRowsPerExpert * E && N > 64) {  // the four-wave kernel, as for the product alone
+        rc = gemm_bf16_wide(MODE_FWD, x, w, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E, out_dtype, 1.0f, 0,
+                            (hipStream_t)stream, nullptr, nullptr, xt, wt, KT);
+        if (rc != MFL_ERR_UNSUPPORTED) return rc;
+    }
     GemmFusion fu = {nullptr, 1, 0, nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr};
     fu.xt = xt, fu.wt = wt, fu.kt = KT;
     return gemm_bf16_pipe(MODE_FWD, x, w, m_sizes, m_sizes_dtype == MFL_I64, y, R, N, K, E, out_dtype, 1.0f, 0,
@@ -271,6 +276,11 @@ int mfl_gemm_dx_lora(const void *dy, const void *w, const void *dy2, const void 
     if (R > 0 && (!xt || !wt)) return MFL_ERR_NULL;
     if (R == 0) return MFL_OK;
     if (in_dtype != MFL_BF16) return MFL_ERR_UNSUPPORTED;
+    if (R >= (int64_t)kFlatTileRowsPerExpert * E && N > 64) {
+        rc = gemm_bf16_wide(MODE_DX, dy, w, m_sizes, m_sizes_dtype == MFL_I64, dx, R, N, K, E, out_dtype, 1.0f, 0,
+                            (hipStream_t)stream, dy2, w2, xt, wt, KT);
+        if (rc != MFL_ERR_UNSUPPORTED) return rc;
+    }
     GemmFusion fu = {nullptr, 1, 0, w2, nullptr, nullptr, 0, nullptr, nullptr, dy2};
     fu.xt = xt, fu.wt = wt, fu.kt = KT;
     return gemm_bf16_pipe(MODE_DX, dy, w, m_sizes, m_sizes_dtype == MFL_I64, dx, R, N, K, E, out_dtype, 1.0f, 0,

@@ -69,10 +69,12 @@ int gemm_bf16_pipe(int mode, const void *a, const void *b, const void *m_sizes, 
 
 // Four-wave kernels with 128 x 128 wave tiles (bf16 in and out, no accumulation, whole tiles along the weight
 // dimensions).  Returns MFL_ERR_UNSUPPORTED for the rest.
-// a2, b2 (DX only, shaped like a, b): a second term in the same reduction, c = a b + a2 b2.
+// a2, b2 (DX only, shaped like a, b): a second term in the same reduction, c = a b + a2 b2.  at, bt, kthin (FWD,
+// DX): a last term with a reduction length of its own, as GemmFusion::xt, wt, kt.
 int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
                    int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream,
-                   const void *a2 = nullptr, const void *b2 = nullptr);
+                   const void *a2 = nullptr, const void *b2 = nullptr, const void *at = nullptr,
+                   const void *bt = nullptr, int kthin = 0);
 
 // The weight-gradient product with one thin side (N or K equal to 8, 16, 32 or 64, the other a multiple of 256; bf16 in,
 // bf16 or fp32 out): steps of 32 rows dealt out evenly over the workgroups, experts cut by a border finished by

@@ -244,11 +244,14 @@ __device__ __forceinline__ float acc_read(float v) {
     return r;
 }
 
-template <int MODE, int MB, int NB, int BK, int SR, typename TO>
+template <int MODE, int MB, int NB, int BK, int SR, bool THIN, typename TO>
 __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict__ a, const bf16_t *__restrict__ b,
                                                         const void *__restrict__ m_sizes, int ms_i64,
                                                         TO *__restrict__ c, int64_t R, int N, int K, int E,
-                                                        const bf16_t *__restrict__ a2, const bf16_t *__restrict__ b2) {
+                                                        const bf16_t *__restrict__ a2, const bf16_t *__restrict__ b2,
+                                                        const bf16_t *__restrict__ at, const bf16_t *__restrict__ bt,
+                                                        int kthin) {
+    static_assert(!THIN || MODE != MODE_DW, "the thin last term belongs to the row-grouped products");
     static_assert(sizeof(TO) == 2, "bf16 output");
     constexpr int WGM = 2, WGN = 2, NW = 4;
     constexpr int BM = MB * 32, BN = NB * 32;
@@ -327,8 +330,12 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     // (a2, b2), in one accumulator: dx = a b + a2 b2 (the input gradient of the gated unit, de w_gate + dg w_up)
     const bool two_term = MODE == MODE_DX && a2 != nullptr;
     const int64_t second_a = (int64_t)((intptr_t)a2 - (intptr_t)a), second_b = (int64_t)((intptr_t)b2 - (intptr_t)b);
+    // THIN: a last term with a reduction length of its own (the rank of a LoRA adapter), after the one or two
+    // terms above, in the same accumulator: c += at bt with at (R, kthin) and bt (E, N, kthin) in FWD, (E, kthin, N)
+    // in DX; kthin a multiple of 8.  Its steps come last in the tile's reduction; chunks past kthin are zeros.
+    const int thin_steps = THIN ? ceil_div(kthin, BK) : 0;
     struct Tile {
-        int i0, i_end, j0, red, KT;
+        int i0, i_end, j0, red, KT, expert;
         const unsigned char *pa, *pb;
         TO *pc;
     };
@@ -379,7 +386,8 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
             if (t.i0 > t.i_end) t.i0 = t.i_end;
             t.j0 = ni * BN;
             t.red = K;
-            t.KT = t.i_end > t.i0 ? (two_term ? 2 : 1) * (K / BK) : 0;
+            t.KT = t.i_end > t.i0 ? (two_term ? 2 : 1) * (K / BK) + thin_steps : 0;
+            t.expert = expert;
             t.pa = (const unsigned char *)(a + (int64_t)t.i0 * K);
             t.pb = B_RC ? (const unsigned char *)(b + (int64_t)expert * N * K + (int64_t)t.j0 * K)
                         : (const unsigned char *)(b + (int64_t)expert * N * K + t.j0);
@@ -447,7 +455,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
             pL += per_xcd;
         }
         pk = 0;
-        p_full = MODE == MODE_DW ? pt.red / BK : pt.KT;
+        p_full = MODE == MODE_DW ? pt.red / BK : pt.KT - thin_steps;
         pa_cur = uniform64((uint64_t)(uintptr_t)pt.pa - kCopyBias);
         pb_cur = uniform64((uint64_t)(uintptr_t)pt.pb - kCopyBias);
     };
@@ -519,8 +527,54 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
             wide_copy<0>(p, st + SA::kBytes + (wave * LB + q) * 1024);
         }
     };
-    auto prod_advance = [&]() {  // after the last copy of a step
-        issued += p_copies;
+    // a step of the thin last term: per-lane addresses from that term's own leading dimensions, all copies at once
+    auto copy_thin = [&](uint32_t slot_off) {
+        if constexpr (THIN) {
+            const uint32_t st = ring_lds + slot_off;
+            const int ks = pk - p_full;
+            const int i_lim = pt.i_end - pt.i0 < BM ? pt.i_end - pt.i0 : BM;
+            const int j_lim = N - pt.j0 < BN ? N - pt.j0 : BN;
+            const unsigned char *at_tile = (const unsigned char *)(at + (int64_t)pt.i0 * kthin);
+            const unsigned char *bt_tile =
+                (const unsigned char *)(bt + (B_RC ? ((int64_t)pt.expert * N + pt.j0) * kthin
+                                                   : (int64_t)pt.expert * N * kthin + pt.j0));
+            // the lane number behind a barrier for the optimiser: what follows is worked out here, once or twice per
+            // tile, and not kept in registers across the tile's other steps
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+#pragma unroll
+            for (int q = 0; q < LA; ++q) {
+                const int load = wave * LA + q;
+                int i = SA::row_of(load, ln);
+                const int r = ks * BK + SA::swz(i, SA::phys_of(load, ln)) * 8;
+                if (i >= i_lim) i = i_lim - 1;
+                const unsigned char *p = r >= kthin ? (const unsigned char *)&g_zero_chunk : at_tile + ((int64_t)i * kthin + r) * 2;
+                wide_copy<0>(p, st + load * 1024);
+            }
+#pragma unroll
+            for (int q = 0; q < LB; ++q) {
+                const int load = wave * LB + q;
+                const int row = SB::row_of(load, ln);
+                const int c = SB::swz(row, SB::phys_of(load, ln));
+                const unsigned char *p;
+                if (B_RC) {
+                    const int j = row < j_lim ? row : j_lim - 1;
+                    const int r = ks * BK + c * 8;
+                    p = r >= kthin ? (const unsigned char *)&g_zero_chunk : bt_tile + ((int64_t)j * kthin + r) * 2;
+                } else {
+                    // rows past the end of the term re-read its last row: they meet zeros of the left operand
+                    int r = ks * BK + row;
+                    if (r >= kthin) r = kthin - 1;
+                    int j = c * 8;
+                    if (j >= j_lim) j = j_lim - 8;
+                    p = bt_tile + ((int64_t)r * N + j) * 2;
+                }
+                wide_copy<0>(p, st + SA::kBytes + load * 1024);
+            }
+        }
+    };
+    auto prod_advance = [&](bool all_copies = false) {  // after the last copy of a step
+        issued += all_copies ? LPW : p_copies;
         mark[pg % SR] = issued;
         ++pg;
         pa_cur += step_a;
@@ -537,10 +591,14 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     auto issue_all = [&]() {  // one whole step, back to back
         const uint32_t slot_off = (pg % SR) * STAGE_BYTES;
         bool tail = false;
-        if constexpr (MODE == MODE_DW) tail = pk >= p_full;
-        if (tail) copy_tail(slot_off);
-        else static_for<NG>([&](auto j_tag) { copy_group(j_tag, slot_off, 1); });
-        prod_advance();
+        if constexpr (MODE == MODE_DW || THIN) tail = pk >= p_full;
+        if (tail) {
+            if constexpr (MODE == MODE_DW) copy_tail(slot_off);
+            else copy_thin(slot_off);
+        } else {
+            static_for<NG>([&](auto j_tag) { copy_group(j_tag, slot_off, 1); });
+        }
+        prod_advance(tail);
     };
 
     // ---- consumer
@@ -696,10 +754,11 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
             const uint32_t slot_off = (pg % SR) * STAGE_BYTES;
             if (p_more) {
                 bool tail = false;
-                if constexpr (MODE == MODE_DW) tail = pk >= p_full;
+                if constexpr (MODE == MODE_DW || THIN) tail = pk >= p_full;
                 if (tail) {
-                    copy_tail(slot_off);
-                    prod_advance();
+                    if constexpr (MODE == MODE_DW) copy_tail(slot_off);
+                    else copy_thin(slot_off);
+                    prod_advance(true);
                 } else {
                     spread = 1;
                 }
@@ -836,9 +895,10 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
 #endif
 }
 
-template <int MODE, int MB, int NB, int BK, int SR>
+template <int MODE, int MB, int NB, int BK, int SR, bool THIN = false>
 int launch_wide(const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N, int K,
-                int E, hipStream_t stream, const void *a2 = nullptr, const void *b2 = nullptr) {
+                int E, hipStream_t stream, const void *a2 = nullptr, const void *b2 = nullptr, const void *at = nullptr,
+                const void *bt = nullptr, int kthin = 0) {
     constexpr int STAGE_BYTES = (MB + NB) * 32 * BK * 2;
     constexpr int WTN = NB / 2 * 32;
     constexpr int EPC = WTN % 64 == 0 ? 64 : WTN;
@@ -849,14 +909,14 @@ int launch_wide(const void *a, const void *b, const void *m_sizes, int ms_i64, v
     constexpr int LDS_BYTES = SR * STAGE_BYTES + 4 * 32 * EP_ROWB + 2 * (kMaxTableExperts + 1) * 4;
 #endif
     static_assert(LDS_BYTES <= 160 * 1024, "LDS capacity of a CDNA4 compute unit");
-    auto kern = gemm_wide_kernel<MODE, MB, NB, BK, SR, bf16_t>;
+    auto kern = gemm_wide_kernel<MODE, MB, NB, BK, SR, THIN, bf16_t>;
     static PerDeviceOnce attr;
     const hipError_t e = attr.run(
         [&] { return hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES); });
     if (e != hipSuccess) return (int)e;
     const int grid = device_info().cu_count / kXcd * kXcd;
     kern<<<grid, 256, LDS_BYTES, stream>>>((const bf16_t *)a, (const bf16_t *)b, m_sizes, ms_i64, (bf16_t *)c, R, N, K, E,
-                                           (const bf16_t *)a2, (const bf16_t *)b2);
+                                           (const bf16_t *)a2, (const bf16_t *)b2, (const bf16_t *)at, (const bf16_t *)bt, kthin);
     return launch_status();
 }
 
@@ -868,7 +928,7 @@ int g_wide_variant = 0;  // 0: 320 x 192 tiles where N allows, 1: 256 x 256 tile
 
 int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,
                    int K, int E, int out_dtype, float alpha, int accumulate, hipStream_t stream, const void *a2,
-                   const void *b2) {
+                   const void *b2, const void *at, const void *bt, int kthin) {
     if (out_dtype != MFL_BF16 || accumulate || alpha != 1.0f || E > kMaxTableExperts || E < 1) return MFL_ERR_UNSUPPORTED;
     if (!aligned(a, 16) || !aligned(b, 16) || !aligned(c, 16)) return MFL_ERR_UNSUPPORTED;
     if ((a2 != nullptr) != (b2 != nullptr) || (a2 != nullptr && mode != MODE_DX) || !aligned(a2, 16) || !aligned(b2, 16))
@@ -886,6 +946,20 @@ int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, 
     const int v = R >= (int64_t)512 * E ? 1 : 0;
 #endif
     if (N % 8 != 0 || N < 8) return MFL_ERR_UNSUPPORTED;
+    if (at != nullptr) {
+        // the thin last term: kernels of their own (its test in every step would cost the plain products)
+        if (bt == nullptr || kthin < 8 || kthin % 8 != 0 || !aligned(at, 16) || !aligned(bt, 16)) return MFL_ERR_UNSUPPORTED;
+        if (v == 0) {
+            if (mode == MODE_FWD)
+                return launch_wide<MODE_FWD, 10, 6, 64, 2, true>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream, nullptr,
+                                                                 nullptr, at, bt, kthin);
+            return launch_wide<MODE_DX, 10, 6, 64, 2, true>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream, a2, b2, at, bt, kthin);
+        }
+        if (mode == MODE_FWD)
+            return launch_wide<MODE_FWD, 8, 8, 64, 2, true>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream, nullptr, nullptr,
+                                                            at, bt, kthin);
+        return launch_wide<MODE_DX, 8, 8, 64, 2, true>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream, a2, b2, at, bt, kthin);
+    }
     if (v == 0) {
         if (mode == MODE_FWD) return launch_wide<MODE_FWD, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
         return launch_wide<MODE_DX, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream, a2, b2);
