@@ -40,9 +40,12 @@ namespace {
 #ifndef MFL_X_NO_MFMA
 #define MFL_X_NO_MFMA 0
 #endif
-constexpr bool kNoStore = MFL_X_NO_STORE, kNoCopy = MFL_X_NO_COPY, kNoMfma = MFL_X_NO_MFMA;
+#ifndef MFL_X_NO_READ
+#define MFL_X_NO_READ 0
+#endif
+constexpr bool kNoStore = MFL_X_NO_STORE, kNoCopy = MFL_X_NO_COPY, kNoMfma = MFL_X_NO_MFMA, kNoRead = MFL_X_NO_READ;
 #else
-constexpr bool kNoStore = false, kNoCopy = false, kNoMfma = false;
+constexpr bool kNoStore = false, kNoCopy = false, kNoMfma = false, kNoRead = false;
 #endif
 
 #if defined(MFL_TUNING_BUILD) && defined(MFL_X_TRACE)
@@ -402,11 +405,14 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
 
     // ---- producer: the (tile, step) whose copies are issued next.  A step's copies go out in groups of up to
     // four (one statement, one M0 write, scalar base + per-lane 32-bit offset + the instruction's offset field).
+    constexpr int GS = 4;  // copies per group (groups of two and of one were measured: no faster)
     static_assert(LA % 2 == 0 && LB % 2 == 0, "copy groups hold two or four copies");
-    constexpr int GA = (LA + 3) / 4, GB = (LB + 3) / 4, NG = GA + GB;  // groups per step: A's first, then B's
-    // With three stages or more a step's copies have two steps to land: the second half of the groups goes out in
-    // the first sub-step of the consumer's next step, so that no sub-step carries more than half of them.
-    constexpr bool SPLIT = SR >= 3 && NG >= 2;
+    constexpr int GA = (LA + GS - 1) / GS, GB = (LB + GS - 1) / GS, NG = GA + GB;  // groups per step: A's first, then B's
+    // The second half of a step's groups goes out in the first sub-step of the consumer's next step, so that no
+    // sub-step carries more than half of them (with two stages they then have three sub-steps to land instead of
+    // four; measured 4 % faster at 1024 rows per expert, where a sub-step's MFMAs do not cover the issue of a whole
+    // step's copies, and no slower at 256).
+    constexpr bool SPLIT = NG >= 2;
     constexpr int NG1 = SPLIT ? (NG + 1) / 2 : NG;  // groups in the sub-step after point P
     Tile pt;
     int pL = L_first, pk = 0, p_full = 0;  // p_full: steps of the producer's tile that are whole
@@ -422,7 +428,7 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     auto prep_voff = [&](int q0, int q1) {
 #pragma unroll
         for (int q = 0; q < LPW; ++q)
-            if (q >= q0 && q < q1) voff[q] = lane_off[q] + kCopyBias - ((q < LA ? q : q - LA) % 4) * 1024;
+            if (q >= q0 && q < q1) voff[q] = lane_off[q] + kCopyBias - ((q < LA ? q : q - LA) % GS) * 1024;
     };
     auto prod_offsets = [&]() {  // row-grouped products: rows past the tile's last and columns past N are clamped
         const int i_lim = pt.i_end - pt.i0 < BM ? pt.i_end - pt.i0 : BM;
@@ -436,10 +442,10 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
         p_amask = 0, p_copies = LB;
 #pragma unroll
         for (int j = 0; j < GA; ++j) {
-            const int first_row = SA::row_of(wave * LA + 4 * j, 0);
+            const int first_row = SA::row_of(wave * LA + GS * j, 0);
             if (first_row < i_lim) {
                 p_amask |= 1u << j;
-                p_copies += LA - 4 * j >= 4 ? 4 : 2;
+                p_copies += LA - GS * j >= GS ? GS : LA - GS * j;
             }
         }
     };
@@ -482,6 +488,9 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
 #if defined(MFL_TUNING_BUILD) && defined(MFL_X_DW_POLICY)
     constexpr int A_POLICY = MODE == MODE_DW ? (MFL_X_DW_POLICY & 1) * 2 : 0;
     constexpr int B_POLICY = MODE == MODE_DW ? (MFL_X_DW_POLICY >> 1) * 2 : 2;
+#elif defined(MFL_TUNING_BUILD) && defined(MFL_X_AB_POLICY)
+    constexpr int A_POLICY = MODE == MODE_DW ? 0 : (MFL_X_AB_POLICY & 1) * 2;
+    constexpr int B_POLICY = MODE == MODE_DW ? 0 : (MFL_X_AB_POLICY >> 1) * 2;
 #else
     constexpr int A_POLICY = 0;
     constexpr int B_POLICY = MODE == MODE_DW ? 0 : 2;
@@ -491,14 +500,14 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     auto copy_group = [&](auto j_tag, uint32_t slot_off, int on) {
         constexpr int j = decltype(j_tag)::value;
         if constexpr (j < GA) {
-            constexpr int q = 4 * j, n = LA - q >= 4 ? 4 : 2;
+            constexpr int q = GS * j, n = LA - q >= GS ? GS : LA - q;
             const uint32_t lds = __builtin_amdgcn_readfirstlane(wave_a_lds + slot_off + q * 1024);
             const uint64_t base = uniform64(pa_cur);
             if constexpr (A_RC) on = on & (int)((p_amask >> j) & 1u);
             if constexpr (n == 4) wide_copy4<A_POLICY>(base, voff[q], voff[q + 1], voff[q + 2], voff[q + 3], lds, on);
             else wide_copy2<A_POLICY>(base, voff[q], voff[q + 1], lds, on);
         } else {
-            constexpr int qb = 4 * (j - GA), q = LA + qb, n = LB - qb >= 4 ? 4 : 2;
+            constexpr int qb = GS * (j - GA), q = LA + qb, n = LB - qb >= GS ? GS : LB - qb;
             const uint32_t lds = __builtin_amdgcn_readfirstlane(wave_b_lds + slot_off + qb * 1024);
             const uint64_t base = uniform64(pb_cur);
             if constexpr (n == 4) wide_copy4<B_POLICY>(base, voff[q], voff[q + 1], voff[q + 2], voff[q + 3], lds, on);
@@ -694,6 +703,10 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
         constexpr int NM = TA * TN, NU = TM + TN;
         auto read_unit = [&](auto u_tag, int rks, int buf) {
             constexpr int U = decltype(u_tag)::value;
+            if constexpr (kNoRead) {
+                asm volatile("" : "+v"(fb[buf][0]));
+                return;
+            }
             if constexpr (U < TN)
                 fb[buf][U] = fo_b.load(smem, U, rks);
             else
@@ -960,6 +973,15 @@ int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, 
                                                             at, bt, kthin);
         return launch_wide<MODE_DX, 8, 8, 64, 2, true>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream, a2, b2, at, bt, kthin);
     }
+#ifdef MFL_TUNING_BUILD
+    // 256 x 256 tiles with four stages of 32 reduction indices (96 KiB in flight instead of 64; rows of 64 bytes in
+    // the stages of the operands that are contiguous along the reduction): measured 9 % slower in the forward
+    // product at 1024 rows per expert (twice the barriers, half-line requests), 3 % faster in dX
+    if (v == 2) {
+        if (mode == MODE_FWD) return launch_wide<MODE_FWD, 8, 8, 32, 4>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
+        return launch_wide<MODE_DX, 8, 8, 32, 4>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream, a2, b2);
+    }
+#endif
     if (v == 0) {
         if (mode == MODE_FWD) return launch_wide<MODE_FWD, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream);
         return launch_wide<MODE_DX, 10, 6, 64, 2>(a, b, m_sizes, ms_i64, c, R, N, K, E, stream, a2, b2);

@@ -64,7 +64,8 @@ struct Stage {
     // bytes = all 64 banks).  Other row lengths (384 bytes) already differ by 128 bytes from row to
     // row, and a 32-byte spread keeps the XOR inside the row.
     static constexpr int kRsShift = kChunksPerRow % 16 == 0 ? 2 : 1;
-    static_assert(kBytes % 1024 == 0 && kChunksPerRow % 8 == 0, "stage must be whole copies, rows whole 128 B");
+    static_assert(kBytes % 1024 == 0 && kChunksPerRow % (RC ? 4 : 8) == 0,
+                  "stage must be whole copies; rows of 64 bytes or more along the reduction, of whole 128 B across it");
 
     // stage row and physical chunk that lane `lane` of wave-load `load` fills (a copy covers 64
     // consecutive chunks of the stage, whatever the row length)
