@@ -408,11 +408,13 @@ __global__ __launch_bounds__(256) void gemm_wide_kernel(const bf16_t *__restrict
     constexpr int GS = 4;  // copies per group (groups of two and of one were measured: no faster)
     static_assert(LA % 2 == 0 && LB % 2 == 0, "copy groups hold two or four copies");
     constexpr int GA = (LA + GS - 1) / GS, GB = (LB + GS - 1) / GS, NG = GA + GB;  // groups per step: A's first, then B's
-    // The second half of a step's groups goes out in the first sub-step of the consumer's next step, so that no
-    // sub-step carries more than half of them (with two stages they then have three sub-steps to land instead of
-    // four; measured 4 % faster at 1024 rows per expert, where a sub-step's MFMAs do not cover the issue of a whole
-    // step's copies, and no slower at 256).
-    constexpr bool SPLIT = NG >= 2;
+    // With three stages or more a step's copies have two steps to land: the second half of the groups goes out in
+    // the first sub-step of the consumer's next step, so that no sub-step carries more than half of them.  With two
+    // stages the second half then has three sub-steps to land instead of four: the 256 x 256 tiles, which run where
+    // experts have many rows and the MFMAs of one sub-step do not cover the issue of a whole step's copies, do it
+    // (4 % faster at 1024 rows per expert); the 320 x 192 tiles do not (the same at 256 rows per expert, 4-7 %
+    // slower at 48-128, where the weights, whose groups come second, are most of the traffic).
+    constexpr bool SPLIT = NG >= 2 && (SR >= 3 || MB * NB >= 64);
     constexpr int NG1 = SPLIT ? (NG + 1) / 2 : NG;  // groups in the sub-step after point P
     Tile pt;
     int pL = L_first, pk = 0, p_full = 0;  // p_full: steps of the producer's tile that are whole
