@@ -205,6 +205,11 @@ def _kernel_tour(n, dev):
         legs.append((f"gemm_fwd_nf4 gate_proj {tokens} tokens ({active} experts hit)",
                      active * nf4_b / E + 2.0 * tokens * TOPK * (HIDDEN + INTER), 2.0 * tokens * TOPK * INTER * HIDDEN,
                      lambda i, x5=x5, ms5=ms5: grouped_gemm_forward_4bit(x5, *qsets[i % 3], ms5)))
+        if tokens == 16384:
+            legs.append(("gemm_fwd gate_proj 16384 tokens (131072 rows, 256 x 256 tiles)",
+                         2.0 * (tokens * TOPK * (HIDDEN + INTER) + E * INTER * HIDDEN),
+                         2.0 * tokens * TOPK * INTER * HIDDEN,
+                         lambda i, x5=x5, ms5=ms5: grouped_gemm_forward(x5, w_gate, ms5)))
         if tokens <= 256:
             legs.append((f"glu_fwd_nf4 (gate + up + SiLU-mul) {tokens} tokens ({active} experts hit)",
                          2 * active * nf4_b / E + 2.0 * tokens * TOPK * (HIDDEN + INTER),
@@ -438,6 +443,12 @@ def main() -> int:
             us_f = _event_us(lambda i: grouped_gemm_forward_4bit(x5, *qsets[i % NB], ms5), n_it, n_wm, stream)
             us_u = _event_us(lambda i: grouped_gemm_forward(x5, dequantize_nf4(*qsets[i % NB], torch.bfloat16), ms5),
                              n_it, n_wm, stream)
+            if tokens > 1000:
+                # the bf16 product alone at this size (131072 rows, about 1024 to an expert: 256 x 256 tiles)
+                us_b = _event_us(lambda i: grouped_gemm_forward(x5, ws[i % NB], ms5), 60, 60, stream)
+                fl = 2.0 * tokens * TOPK * INTER * HIDDEN
+                extra["fwd_gate_proj_131072_rows"] = {"us": round(us_b, 1), "tflops": round(fl / us_b / 1e6, 1),
+                                                      "mfma_frac": round(fl / us_b / 1e6 / PEAK_BF16_TFLOPS, 4)}
             active = int((ms5 > 0).sum().item())                       # host read outside any timed loop
             packed_bytes = active * INTER * HIDDEN * (0.5 + 4.0 / 64)
             nf4[f"tokens_{tokens}"] = {"fused_us": round(us_f, 1), "dequant_then_gemm_us": round(us_u, 1),
