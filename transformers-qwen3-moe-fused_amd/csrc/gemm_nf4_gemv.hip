@@ -127,8 +127,8 @@ __global__ __launch_bounds__(kGemvThreads) void nf4_gemv_kernel(const bf16_t *__
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    // the lookups address the table from LDS address 0 (the kernel has no static LDS in front of the dynamic)
-    if ((uint32_t)(uintptr_t)(lds_void_ptr)smem != 0) __builtin_trap();
+    // the lookups address the table from LDS address 0: the kernel has no static LDS in front of the dynamic
+    // (the launcher asks the runtime and does not launch a build that has)
     // the counts, asked for first: their latency runs under the filling of the table
     int ms_own[2];
 #pragma unroll
@@ -401,10 +401,18 @@ int launch_gemv(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4M
     const int lds = kGemvTable + (int)max_groups * 8 + 16 + E * 4;
     auto *kernel = nf4_gemv_kernel<NL, ROWS, D, GLU, EXACT, HALF, TO>;
     static PerDeviceOnce attr;
+    // The table lookups take the dynamic LDS to start at address 0; static LDS in this kernel would move it, so
+    // such a build is left to the kernels that decode in registers.
+    static std::atomic<int> static_lds{-1};
     const hipError_t e = attr.run([&] {
+        hipFuncAttributes fa;
+        const hipError_t e1 = hipFuncGetAttributes(&fa, (const void *)kernel);
+        if (e1 != hipSuccess) return e1;
+        static_lds.store((int)fa.sharedSizeBytes, std::memory_order_release);
         return hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kGemvTable + 4096 * 8 + 16 + 2048 * 4);
     });
     if (e != hipSuccess) return (int)e;
+    if (static_lds.load(std::memory_order_acquire) != 0) return MFL_ERR_UNSUPPORTED;
     kernel<<<(unsigned)device_info().cu_count, kGemvThreads, lds, stream>>>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64,
                                                                             y, e_out, g_out, R, N, K, E,
                                                                             N / ((GLU && !HALF) ? 16 : 32), (int)max_groups);
