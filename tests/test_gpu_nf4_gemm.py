@@ -119,6 +119,38 @@ def test_streaming_decode_kernel_edges(m_sizes, N, K, blocksize, ms_dtype, out_d
     assert torch.equal(y2[:R - 3], y[:R - 3])
 
 
+# The same kernel with 64-row tiles, which the plain product takes from 36 up to 100 rows per expert on average:
+# experts that end inside the first or the second 32-row block of a tile, experts of two and three tiles, empty
+# experts, a last column tile that is partly empty, fp32 output, rows past sum(m_sizes); with and without the
+# tile-ordered scales (the same bits).
+@pytest.mark.parametrize("m_sizes,N,K,blocksize,ms_dtype,out_dtype", [
+    ([65, 0, 40, 128, 33, 1, 64, 97], 200, 256, 128, torch.int32, torch.bfloat16),
+    ([70, 70, 0, 150, 31], 136, 384, 64, torch.int64, torch.float32),
+    ([100] * 3 + [0] + [96] * 2, 768, 2048, 64, torch.int32, torch.bfloat16),
+])
+def test_streaming_kernel_64_row_tiles(m_sizes, N, K, blocksize, ms_dtype, out_dtype):
+    E = len(m_sizes)
+    ms = torch.tensor(m_sizes, dtype=ms_dtype)
+    R = int(ms.sum()) + 3
+    assert 36 * E < R <= 100 * E and K % 128 == 0 and blocksize >= 64
+    packed, state, w_deq = _quantised(E, N, K, blocksize, N + K + 1)
+    x = randn((R, K), gen(K + 1), 1.0, torch.bfloat16)
+    sel = oracle.sel_from_m_sizes(np.asarray(m_sizes))
+    y = torch.full((R, N), 7.0, device=DEV, dtype=out_dtype)
+    from qwen3_moe_fused import _lib
+    xd, msd = x.to(DEV), ms.to(DEV)
+    rc = _lib.lib().mfl_gemm_fwd_nf4(_lib.ptr(xd), _lib.ptr(packed), _lib.ptr(state.code), _lib.ptr(state.absmax), blocksize,
+                                     _lib.ptr(msd), _lib.itype_code(ms_dtype), _lib.ptr(y), R, N, K, E,
+                                     _lib.dtype_code(torch.bfloat16), _lib.dtype_code(out_dtype), _lib.stream())
+    _lib.check(rc, "mfl_gemm_fwd_nf4")
+    ref = oracle.linear_fwd(to_np32(x)[:R - 3], w_deq, sel)
+    check_close(y[:R - 3], ref, what=f"streaming kernel, 64-row tiles, m_sizes={m_sizes} N={N} K={K}")
+    assert torch.all(y[R - 3:] == 7.0), "rows past sum(m_sizes) stay as they were"
+    # through the wrapper (which brings the tile-ordered scales): the same bits
+    y2 = grouped_gemm_forward_4bit(xd, packed, state, msd, out_dtype)
+    assert torch.equal(y2[:R - 3], y[:R - 3])
+
+
 def _tile_ordered(absmax, E, N, K, blocksize):
     """The scales in the order the streaming kernel's waves consume them: [expert][32-column tile][128-wide
     stage][column of the tile][half of the stage], columns past N repeating the last one."""

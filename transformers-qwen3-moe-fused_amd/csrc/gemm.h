@@ -21,6 +21,13 @@ constexpr int kNf4DecodeRowsPerExpert = MFL_X_NF4_ROWS;
 #else
 constexpr int kNf4DecodeRowsPerExpert = 72;
 #endif
+// The plain packed-weight forward stays on the streaming kernel up to this many rows per expert: from
+// kNf4StreamTwoBlockRows rows per expert on its workgroups take 64 rows of an expert (the weights are streamed and
+// decoded once per row tile).  Same shape and routing: 32- / 64-row tiles / pipelined kernel 59 / 55 / - us at
+// 40 rows per expert, 66 / 57 / - at 48, 75 / 74 / - at 64, 95-103 / 88 / 95-103 at 80, 110 / 92 / 96-98 at 96,
+// 138 / 117 / 104 at 128; 50 / 52 at 32.
+constexpr int kNf4StreamRowsPerExpert = 100;
+constexpr int kNf4StreamTwoBlockRows = 36;
 
 // Any shape / any float type; plain FMA.
 int gemm_generic(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,

@@ -5,9 +5,10 @@
 // or scales issued after a copy would, when waited for, hold the wave until the copy has landed too, and the
 // copies would never be further ahead than those loads.
 //
-// A workgroup (4 waves) owns 32 rows of one expert and 128 output columns, a wave 32 of the columns (of both
-// matrices in the gated linear unit).
-//   stage = rows     32 x 128 bf16 (8 KiB, shared by the four waves; chunk c of row r at c ^ (r & 15))
+// A workgroup (4 waves) owns 32 MR rows of one expert (MR = 1, or 2 where experts hold some forty rows and more:
+// the weights are streamed and decoded once per row tile) and 128 output columns, a wave 32 of the columns (of
+// both matrices in the gated linear unit) for all of the rows.
+//   stage = rows     32 MR x 128 bf16 (8 KiB a block of 32, shared by the four waves; chunk c of row r at c ^ (r & 15))
 //         + weights  per wave and matrix 32 columns x 64 packed bytes (2 KiB; chunk c of row r at c ^ ((r >> 2) & 3))
 //         + scales   per wave and matrix 32 columns x 2 floats (one per 64 reduction elements)
 //   One barrier per stage: it publishes the rows that the other waves copied and frees the slot of the
@@ -72,20 +73,31 @@ __device__ __forceinline__ uint32_t byte_times_4(uint32_t w) {
     return r;
 }
 
-template <bool GLU>
+template <bool GLU, int MR>
 struct StreamShape {
     static constexpr int CB = GLU ? 2 : 1;     // weight matrices per wave
     static constexpr int RING = 3;             // stages in LDS; two of them in flight
-    static constexpr int kX = 32 * 256;        // rows of a stage
+    static constexpr int kX = MR * 32 * 256;   // rows of a stage: MR blocks of 32
     static constexpr int kW = 32 * 64;         // packed weights of a stage, per wave and matrix
     static constexpr int kA = 32 * 2 * 4;      // scales of a stage, per wave and matrix
     static constexpr int kStage = kX + 4 * CB * (kW + kA);
     static constexpr int kTable = CB * 256 * 4;
-    static constexpr int kLds = RING * kStage + kTable;  // 53248: three workgroups per CU; gated: 81920, two
-    static constexpr int kOps = 2 * CB + 2 + CB;  // copies per wave and stage
+    static constexpr int kLds = RING * kStage + kTable;  // MR = 1: 53248, three workgroups per CU; gated: 81920, two
+    static constexpr int kWOps = 2 * CB + CB;  // copies of weights and scales per wave and stage (the rows: up to 2 MR more)
 };
 
-template <bool GLU, bool TILED, typename TO>
+// at most OPS + xc (xc = 0 .. XMAX, wave-uniform) vector-memory operations outstanding
+template <int OPS, int XMAX>
+__device__ __forceinline__ void wait_stage_ops(int xc) {
+    if constexpr (XMAX == 0) {
+        wait_vmcnt<OPS>();
+    } else {
+        if (xc == XMAX) wait_vmcnt<OPS + XMAX>();
+        else wait_stage_ops<OPS, XMAX - 1>(xc);
+    }
+}
+
+template <bool GLU, bool TILED, int MR, typename TO>
 __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restrict__ x,
                                                          const int32_t *__restrict__ row_idx, int idx_div,
                                                          Nf4Matrix w0, Nf4Matrix w1,
@@ -93,8 +105,8 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
                                                          TO *__restrict__ y, TO *__restrict__ e_out,
                                                          TO *__restrict__ g_out, int64_t R, int N, int K, int E,
                                                          int tiles_n) {
-    using S = StreamShape<GLU>;
-    constexpr int CB = S::CB, RING = S::RING;
+    using S = StreamShape<GLU, MR>;
+    constexpr int CB = S::CB, RING = S::RING, TR = 32 * MR;  // TR: rows of a workgroup's tile
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     // the pair table first, at LDS address 0 (the kernel has no static LDS, which the launcher checks): a lookup's address is then the shifted
     // byte itself plus a constant that fits the instruction's offset field, no add
@@ -133,7 +145,7 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
         for (int e0 = 0; e0 < E; e0 += 64) {
             const int e = e0 + lane;
             const int m = e < E ? load_msize(m_sizes, ms_i64, e) : 0;
-            const int t = ceil_div(m, 32);
+            const int t = ceil_div(m, TR);
             const int minc = wave_inclusive_scan(m), tinc = wave_inclusive_scan(t);
             const int tb = tile_carry + tinc - t;
             const uint64_t hits = __ballot(rt >= tb && rt < tb + t);
@@ -152,10 +164,10 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     // every wave of the workgroup takes the same path here: the values above are the same in all of them
     if (expert < 0) return;
     expert = __builtin_amdgcn_readfirstlane(expert);
-    const int i0 = __builtin_amdgcn_readfirstlane(m_start) + (rt - __builtin_amdgcn_readfirstlane(t_begin)) * 32;
+    const int i0 = __builtin_amdgcn_readfirstlane(m_start) + (rt - __builtin_amdgcn_readfirstlane(t_begin)) * TR;
     int i_end = __builtin_amdgcn_readfirstlane(m_start) + __builtin_amdgcn_readfirstlane(m_size);
     if ((int64_t)i_end > R) i_end = (int)R;
-    const int rows = i_end - i0 < 32 ? i_end - i0 : 32;
+    const int rows = i_end - i0 < TR ? i_end - i0 : TR;
     if (rows <= 0) return;
 
     // ---- sources of this lane's pieces of a stage
@@ -177,10 +189,10 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
         if (col >= N) col = N - 1;
         a_el[cb] = ((int64_t)expert * N + col) * K + (lane & 1) * 64;
     }
-    const bf16_t *x_src[2];  // copy j: rows 8 wave + 4j .. + 3, sixteen lanes to a row
+    const bf16_t *x_src[2 * MR];  // copy j: rows 32 (j / 2) + 8 wave + 4 (j % 2) .. + 3, sixteen lanes to a row
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int r = 8 * wave + 4 * j + (lane >> 4);
+    for (int j = 0; j < 2 * MR; ++j) {
+        const int r = 32 * (j >> 1) + 8 * wave + 4 * (j & 1) + (lane >> 4);
         const int c = (lane & 15) ^ (r & 15);
         int64_t src_row = i0 + (r < rows ? r : rows - 1);
         if (row_idx != nullptr) src_row = (uint32_t)row_idx[src_row] / (uint32_t)idx_div;
@@ -188,13 +200,18 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     }
     const int NS = K / 128, tiles32 = (N + 31) / 32;
     // A copy of rows whose four rows all lie past the tile's last row is left out (nobody stores what the MFMAs
-    // make of that part of the stage): x_copies of the wave's two, the same number in every stage.
-    const int x_copies = rows > 8 * wave + 4 ? 2 : rows > 8 * wave ? 1 : 0;
+    // make of that part of the stage): the first x_copies of the wave's 2 MR (their rows ascend with j), the same
+    // number in every stage.
+    int x_copies = 0;
+#pragma unroll
+    for (int j = 0; j < 2 * MR; ++j) x_copies += rows > 32 * (j >> 1) + 8 * wave + 4 * (j & 1) ? 1 : 0;
+    x_copies = __builtin_amdgcn_readfirstlane(x_copies);
+    const int m_blocks = ceil_div(rows, 32);  // 32-row blocks of the tile that hold rows
     auto issue = [&](int stg) {
         unsigned char *const base = ring + (stg % RING) * S::kStage;
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-            if (j < x_copies) copy16_to_lds(x_src[j] + (int64_t)stg * 128, base + (wave * 2 + j) * 1024);
+        for (int j = 0; j < 2 * MR; ++j)
+            if (j < x_copies) copy16_to_lds(x_src[j] + (int64_t)stg * 128, base + ((j >> 1) * 8 + wave * 2 + (j & 1)) * 1024);
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
 #pragma unroll
@@ -217,22 +234,23 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
         for (int ks = 0; ks < 4; ++ks) x_rd[s2][ks] = n * 256 + (((8 * s2 + 4 * h + ks) ^ (n & 15)) << 4);
     }
 
-    floatx16 tot[CB];
+    floatx16 tot[MR][CB];
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb)
+    for (int m = 0; m < MR; ++m)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) tot[cb][r] = 0.f;
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tot[m][cb][r] = 0.f;
 
-    // Every wave issues the same number of copies per stage (S::kOps less the row copies it leaves out),
+    // Every wave issues the same number of copies per stage (S::kWOps and the row copies it does not leave out),
     // unconditionally (past the end they repeat the last stage, into a slot that is free), so "at most RING - 2
     // stages' worth of my copies outstanding" means that the stage about to be read has landed.
 #pragma unroll
     for (int q = 0; q < RING - 1; ++q) issue(q < NS ? q : NS - 1);
     for (int q = 0; q < NS; ++q) {
         // at most (RING - 2) stages' worth of this wave's copies outstanding
-        if (x_copies == 2) wait_vmcnt<(RING - 2) * S::kOps>();
-        else if (x_copies == 1) wait_vmcnt<(RING - 2) * (S::kOps - 1)>();
-        else wait_vmcnt<(RING - 2) * (S::kOps - 2)>();
+        static_assert(RING == 3, "one stage's worth of copies may be outstanding");
+        wait_stage_ops<S::kWOps, 2 * MR>(x_copies);
         __syncthreads();  // stage q is whole (the first time round: so is the pair table); nobody reads stage q - 1 any more
         const unsigned char *const base = ring + (q % RING) * S::kStage;
         // the stage's packed weights and scales are asked of the LDS before the next copies are set up (some
@@ -251,12 +269,14 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
         // table lookups per matrix) asked of the LDS one step ahead: asked for right in front of their MFMA, every
         // step would wait out the LDS latency and the stage would be a chain of eight of them.
         struct StepOps {
-            uint4_t xa;
+            uint4_t xa[MR];
             uint4_t wf[CB];
         };
         auto fetch = [&](int step, StepOps &o) {
             const int s2 = step >> 2, ks = step & 3;
-            o.xa = *(const uint4_t *)(base + x_rd[s2][ks]);
+#pragma unroll
+            for (int m = 0; m < MR; ++m)
+                if (m == 0 || m < m_blocks) o.xa[m] = *(const uint4_t *)(base + m * 8192 + x_rd[s2][ks]);
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 const uint32_t w = wl2[s2][cb][ks];
@@ -270,34 +290,40 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
         StepOps ops[AHEAD + 1];
 #pragma unroll
         for (int a = 0; a < AHEAD; ++a) fetch(a, ops[a]);
-        floatx16 blk[CB];
+        floatx16 blk[MR][CB];
 #pragma unroll
         for (int step = 0; step < 8; ++step) {
             if (step + AHEAD < 8) fetch(step + AHEAD, ops[(step + AHEAD) % (AHEAD + 1)]);
             const StepOps &o = ops[step % (AHEAD + 1)];
             const int s2 = step >> 2, ks = step & 3;
+            // a block past the tile's last row (wave-uniform) is neither read nor multiplied
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) {
-                union {
-                    uint4_t u;
-                    bf16x8 v;
-                } xa, wf;
-                xa.u = o.xa;
-                wf.u = o.wf[cb];
-                if (ks == 0) {
-                    floatx16 zero;
+            for (int m = 0; m < MR; ++m) {
+                if (m > 0 && m >= m_blocks) continue;
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) zero[r] = 0.f;
-                    blk[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa.v, wf.v, zero, 0, 0, 0);
-                } else {
-                    blk[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa.v, wf.v, blk[cb], 0, 0, 0);
+                for (int cb = 0; cb < CB; ++cb) {
+                    union {
+                        uint4_t u;
+                        bf16x8 v;
+                    } xa, wf;
+                    xa.u = o.xa[m];
+                    wf.u = o.wf[cb];
+                    if (ks == 0) {
+                        floatx16 zero;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+                        blk[m][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa.v, wf.v, zero, 0, 0, 0);
+                    } else {
+                        blk[m][cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xa.v, wf.v, blk[m][cb], 0, 0, 0);
+                    }
                 }
-            }
-            if (ks == 3) {
+                if (ks == 3) {
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb)
+                    for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) tot[cb][r] = __builtin_fmaf(am2[s2][cb], blk[cb][r], tot[cb][r]);
+                        for (int r = 0; r < 16; ++r)
+                            tot[m][cb][r] = __builtin_fmaf(am2[s2][cb], blk[m][cb][r], tot[m][cb][r]);
+                }
             }
         }
     }
@@ -307,32 +333,34 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     const int col = j0 + n;
     if (col >= N) return;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int row = 8 * (r >> 2) + 4 * h + (r & 3);
-        if (row >= rows) continue;
-        const int64_t o = (int64_t)(i0 + row) * N + col;
-        if constexpr (GLU) {
-            const bf16_t pe = (bf16_t)tot[0][r], pg = (bf16_t)tot[1][r];
-            ((bf16_t *)y)[o] = silu_fwd_one<bf16_t>(pe, pg);
-            if (e_out) ((bf16_t *)e_out)[o] = pe;
-            if (g_out) ((bf16_t *)g_out)[o] = pg;
-        } else {
-            y[o] = from_f32<TO>(tot[0][r]);
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = 32 * m + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (row >= rows) continue;
+            const int64_t o = (int64_t)(i0 + row) * N + col;
+            if constexpr (GLU) {
+                const bf16_t pe = (bf16_t)tot[m][0][r], pg = (bf16_t)tot[m][1][r];
+                ((bf16_t *)y)[o] = silu_fwd_one<bf16_t>(pe, pg);
+                if (e_out) ((bf16_t *)e_out)[o] = pe;
+                if (g_out) ((bf16_t *)g_out)[o] = pg;
+            } else {
+                y[o] = from_f32<TO>(tot[m][0][r]);
+            }
         }
-    }
 }
 
-template <bool GLU, bool TILED, typename TO>
+template <bool GLU, bool TILED, int MR, typename TO>
 int launch_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
                   const void *m_sizes, int ms_i64, TO *y, TO *e_out, TO *g_out, int64_t R, int N, int K, int E,
                   hipStream_t stream) {
-    using S = StreamShape<GLU>;
+    using S = StreamShape<GLU, MR>;
     constexpr int kLds = S::kLds;
     const int tiles_n = ceil_div(N, 128);
-    const int64_t row_tiles = R / 32 + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / 32)
+    const int64_t row_tiles = R / (32 * MR) + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / (32 MR))
     const int64_t grid = (row_tiles + 7) / 8 * 8 * tiles_n;  // row tiles in eights: one per XCD
     if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
-    auto *kernel = nf4_stream_kernel<GLU, TILED, TO>;
+    auto *kernel = nf4_stream_kernel<GLU, TILED, MR, TO>;
     static PerDeviceOnce attr;
     // The kernel's table lookups take the dynamic LDS to start at address 0: any static LDS in this kernel
     // (a later __shared__ variable, an inlined helper that brings one) would move it, so the launcher asks the
@@ -397,13 +425,19 @@ int gemm_nf4_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const 
     // the tile-ordered scales are used where the caller brought them for every matrix of the product
     const bool tiled = w0.absmax_tiled != nullptr && (!glu || w1.absmax_tiled != nullptr) &&
                        aligned(w0.absmax_tiled, 4) && (!glu || aligned(w1.absmax_tiled, 4));
-#define MFL_STREAM(GLU, TO, Y, EO, GO)                                                                          \
-    (tiled ? launch_stream<GLU, true, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream) \
-           : launch_stream<GLU, false, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream))
-    if (glu) return MFL_STREAM(true, bf16_t, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out);
-    if (out_dtype == MFL_BF16) return MFL_STREAM(false, bf16_t, (bf16_t *)y, nullptr, nullptr);
-    return MFL_STREAM(false, float, (float *)y, nullptr, nullptr);
+    // rows of a workgroup's tile: 64 where experts hold more than kNf4StreamTwoBlockRows rows on average (the
+    // weights of an expert are streamed and decoded once per row tile; two workgroups per CU instead of three).
+    // The gated form keeps 32 (with 64 its three stages leave room for one workgroup per CU).
+    const int mr = !glu && R > (int64_t)kNf4StreamTwoBlockRows * E ? 2 : 1;
+#define MFL_STREAM_MR(GLU, MR, TO, Y, EO, GO)                                                                              \
+    (tiled ? launch_stream<GLU, true, MR, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream) \
+           : launch_stream<GLU, false, MR, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream))
+#define MFL_STREAM(TO, Y) (mr == 2 ? MFL_STREAM_MR(false, 2, TO, Y, nullptr, nullptr) : MFL_STREAM_MR(false, 1, TO, Y, nullptr, nullptr))
+    if (glu) return MFL_STREAM_MR(true, 1, bf16_t, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out);
+    if (out_dtype == MFL_BF16) return MFL_STREAM(bf16_t, (bf16_t *)y);
+    return MFL_STREAM(float, (float *)y);
 #undef MFL_STREAM
+#undef MFL_STREAM_MR
 }
 
 }  // namespace mfl

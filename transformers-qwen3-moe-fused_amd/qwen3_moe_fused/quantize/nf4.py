@@ -170,8 +170,9 @@ def resolve_absmax(quant_state) -> torch.Tensor:
     return absmax.contiguous()
 
 
-# rows per expert up to which the library's NF4 products run on the kernels that read tile-ordered scales
-_TILED_ROWS_PER_EXPERT = 72
+# rows per expert up to which the library's NF4 products run on the kernels that read tile-ordered scales (the plain
+# forward product up to 100, the gated one up to 72: a copy brought along above that is not read)
+_TILED_ROWS_PER_EXPERT = 100
 
 
 def tiled_absmax(quant_state, absmax: torch.Tensor, rows: int):
