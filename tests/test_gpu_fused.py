@@ -124,6 +124,8 @@ def test_glu_forward(T, E, k, N, K, gathered):
                                                  (1024, 4, 2, 264, 192, 32, 8), (16, 128, 8, 768, 2048, 64, 64),
                                                  (256, 128, 8, 768, 2048, 64, 64),
                                                  (24, 6, 2, 136, 384, 64, 128),    # streaming kernel, ragged edges
+                                                 (160, 6, 2, 136, 384, 64, 128),   # the same with 64-row tiles
+                                                 (640, 128, 8, 768, 2048, 64, 64),
                                                  (9, 12, 2, 96, 1280, 128, 256),   # matrix-vector kernel
                                                  (3, 5, 3, 32, 2048, 2048, 8),
                                                  (4, 9, 2, 64, 768, 64, 256)])    # 32 lanes to a column

@@ -21,13 +21,16 @@ constexpr int kNf4DecodeRowsPerExpert = MFL_X_NF4_ROWS;
 #else
 constexpr int kNf4DecodeRowsPerExpert = 72;
 #endif
-// The plain packed-weight forward stays on the streaming kernel up to this many rows per expert: from
-// kNf4StreamTwoBlockRows rows per expert on its workgroups take 64 rows of an expert (the weights are streamed and
-// decoded once per row tile).  Same shape and routing: 32- / 64-row tiles / pipelined kernel 59 / 55 / - us at
-// 40 rows per expert, 66 / 57 / - at 48, 75 / 74 / - at 64, 95-103 / 88 / 95-103 at 80, 110 / 92 / 96-98 at 96,
-// 138 / 117 / 104 at 128; 50 / 52 at 32.
-constexpr int kNf4StreamRowsPerExpert = 100;
-constexpr int kNf4StreamTwoBlockRows = 36;
+// The packed-weight forward stays on the streaming kernel up to this many rows per expert on average (plain / gated
+// product); from kNf4StreamTwoBlockRows on its workgroups take 64 rows of an expert.  Gate_proj shape, 128 experts,
+// uniform routing, streaming (64-row tiles, two stages) against what ran before (32-row tiles to 72 rows per expert,
+// the pipelined kernel beyond): plain 35 / 42 / 44 / 56 / 68 / 77 / 79 / 88 / 100 us against 42 / 51 / 58 / 63 / 73 /
+// 103 / 96 / 99 / 103 at 24 / 32 / 40 / 48 / 64 / 80 / 96 / 112 / 128 rows per expert, 115 against 110 at 160;
+// gated 68 / 80 / 84 / 118 / 144 / 196 / 257 / 323 against 76 / 94 / 109 / 142 / 227 / 252 / 268 / 334 at
+// 24 / 32 / 40 / 64 / 96 / 128 / 192 / 256, 394 / 465 / 598 against 455 / 476 / 527 at 320 / 384 / 512.
+constexpr int kNf4StreamRowsPerExpert = 128;
+constexpr int kNf4StreamGatedRowsPerExpert = 256;
+constexpr int kNf4StreamTwoBlockRows = 20;
 
 // Any shape / any float type; plain FMA.
 int gemm_generic(int mode, const void *a, const void *b, const void *m_sizes, int ms_i64, void *c, int64_t R, int N,

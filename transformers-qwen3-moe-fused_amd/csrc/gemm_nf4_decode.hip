@@ -287,11 +287,11 @@ __global__ __launch_bounds__(256) void nf4_decode_kernel(const bf16_t *__restric
 int gemm_nf4_decode(const void *x, const uint8_t *wq, const float *code16, const float *absmax, int blocksize,
                     const void *m_sizes, int ms_i64, void *y, int64_t R, int N, int K, int E, int out_dtype,
                     hipStream_t stream, const GemmFusion *fusion) {
-    // decode-sized batches only: with more rows per expert every row tile decodes the weights again (the plain
-    // product has 64-row tiles in the streaming kernel and stays ahead of the pipelined kernel for longer)
+    // up to where the streaming kernel (64-row tiles) is ahead of the pipelined one: with more rows per expert every
+    // row tile streams and decodes the weights again
     const bool gated = fusion != nullptr && fusion->w2 != nullptr;
     if (R <= 0) return MFL_OK;
-    if (R > (int64_t)(gated ? kNf4DecodeRowsPerExpert : kNf4StreamRowsPerExpert) * E) return MFL_ERR_UNSUPPORTED;
+    if (R > (int64_t)(gated ? kNf4StreamGatedRowsPerExpert : kNf4StreamRowsPerExpert) * E) return MFL_ERR_UNSUPPORTED;
     int shift = 0;
     while ((1 << shift) < blocksize) ++shift;
     if (K % 64 != 0 || N % 8 != 0 || N < 8 || blocksize < 8) return MFL_ERR_UNSUPPORTED;

@@ -5,17 +5,17 @@
 // or scales issued after a copy would, when waited for, hold the wave until the copy has landed too, and the
 // copies would never be further ahead than those loads.
 //
-// A workgroup (4 waves) owns 32 MR rows of one expert (MR = 1, or 2 where experts hold some forty rows and more:
-// the weights are streamed and decoded once per row tile) and 128 output columns, a wave 32 of the columns (of
+// A workgroup (4 waves) owns 32 MR rows of one expert (MR = 1 at decode sizes, 2 from some twenty rows per expert
+// on: the weights are streamed and decoded once per row tile) and 128 output columns, a wave 32 of the columns (of
 // both matrices in the gated linear unit) for all of the rows.
 //   stage = rows     32 MR x 128 bf16 (8 KiB a block of 32, shared by the four waves; chunk c of row r at c ^ (r & 15))
 //         + weights  per wave and matrix 32 columns x 64 packed bytes (2 KiB; chunk c of row r at c ^ ((r >> 2) & 3))
 //         + scales   per wave and matrix 32 columns x 2 floats (one per 64 reduction elements)
 //   One barrier per stage: it publishes the rows that the other waves copied and frees the slot of the
-//   stage before for the next copies.  Three stages are 52 KiB: three workgroups share a CU (two of the gated
-//   form), and what counts at decode sizes is that every workgroup of the launch is resident at once: a
-//   workgroup's loop is a chain of latencies (about 1.1 us per stage whatever is taken out of it), so a second
-//   round of workgroups doubles the time of the launch.
+//   stage before for the next copies.  Three stages of 32-row tiles are 52 KiB, two stages of 64-row tiles 51 KiB:
+//   three workgroups share a CU (two of the gated form), and what counts is how many workgroups of the launch
+//   are resident at once: a workgroup's loop is a chain of latencies (about 1.1 us per stage whatever is taken
+//   out of it), so a second round of workgroups doubles the time of the launch.
 //
 // Decoding costs about one vector instruction per weight instead of three and a half:
 //   * a byte of packed weights is two weights, and two bf16 are one dword of an MFMA operand: a 256-entry
@@ -73,16 +73,17 @@ __device__ __forceinline__ uint32_t byte_times_4(uint32_t w) {
     return r;
 }
 
-template <bool GLU, int MR>
+template <bool GLU, int MR, int RING_>
 struct StreamShape {
     static constexpr int CB = GLU ? 2 : 1;     // weight matrices per wave
-    static constexpr int RING = 3;             // stages in LDS; two of them in flight
+    static constexpr int RING = RING_;         // stages in LDS; all but one of them in flight
     static constexpr int kX = MR * 32 * 256;   // rows of a stage: MR blocks of 32
     static constexpr int kW = 32 * 64;         // packed weights of a stage, per wave and matrix
     static constexpr int kA = 32 * 2 * 4;      // scales of a stage, per wave and matrix
     static constexpr int kStage = kX + 4 * CB * (kW + kA);
     static constexpr int kTable = CB * 256 * 4;
-    static constexpr int kLds = RING * kStage + kTable;  // MR = 1: 53248, three workgroups per CU; gated: 81920, two
+    // RING 3, MR 1: 53248, three workgroups per CU; gated: 81920, two.  RING 2, MR 2: 52224, three; gated: 72704, two.
+    static constexpr int kLds = RING * kStage + kTable;
     static constexpr int kWOps = 2 * CB + CB;  // copies of weights and scales per wave and stage (the rows: up to 2 MR more)
 };
 
@@ -97,7 +98,7 @@ __device__ __forceinline__ void wait_stage_ops(int xc) {
     }
 }
 
-template <bool GLU, bool TILED, int MR, typename TO>
+template <bool GLU, bool TILED, int MR, int RING_, typename TO>
 __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restrict__ x,
                                                          const int32_t *__restrict__ row_idx, int idx_div,
                                                          Nf4Matrix w0, Nf4Matrix w1,
@@ -105,7 +106,7 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
                                                          TO *__restrict__ y, TO *__restrict__ e_out,
                                                          TO *__restrict__ g_out, int64_t R, int N, int K, int E,
                                                          int tiles_n) {
-    using S = StreamShape<GLU, MR>;
+    using S = StreamShape<GLU, MR, RING_>;
     constexpr int CB = S::CB, RING = S::RING, TR = 32 * MR;  // TR: rows of a workgroup's tile
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
     // the pair table first, at LDS address 0 (the kernel has no static LDS, which the launcher checks): a lookup's address is then the shifted
@@ -249,8 +250,8 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
     for (int q = 0; q < RING - 1; ++q) issue(q < NS ? q : NS - 1);
     for (int q = 0; q < NS; ++q) {
         // at most (RING - 2) stages' worth of this wave's copies outstanding
-        static_assert(RING == 3, "one stage's worth of copies may be outstanding");
-        wait_stage_ops<S::kWOps, 2 * MR>(x_copies);
+        if constexpr (RING == 3) wait_stage_ops<S::kWOps, 2 * MR>(x_copies);
+        else wait_vmcnt<0>();
         __syncthreads();  // stage q is whole (the first time round: so is the pair table); nobody reads stage q - 1 any more
         const unsigned char *const base = ring + (q % RING) * S::kStage;
         // the stage's packed weights and scales are asked of the LDS before the next copies are set up (some
@@ -350,17 +351,17 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
         }
 }
 
-template <bool GLU, bool TILED, int MR, typename TO>
+template <bool GLU, bool TILED, int MR, int RING_, typename TO>
 int launch_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const Nf4Matrix &w0, const Nf4Matrix &w1,
                   const void *m_sizes, int ms_i64, TO *y, TO *e_out, TO *g_out, int64_t R, int N, int K, int E,
                   hipStream_t stream) {
-    using S = StreamShape<GLU, MR>;
+    using S = StreamShape<GLU, MR, RING_>;
     constexpr int kLds = S::kLds;
     const int tiles_n = ceil_div(N, 128);
     const int64_t row_tiles = R / (32 * MR) + (R < E ? R : E);  // upper bound on sum over experts of ceil(m / (32 MR))
     const int64_t grid = (row_tiles + 7) / 8 * 8 * tiles_n;  // row tiles in eights: one per XCD
     if (grid > 0x7fffffff) return MFL_ERR_UNSUPPORTED;
-    auto *kernel = nf4_stream_kernel<GLU, TILED, MR, TO>;
+    auto *kernel = nf4_stream_kernel<GLU, TILED, MR, RING_, TO>;
     static PerDeviceOnce attr;
     // The kernel's table lookups take the dynamic LDS to start at address 0: any static LDS in this kernel
     // (a later __shared__ variable, an inlined helper that brings one) would move it, so the launcher asks the
@@ -425,17 +426,19 @@ int gemm_nf4_stream(const bf16_t *x, const int32_t *row_idx, int idx_div, const 
     // the tile-ordered scales are used where the caller brought them for every matrix of the product
     const bool tiled = w0.absmax_tiled != nullptr && (!glu || w1.absmax_tiled != nullptr) &&
                        aligned(w0.absmax_tiled, 4) && (!glu || aligned(w1.absmax_tiled, 4));
-    // rows of a workgroup's tile: 64 where experts hold more than kNf4StreamTwoBlockRows rows on average (the
-    // weights of an expert are streamed and decoded once per row tile; two workgroups per CU instead of three).
-    // The gated form keeps 32 (with 64 its three stages leave room for one workgroup per CU).
-    const int mr = !glu && R > (int64_t)kNf4StreamTwoBlockRows * E ? 2 : 1;
-#define MFL_STREAM_MR(GLU, MR, TO, Y, EO, GO)                                                                              \
-    (tiled ? launch_stream<GLU, true, MR, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream) \
-           : launch_stream<GLU, false, MR, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream))
-#define MFL_STREAM(TO, Y) (mr == 2 ? MFL_STREAM_MR(false, 2, TO, Y, nullptr, nullptr) : MFL_STREAM_MR(false, 1, TO, Y, nullptr, nullptr))
-    if (glu) return MFL_STREAM_MR(true, 1, bf16_t, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out);
-    if (out_dtype == MFL_BF16) return MFL_STREAM(bf16_t, (bf16_t *)y);
-    return MFL_STREAM(float, (float *)y);
+    // Tile height and ring depth.  Up to kNf4StreamTwoBlockRows rows per expert on average: 32-row tiles, three
+    // stages.  Above: 64-row tiles (an expert's weights are streamed and decoded once per row tile) with two stages,
+    // which leaves the plain product its three workgroups per CU and the gated one its two: residency counts for
+    // more than a second stage in flight (plain product, 40 rows per expert: 43 us against 55 with three stages
+    // and two workgroups per CU, 59 with 32-row tiles).  The bits are the same whatever the tile height.
+    const bool two = R > (int64_t)kNf4StreamTwoBlockRows * E;
+#define MFL_STREAM_MR(GLU, MR, RG, TO, Y, EO, GO)                                                                              \
+    (tiled ? launch_stream<GLU, true, MR, RG, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream) \
+           : launch_stream<GLU, false, MR, RG, TO>(x, row_idx, idx_div, w0, w1, m_sizes, ms_i64, Y, EO, GO, R, N, K, E, stream))
+#define MFL_STREAM(GLU, TO, Y, EO, GO) (two ? MFL_STREAM_MR(GLU, 2, 2, TO, Y, EO, GO) : MFL_STREAM_MR(GLU, 1, 3, TO, Y, EO, GO))
+    if (glu) return MFL_STREAM(true, bf16_t, (bf16_t *)y, (bf16_t *)e_out, (bf16_t *)g_out);
+    if (out_dtype == MFL_BF16) return MFL_STREAM(false, bf16_t, (bf16_t *)y, nullptr, nullptr);
+    return MFL_STREAM(false, float, (float *)y, nullptr, nullptr);
 #undef MFL_STREAM
 #undef MFL_STREAM_MR
 }
