@@ -82,7 +82,7 @@ struct StreamShape {
     static constexpr int kA = 32 * 2 * 4;      // scales of a stage, per wave and matrix
     static constexpr int kStage = kX + 4 * CB * (kW + kA);
     static constexpr int kTable = CB * 256 * 4;
-    // RING 3, MR 1: 53248, three workgroups per CU; gated: 81920, two.  RING 2, MR 2: 52224, three; gated: 72704, two.
+    // RING 3, MR 1: 53248, three workgroups per CU; gated: 81920, two.  RING 2, MR 2: 52224, three; gated: 71680, two.
     static constexpr int kLds = RING * kStage + kTable;
     static constexpr int kWOps = 2 * CB + CB;  // copies of weights and scales per wave and stage (the rows: up to 2 MR more)
 };
