@@ -92,6 +92,7 @@ def _reference_sweep(dev, stream, ws, qsets):
     from qwen3_moe_fused.grouped_gemm.forward import grouped_gemm_forward
     from qwen3_moe_fused.grouped_gemm.forward_4bit import grouped_gemm_forward_4bit
     from qwen3_moe_fused.grouped_gemm.forward_transposed import grouped_gemm_forward_transposed
+    from qwen3_moe_fused.grouped_gemm.fused import grouped_glu_forward_4bit
 
     NB = len(ws)
     g = torch.Generator().manual_seed(1)
@@ -116,12 +117,17 @@ def _reference_sweep(dev, stream, ws, qsets):
             "dw": (lambda i: grouped_gemm_backward_dw(xr, dyr, ms, torch.bfloat16), io + wbytes),
             "fwd_4bit": (lambda i: grouped_gemm_forward_4bit(xr, *qsets[i % NB], ms),
                          io + E * INTER * HIDDEN * (0.5 + 4.0 / 64)),
+            # not one of the reference's benchmarks: gate and up projection with packed weights and SiLU-mul in one
+            # launch, as the sparse block's front half runs them (twice the flops of the other legs)
+            "glu_4bit": (lambda i: grouped_glu_forward_4bit(xr, *qsets[i % NB], *qsets[(i + 1) % NB], ms),
+                         io + 2 * E * INTER * HIDDEN * (0.5 + 4.0 / 64)),
         }
         point = {"rows": rows}
         for name, (fn, nbytes) in legs.items():
             med, q20, q80 = _per_launch_us(fn, iters, warm, stream)
+            fl = 2 * flop if name == "glu_4bit" else flop
             point[name] = {"us": round(med, 1), "us_q20": round(q20, 1), "us_q80": round(q80, 1),
-                           "tflops": round(flop / med / 1e6, 1), "gbs": round(nbytes / med / 1e3, 1),
+                           "tflops": round(fl / med / 1e6, 1), "gbs": round(nbytes / med / 1e3, 1),
                            "hbm_frac": round(nbytes / med / 1e3 / PEAK_HBM_GBS, 4)}
         points.append(point)
     # largest step in achieved GB/s between neighbouring points, per product (a cliff marks a bad switch of
@@ -215,6 +221,22 @@ def _kernel_tour(n, dev):
                          2 * active * nf4_b / E + 2.0 * tokens * TOPK * (HIDDEN + INTER),
                          4.0 * tokens * TOPK * INTER * HIDDEN,
                          lambda i, x5=x5, ms5=ms5: grouped_glu_forward_4bit(x5, *qsets[i % 3], *qsets[(i + 1) % 3], ms5)))
+    # the middle of the reference's row sweep (1024 tokens, 64 rows per expert): packed weights on the streaming
+    # kernel's 64-row tiles, and the input gradient whose output is 2048 wide (192 x 256 tiles)
+    lgt = torch.randn((1024, E), device=dev, generator=g)
+    _, _, s6 = softmax_topk_raw(lgt, TOPK, True, bf)
+    ms6, _, _ = get_expert_counts_and_idx(s6.view(-1), E)
+    x6, dy6 = rnd(1024 * TOPK, HIDDEN), rnd(1024 * TOPK, INTER)
+    io6 = 2.0 * 1024 * TOPK * (HIDDEN + INTER)
+    legs += [
+        ("gemm_fwd_nf4 gate_proj 1024 tokens (64-row tiles)", nf4_b + io6, 2.0 * 1024 * TOPK * INTER * HIDDEN,
+         lambda i: grouped_gemm_forward_4bit(x6, *qsets[i % 3], ms6)),
+        ("glu_fwd_nf4 (gate + up + SiLU-mul) 1024 tokens (64-row tiles)", 2 * nf4_b + io6,
+         4.0 * 1024 * TOPK * INTER * HIDDEN,
+         lambda i: grouped_glu_forward_4bit(x6, *qsets[i % 3], *qsets[(i + 1) % 3], ms6)),
+        ("gemm_dx gate_proj 1024 tokens (output 2048 wide, 192 x 256 tiles)", 2.0 * E * INTER * HIDDEN + io6,
+         2.0 * 1024 * TOPK * INTER * HIDDEN, lambda i: grouped_gemm_forward_transposed(dy6, w_gate, ms6)),
+    ]
     # configuration 4: rank-16 adapter products at 8192 tokens under Zipf(1.2)-skewed routing (65536 rows)
     from qwen3_moe_fused.grouped_gemm.fused import grouped_gemm_forward_lora
     T4, R4, RANK = 8192, 8192 * TOPK, 16
