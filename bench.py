@@ -583,11 +583,11 @@ def main() -> int:
         blk = blk.to(dev)
         block = {}
         with torch.no_grad():
-            for tokens in (16, 256, 16384):
+            for tokens in (16, 256, 1024, 16384):
                 h5 = torch.randn((1, tokens, HIDDEN), device=dev, dtype=torch.bfloat16)
                 # short calls need a long warm-up to leave the power-management transient of a launch burst
-                n_it, n_wm = (20, 30) if tokens > 1000 else (40, 200)
-                timer = _event_us if tokens > 1000 else _event_us_median
+                n_it, n_wm = (20, 30) if tokens > 2000 else (40, 200)
+                timer = _event_us if tokens > 2000 else _event_us_median
                 blk.fuse_front = False                        # gather, gate_proj, up_proj, SiLU-mul one by one
                 us_sep = timer(lambda i: blk(h5), n_it, n_wm, stream)
                 blk.fuse_front = True                         # the default: the four as one kernel
