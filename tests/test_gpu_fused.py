@@ -253,7 +253,8 @@ from qwen3_moe_fused.grouped_gemm.fused import grouped_gemm_forward_transposed_d
 
 # dx (R, N) = dy1 (R, K) @ w1[e] + dy2 (R, K) @ w2[e], w (E, K, N)
 @pytest.mark.parametrize("R,N,K,E", [(2048, 2048, 768, 8), (700, 200, 64, 5), (300, 72, 128, 3), (33, 8, 192, 40),
-                                     (5000, 392, 64, 2), (64, 24, 72, 4)])   # the last: K % 64 != 0, two plain products
+                                     (5000, 392, 64, 2), (1000, 1024, 128, 8),   # 192 x 256 tiles
+                                     (64, 24, 72, 4)])   # the last: K % 64 != 0, two plain products
 def test_two_term_input_gradient(R, N, K, E):
     g = gen(R + N)
     dy1, dy2 = randn((R, K), g, 1.0, torch.bfloat16), randn((R, K), g, 1.0, torch.bfloat16)

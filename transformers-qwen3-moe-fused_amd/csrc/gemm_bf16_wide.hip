@@ -961,7 +961,7 @@ int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, 
     // reduction steps per CU than with 192-column slices (N = 2048, K = 768, 128 experts: 8 slices an expert
     // instead of 11, 4 tiles a CU instead of 5.5; 88 / 91 / 97 / 106 / 110 us against 95 / 100 / 107 / 118 / 124 at
     // 48 / 64 / 96 / 128 / 160 rows per expert, forward and input gradient alike; 154 against 137 at 192).
-    const bool wide_out = N % 256 == 0 && N >= 1024 && R <= (int64_t)kWideOutRowsPerExpert * E && a2 == nullptr && at == nullptr;
+    const bool wide_out = N % 256 == 0 && N >= 1024 && R <= (int64_t)kWideOutRowsPerExpert * E && at == nullptr;
 #ifdef MFL_TUNING_BUILD
     const int v = g_wide_variant >= 0 ? g_wide_variant : (R >= (int64_t)512 * E ? 1 : wide_out ? 3 : 0);
 #else
