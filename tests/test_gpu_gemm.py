@@ -315,11 +315,13 @@ WIDE_ROW_CASES = [
     (768, 2048, [48, 60, 0, 130, 50, 49]),
     (520, 128, [1000, 0, 700]),
     (768, 256, [513, 2047, 256, 1300]),
-    # 192 x 256 tiles (outputs a multiple of 256 columns and at least 1024 wide, at most 168 rows per expert on
+    # 192 x 256 tiles (outputs a multiple of 256 columns and at least 1024 wide, at most 152 rows per expert on
     # average): experts of 0, 1, 191, 192 and 193 rows, one of two tiles, a reduction of one step
     (2048, 768, [100 + 13 * (e % 7) for e in range(16)]),
     (1024, 128, [0, 193, 60, 192, 1, 150, 191, 120]),
     (1280, 64, [64] * 3 + [400, 48, 0, 97, 129]),
+    # the same widths between 152 and 232 rows per expert: 256 x 256 tiles (experts of 255, 256, 257 and 520 rows)
+    (1024, 192, [255, 256, 257, 0, 190, 520, 100, 180]),
 ]
 
 

@@ -29,7 +29,7 @@ namespace mfl {
 
 namespace {
 
-constexpr int kWideOutRowsPerExpert = 168;
+constexpr int kWideOutRowsPerExpert = 152, kWideMidRowsPerExpert = 232;
 
 // Tuning builds can take parts of the kernel out (timing experiments only; the results are then wrong).
 #ifdef MFL_TUNING_BUILD
@@ -956,16 +956,21 @@ int gemm_bf16_wide(int mode, const void *a, const void *b, const void *m_sizes, 
     }
     if (K % 64 != 0 || K < 64 || R <= 0) return R <= 0 ? MFL_OK : MFL_ERR_UNSUPPORTED;
     // 320 x 192 tiles (an expert of up to 320 rows is one tile per column slice) up to about 512 rows per expert,
-    // 256 x 256 beyond (fewer bytes per flop).  Outputs that are wide and a multiple of 256 columns, up to 168 rows
+    // 256 x 256 beyond (fewer bytes per flop).  Outputs that are wide and a multiple of 256 columns, up to 152 rows
     // per expert on average (few experts then hold more than 192 rows): 192 x 256 tiles, a quarter fewer tiles and
     // reduction steps per CU than with 192-column slices (N = 2048, K = 768, 128 experts: 8 slices an expert
     // instead of 11, 4 tiles a CU instead of 5.5; 88 / 91 / 97 / 106 / 110 us against 95 / 100 / 107 / 118 / 124 at
     // 48 / 64 / 96 / 128 / 160 rows per expert, forward and input gradient alike; 154 against 137 at 192).
-    const bool wide_out = N % 256 == 0 && N >= 1024 && R <= (int64_t)kWideOutRowsPerExpert * E && at == nullptr;
+    // From there to 232 rows per expert such outputs take the 256 x 256 tiles (few experts hold more than 256 rows;
+    // 8 slices an expert again): 111 / 114 / 118 / 139 us against 120 / 127 / 134 / 147 at 168 / 184 / 192 / 224 rows
+    // per expert (and against 120 at 168 on the 192 x 256 tiles), 164 against 158 at 256.
+    const bool wide_n = N % 256 == 0 && N >= 1024;
+    const bool wide_out = wide_n && R <= (int64_t)kWideOutRowsPerExpert * E && at == nullptr;
+    const bool wide_mid = wide_n && R > (int64_t)kWideOutRowsPerExpert * E && R <= (int64_t)kWideMidRowsPerExpert * E;
 #ifdef MFL_TUNING_BUILD
-    const int v = g_wide_variant >= 0 ? g_wide_variant : (R >= (int64_t)512 * E ? 1 : wide_out ? 3 : 0);
+    const int v = g_wide_variant >= 0 ? g_wide_variant : (R >= (int64_t)512 * E || wide_mid ? 1 : wide_out ? 3 : 0);
 #else
-    const int v = R >= (int64_t)512 * E ? 1 : wide_out ? 3 : 0;
+    const int v = R >= (int64_t)512 * E || wide_mid ? 1 : wide_out ? 3 : 0;
 #endif
     if (N % 8 != 0 || N < 8) return MFL_ERR_UNSUPPORTED;
     if (at != nullptr) {
