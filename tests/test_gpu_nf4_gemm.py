@@ -31,6 +31,8 @@ def _quantised(E, N, K, blocksize, seed):
                                                # >= 32 rows per expert: the pipelined kernel, several row tiles
                                                # per expert and many reduction steps
                                                (8192, 768, 2048, 16, 64), (4096, 200, 512, 4, 128),
+                                               # an output of 1024 columns at 200 rows per expert: 256 x 256 tiles
+                                               (1600, 1024, 128, 8, 64),
                                                # small quantisation blocks on the pipelined kernel
                                                (2048, 64, 128, 2, 16), (1500, 72, 192, 3, 8),
                                                # decode-sized batches (register-decode kernel), small blocks, a
@@ -303,7 +305,8 @@ from qwen3_moe_fused.grouped_gemm.forward_transposed import grouped_gemm_forward
 # weight (E, K = out_features, N = in_features); dx (R, N) = dy (R, K) @ w[e]
 @pytest.mark.parametrize("R,N,K,E,blocksize", [(1024, 2048, 768, 128, 64), (4096, 768, 2048, 16, 64),
                                                (300, 64, 64, 5, 8), (513, 160, 128, 3, 32), (2000, 96, 192, 2, 16),
-                                               (40, 32, 64, 7, 128), (5000, 416, 128, 3, 256)])
+                                               (40, 32, 64, 7, 128), (5000, 416, 128, 3, 256),
+                                               (1600, 1024, 128, 8, 64)])   # 256 x 256 tiles at 200 rows per expert
 def test_fused_nf4_input_gradient(R, N, K, E, blocksize):
     packed, state, w_deq = _quantised(E, K, N, blocksize, R + N)
     g = gen(R + 1)

@@ -1091,10 +1091,14 @@ int dispatch_pipe(int mode, const void *a, const void *b, const void *m_sizes, i
     } else if (cfg == 0 || nf4 != nullptr) {
         if (mode == MODE_DW)
             cfg = (N <= 64 || K <= 64) ? 11 : 8;
-        else
+        else {
+            // packed weights with an output of 1024 columns and more that is a multiple of 256 wide, up to 232 rows per
+            // expert: 256 x 256 tiles as well (8 column slices an expert instead of 11 of 192 columns)
+            const bool nf4_wide = nf4 != nullptr && N % 256 == 0 && N >= 1024 && R <= (int64_t)232 * E;
             cfg = (N <= 64 && nf4 == nullptr) ? 10
                   : (R <= (int64_t)kFlatTileRowsPerExpert * E && nf4 == nullptr) ? 15
-                  : R >= (int64_t)512 * E ? 8 : 3;
+                  : (R >= (int64_t)512 * E || nf4_wide) ? 8 : 3;
+        }
     }
     switch (cfg) {
         case 1:
