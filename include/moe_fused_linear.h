@@ -236,7 +236,7 @@ MFL_API int mfl_glu_fwd_nf4(const void *x, int64_t src_rows, const int32_t *row_
  * are mfl_gemm_fwd_nf4 / mfl_gemm_fwd_nf4_gather (row_idx NULL: x_src is x, src_rows and idx_div ignored)
  * and mfl_glu_fwd_nf4 with one more argument per matrix; absmax_tiled may be NULL (then they are those
  * entry points), and results are bit-identical with and without it.  The kernels that read the copy take the
- * plain product up to 128 rows per expert on average and the gated one up to 256; beyond that it is ignored.
+ * plain product up to 128 rows per expert on average and the gated one up to 384; beyond that it is ignored.
  * No counterpart in the reference, whose
  * 4-bit product (qwen3_moe_fused/grouped_gemm/forward_4bit.py:99-106) reads absmax in place. */
 MFL_API int64_t mfl_nf4_tiled_absmax_floats(int blocksize, int N, int K, int E);

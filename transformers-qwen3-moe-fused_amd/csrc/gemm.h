@@ -29,7 +29,7 @@ constexpr int kNf4DecodeRowsPerExpert = 72;
 // gated 68 / 80 / 84 / 118 / 144 / 196 / 257 / 323 against 76 / 94 / 109 / 142 / 227 / 252 / 268 / 334 at
 // 24 / 32 / 40 / 64 / 96 / 128 / 192 / 256, 394 / 465 / 598 against 455 / 476 / 527 at 320 / 384 / 512.
 constexpr int kNf4StreamRowsPerExpert = 128;
-constexpr int kNf4StreamGatedRowsPerExpert = 256;
+constexpr int kNf4StreamGatedRowsPerExpert = 384;
 constexpr int kNf4StreamTwoBlockRows = 20;
 
 // Any shape / any float type; plain FMA.

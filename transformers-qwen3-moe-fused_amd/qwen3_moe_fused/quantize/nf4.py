@@ -171,8 +171,8 @@ def resolve_absmax(quant_state) -> torch.Tensor:
 
 
 # rows per expert up to which the library's NF4 products run on the kernels that read tile-ordered scales (the plain
-# forward product up to 128, the gated one up to 256: a copy brought along above that is not read)
-_TILED_ROWS_PER_EXPERT = 256
+# forward product up to 128, the gated one up to 384: a copy brought along above that is not read)
+_TILED_ROWS_PER_EXPERT = 384
 
 
 def tiled_absmax(quant_state, absmax: torch.Tensor, rows: int):
