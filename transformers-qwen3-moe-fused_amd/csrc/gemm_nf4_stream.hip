@@ -200,6 +200,9 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
         x_src[j] = x + src_row * K + c * 8;
     }
     const int NS = K / 128, tiles32 = (N + 31) / 32;
+    // a wave whose 32 columns all lie past N (N not a multiple of 128) takes the scales of the last tile of its
+    // expert: copied, multiplied, never stored, and inside the array also for the last expert
+    const int a_tile = j0 / 32 < tiles32 ? j0 / 32 : tiles32 - 1;
     // A copy of rows whose four rows all lie past the tile's last row is left out (nobody stores what the MFMAs
     // make of that part of the stage): the first x_copies of the wave's 2 MR (their rows ascend with j), the same
     // number in every stage.
@@ -220,7 +223,7 @@ __global__ __launch_bounds__(256) void nf4_stream_kernel(const bf16_t *__restric
                 copy16_to_lds(w_src[cb][j] + (int64_t)stg * 64, base + S::kX + (wave * CB + cb) * S::kW + j * 1024);
             // the wave's 64 scales of the stage: 256 consecutive bytes of the tile-ordered copy where the caller
             // brought one (two lines per copy), else two neighbours out of each column's own run (32 lines)
-            const float *a_src = TILED ? mat[cb].absmax_tiled + ((((int64_t)expert * tiles32 + j0 / 32) * NS + stg) * 64 + lane)
+            const float *a_src = TILED ? mat[cb].absmax_tiled + ((((int64_t)expert * tiles32 + a_tile) * NS + stg) * 64 + lane)
                                        : mat[cb].absmax + ((a_el[cb] + (int64_t)stg * 128) >> mat[cb].bs_shift);
             copy4_to_lds(a_src, base + S::kX + 4 * CB * S::kW + (wave * CB + cb) * S::kA);
         }
